@@ -1,0 +1,136 @@
+/*
+ * nf4hip.h -- C ABI of libnf4hip.so: NF4 blockwise weight-only quantisation kernels for
+ * AMD MI355X (gfx950).  Plain pointers and sizes only; no torch types.
+ *
+ * This is the boundary that replaces the third-party calls made by Thunder's 4-bit path:
+ *   thunder/transforms/quantization.py:63     bitsandbytes.functional.quantize_4bit(w, quant_type="nf4")
+ *   thunder/transforms/quantization.py:34-39  bitsandbytes.matmul_4bit(x, qweight.t(), bias, quant_state)
+ *       -> gemv_4bit                 (single-row x)              -> nf4hip_gemv
+ *       -> dequantize_4bit + linear  (everything else)           -> nf4hip_dequantize / nf4hip_gemm
+ *
+ * Conventions
+ *   - Every function returns 0 on success or a negative NF4HIP_E_* code; the text of the last
+ *     failure on the calling thread is available from nf4hip_last_error().
+ *   - All argument validation happens before the first HIP call, so every error code except
+ *     NF4HIP_E_HIP can be reached on a machine without a GPU.
+ *   - All data pointers are BORROWED DEVICE pointers; the caller keeps them alive until the work
+ *     queued on `stream` has finished.  Outputs are caller-allocated.
+ *   - `stream` is a hipStream_t (NULL = the default stream).  Nothing here synchronises the
+ *     device, allocates or frees memory, or blocks the host.
+ *   - dtype codes: NF4HIP_BF16 = 0, NF4HIP_F16 = 1, NF4HIP_F32 = 2.
+ *   - Weight layout: the [N, K] weight is flattened row-major into n = N*K elements; quantisation
+ *     blocks are `blocksize` consecutive elements of that flat view.  `packed` holds two 4-bit
+ *     codes per byte, the element with the even index in the HIGH nibble; `absmax` holds one
+ *     fp32 per block; `lut16` is the 16-entry fp32 code book (the op's `quant_map` argument).
+ */
+#ifndef NF4HIP_H
+#define NF4HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NF4HIP_ABI_VERSION 1
+
+#define NF4HIP_BF16 0
+#define NF4HIP_F16 1
+#define NF4HIP_F32 2
+
+#define NF4HIP_OK 0
+#define NF4HIP_E_NULL (-1)      /* a required pointer is NULL */
+#define NF4HIP_E_DTYPE (-2)     /* dtype code unknown or unsupported by this entry point */
+#define NF4HIP_E_BLOCKSIZE (-3) /* blocksize not one of 64,128,256,512,1024,2048,4096 */
+#define NF4HIP_E_SHAPE (-4)     /* a size is negative/zero where it may not be, or violates a fast-path rule */
+#define NF4HIP_E_ALIGN (-5)     /* a pointer is not 16-byte aligned */
+#define NF4HIP_E_WORKSPACE (-6) /* workspace missing or smaller than nf4hip_*_workspace_bytes() */
+#define NF4HIP_E_HIP (-7)       /* a HIP runtime call failed; text in nf4hip_last_error() */
+
+/* ABI version of the loaded library; the host side refuses a mismatch. */
+int nf4hip_abi_version(void);
+
+/* Thread-local description of the last failure on this thread ("" if none). */
+const char* nf4hip_last_error(void);
+
+/*
+ * Blockwise NF4 quantisation.  Replaces bitsandbytes.functional.quantize_4bit(A, blocksize,
+ * quant_type="nf4") as called at thunder/transforms/quantization.py:63.
+ *   w        n elements of dtype w_dtype (bf16/f16/f32)
+ *   packed   (n+1)/2 bytes out
+ *   absmax   ceil(n/blocksize) fp32 out
+ * absmax = max|w| per block; code = #{thresholds < w * (1.0f/absmax)}.  n == 0 is a no-op.
+ */
+int nf4hip_quantize(const void* w, int w_dtype, int64_t n, int blocksize, uint8_t* packed, float* absmax,
+                    void* stream);
+
+/*
+ * Blockwise NF4 dequantisation.  Replaces bitsandbytes.functional.dequantize_4bit (reached from
+ * matmul_4bit, thunder/transforms/quantization.py:39).
+ *   out[i] = round_to_nearest_even(out_dtype, lut16[code_i] * absmax[i / blocksize])
+ */
+int nf4hip_dequantize(const uint8_t* packed, const float* absmax, const float* lut16, int64_t n, int blocksize,
+                      void* out, int out_dtype, void* stream);
+
+/*
+ * Nested ("double") quantisation of absmax, bitsandbytes' compress_statistics=True.  The
+ * reference transform does not call it (thunder/transforms/quantization.py:84 "TODO: double
+ * quant support"); provided for 70B-class shapes.
+ *   compress:    r = absmax - offset; absmax2[c] = max|r| over nested block c;
+ *                absmax_q[b] = argmin_j |r_b * (1.0f/absmax2[c]) - map256[j]|   (lowest j on ties)
+ *   reconstruct: absmax[b] = map256[absmax_q[b]] * absmax2[b / nested_blocksize] + offset
+ * nested_blocksize must be a power of two in [64, 4096].
+ */
+int nf4hip_dq_compress(const float* absmax, int64_t nblocks, int nested_blocksize, const float* map256, float offset,
+                       uint8_t* absmax_q, float* absmax2, void* stream);
+int nf4hip_dq_reconstruct(const uint8_t* absmax_q, const float* absmax2, const float* map256, float offset,
+                          int64_t nblocks, int nested_blocksize, float* absmax, void* stream);
+
+/* Same as nf4hip_dequantize with absmax given in nested form. */
+int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const float* absmax2, const float* map256,
+                         float offset, int nested_blocksize, const float* lut16, int64_t n, int blocksize, void* out,
+                         int out_dtype, void* stream);
+
+/*
+ * Decode-shape fused dequant-matmul, 1 <= M <= 16.  Replaces bitsandbytes' gemv_4bit
+ * (kgemm_4bit_inference_naive), reached from thunder/transforms/quantization.py:39.
+ *   out[m][n] = bf16( sum_k x[m][k] * lut16[code(n,k)] * absmax[(n*K+k)/blocksize] + bias[n] )
+ *   x    [M, K] bf16 row-major      out  [M, N] bf16 row-major      bias [N] bf16 or NULL
+ * Fast-path rules (else NF4HIP_E_SHAPE; the host side then takes dequantize + matmul):
+ *   x_dtype == NF4HIP_BF16, K % 512 == 0, blocksize divides K.
+ * `workspace` must hold nf4hip_gemv_workspace_bytes(M,N,K) bytes, be 16-byte aligned, and have
+ * been ZEROED once before its first use; every call leaves it zeroed where that matters, so it
+ * can be reused by later calls on the same stream.  Two calls that may overlap in time (different
+ * streams) need different workspaces.
+ */
+size_t nf4hip_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
+                const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                size_t workspace_bytes, void* stream);
+int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,
+                   const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
+                   const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/*
+ * Prefill-shape fused dequant-matmul, M > 16.  Replaces the dequantize_4bit + F.linear route of
+ * bitsandbytes.matmul_4bit (MatMul4Bit.forward), reached from thunder/transforms/quantization.py:39.
+ * NF4 tiles are expanded to bf16 ( bf16(lut16[c] * absmax) ) in LDS and contracted with bf16 MFMA,
+ * fp32 accumulation, bf16 output.  Same operand layout and fast-path rules as nf4hip_gemv, except
+ * K % 64 == 0 and blocksize == 64 ... 4096 dividing K.  The workspace is reserved for split-K
+ * variants; nf4hip_gemm_workspace_bytes may return 0, in which case NULL is accepted.
+ */
+size_t nf4hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int nf4hip_gemm(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
+                const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                size_t workspace_bytes, void* stream);
+int nf4hip_gemm_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,
+                   const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
+                   const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NF4HIP_H */

@@ -1,0 +1,235 @@
+// C ABI of libnf4hip.so (declared in include/nf4hip.h): argument validation, then launch.
+// Every check runs before the first HIP call so that the error paths are testable without a GPU.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/nf4hip.h"
+#include "nf4_common.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(const char* what, hipError_t e) {
+    return fail(NF4HIP_E_HIP, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// log2 of a supported blocksize, or -1
+int block_log2(int blocksize) {
+    switch (blocksize) {
+        case 64: return 6;
+        case 128: return 7;
+        case 256: return 8;
+        case 512: return 9;
+        case 1024: return 10;
+        case 2048: return 11;
+        case 4096: return 12;
+        default: return -1;
+    }
+}
+
+bool valid_dtype(int d) { return d == NF4HIP_BF16 || d == NF4HIP_F16 || d == NF4HIP_F32; }
+
+int check_nested(const uint8_t* absmax_q, const float* absmax2, const float* map256, int nested_blocksize,
+                 int* nested_log2) {
+    if (!absmax_q || !absmax2 || !map256) return fail(NF4HIP_E_NULL, "nested absmax: null pointer");
+    *nested_log2 = block_log2(nested_blocksize);
+    if (*nested_log2 < 0) return fail(NF4HIP_E_BLOCKSIZE, "nested_blocksize %d unsupported", nested_blocksize);
+    if (!aligned16(absmax_q) || !aligned16(absmax2) || !aligned16(map256))
+        return fail(NF4HIP_E_ALIGN, "nested absmax: pointer not 16-byte aligned");
+    return NF4HIP_OK;
+}
+
+enum MatmulKind { GEMV, GEMM };
+
+int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
+                  const nf4::NestedAbsmax* nested, const float* lut16, const void* bias, int64_t N, int64_t K,
+                  int blocksize, void* out, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* name = kind == GEMV ? "nf4hip_gemv" : "nf4hip_gemm";
+    if (!x || !packed || !lut16 || !out) return fail(NF4HIP_E_NULL, "%s: null pointer", name);
+    if (!nested && !absmax) return fail(NF4HIP_E_NULL, "%s: absmax is null", name);
+    if (x_dtype != NF4HIP_BF16)
+        return fail(valid_dtype(x_dtype) ? NF4HIP_E_DTYPE : NF4HIP_E_DTYPE, "%s: only bf16 x is fused (got dtype %d)",
+                    name, x_dtype);
+    const int bl = block_log2(blocksize);
+    if (bl < 0) return fail(NF4HIP_E_BLOCKSIZE, "%s: blocksize %d unsupported", name, blocksize);
+    if (M <= 0 || N <= 0 || K <= 0) return fail(NF4HIP_E_SHAPE, "%s: M, N, K must be positive", name);
+    if (N > INT32_MAX || K > INT32_MAX || M > INT32_MAX) return fail(NF4HIP_E_SHAPE, "%s: dimension too large", name);
+    if (kind == GEMV) {
+        if (M > 16) return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: M = %lld > 16", (long long)M);
+        if (K % 512) return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: K = %lld is not a multiple of 512", (long long)K);
+    } else {
+        if (K % 64) return fail(NF4HIP_E_SHAPE, "nf4hip_gemm: K = %lld is not a multiple of 64", (long long)K);
+    }
+    if (K % blocksize) return fail(NF4HIP_E_SHAPE, "%s: blocksize %d does not divide K = %lld", name, blocksize, (long long)K);
+    if (!aligned16(x) || !aligned16(packed) || !aligned16(out) || (absmax && !aligned16(absmax)) ||
+        (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
+        return fail(NF4HIP_E_ALIGN, "%s: pointer not 16-byte aligned", name);
+    const size_t need = kind == GEMV ? nf4::gemv_workspace_bytes(M, N, K) : nf4::gemm_workspace_bytes(M, N, K);
+    if (need) {
+        if (!workspace || workspace_bytes < need)
+            return fail(NF4HIP_E_WORKSPACE, "%s: workspace of %zu bytes required, got %zu", name, need,
+                        workspace ? workspace_bytes : (size_t)0);
+        if (!aligned16(workspace)) return fail(NF4HIP_E_ALIGN, "%s: workspace not 16-byte aligned", name);
+    }
+
+    nf4::MatmulArgs a;
+    a.x = static_cast<const uint16_t*>(x);
+    a.packed = packed;
+    a.absmax = absmax;
+    a.nested = nested ? *nested : nf4::NestedAbsmax{nullptr, nullptr, nullptr, 0.0f, 0};
+    a.lut16 = lut16;
+    a.bias = static_cast<const uint16_t*>(bias);
+    a.out = static_cast<uint16_t*>(out);
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.block_log2 = bl;
+    a.workspace = workspace;
+    a.workspace_bytes = workspace_bytes;
+    const hipError_t e = kind == GEMV ? nf4::launch_gemv(a, static_cast<hipStream_t>(stream))
+                                      : nf4::launch_gemm(a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(name, e);
+    return NF4HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nf4hip_abi_version(void) { return NF4HIP_ABI_VERSION; }
+
+const char* nf4hip_last_error(void) { return g_err; }
+
+int nf4hip_quantize(const void* w, int w_dtype, int64_t n, int blocksize, uint8_t* packed, float* absmax,
+                    void* stream) {
+    if (n < 0) return fail(NF4HIP_E_SHAPE, "nf4hip_quantize: n = %lld is negative", (long long)n);
+    if (!valid_dtype(w_dtype)) return fail(NF4HIP_E_DTYPE, "nf4hip_quantize: unknown dtype code %d", w_dtype);
+    const int bl = block_log2(blocksize);
+    if (bl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_quantize: blocksize %d unsupported", blocksize);
+    if (n == 0) return NF4HIP_OK;
+    if (!w || !packed || !absmax) return fail(NF4HIP_E_NULL, "nf4hip_quantize: null pointer");
+    if (!aligned16(w) || !aligned16(packed) || !aligned16(absmax))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_quantize: pointer not 16-byte aligned");
+    const hipError_t e = nf4::launch_quantize(w, w_dtype, n, bl, packed, absmax, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail("nf4hip_quantize", e);
+    return NF4HIP_OK;
+}
+
+int nf4hip_dequantize(const uint8_t* packed, const float* absmax, const float* lut16, int64_t n, int blocksize,
+                      void* out, int out_dtype, void* stream) {
+    if (n < 0) return fail(NF4HIP_E_SHAPE, "nf4hip_dequantize: n = %lld is negative", (long long)n);
+    if (!valid_dtype(out_dtype)) return fail(NF4HIP_E_DTYPE, "nf4hip_dequantize: unknown dtype code %d", out_dtype);
+    const int bl = block_log2(blocksize);
+    if (bl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dequantize: blocksize %d unsupported", blocksize);
+    if (n == 0) return NF4HIP_OK;
+    if (!packed || !absmax || !lut16 || !out) return fail(NF4HIP_E_NULL, "nf4hip_dequantize: null pointer");
+    if (!aligned16(packed) || !aligned16(absmax) || !aligned16(out))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_dequantize: pointer not 16-byte aligned");
+    const nf4::NestedAbsmax none{nullptr, nullptr, nullptr, 0.0f, 0};
+    const hipError_t e =
+        nf4::launch_dequantize(packed, absmax, none, lut16, n, bl, out, out_dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail("nf4hip_dequantize", e);
+    return NF4HIP_OK;
+}
+
+int nf4hip_dq_compress(const float* absmax, int64_t nblocks, int nested_blocksize, const float* map256, float offset,
+                       uint8_t* absmax_q, float* absmax2, void* stream) {
+    if (nblocks < 0) return fail(NF4HIP_E_SHAPE, "nf4hip_dq_compress: nblocks is negative");
+    const int nl = block_log2(nested_blocksize);
+    if (nl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dq_compress: nested_blocksize %d unsupported", nested_blocksize);
+    if (nblocks == 0) return NF4HIP_OK;
+    if (!absmax || !map256 || !absmax_q || !absmax2) return fail(NF4HIP_E_NULL, "nf4hip_dq_compress: null pointer");
+    const hipError_t e =
+        nf4::launch_dq_compress(absmax, nblocks, nl, map256, offset, absmax_q, absmax2, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail("nf4hip_dq_compress", e);
+    return NF4HIP_OK;
+}
+
+int nf4hip_dq_reconstruct(const uint8_t* absmax_q, const float* absmax2, const float* map256, float offset,
+                          int64_t nblocks, int nested_blocksize, float* absmax, void* stream) {
+    if (nblocks < 0) return fail(NF4HIP_E_SHAPE, "nf4hip_dq_reconstruct: nblocks is negative");
+    const int nl = block_log2(nested_blocksize);
+    if (nl < 0)
+        return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dq_reconstruct: nested_blocksize %d unsupported", nested_blocksize);
+    if (nblocks == 0) return NF4HIP_OK;
+    if (!absmax_q || !absmax2 || !map256 || !absmax) return fail(NF4HIP_E_NULL, "nf4hip_dq_reconstruct: null pointer");
+    const nf4::NestedAbsmax nq{absmax_q, absmax2, map256, offset, nl};
+    const hipError_t e = nf4::launch_dq_reconstruct(nq, nblocks, absmax, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail("nf4hip_dq_reconstruct", e);
+    return NF4HIP_OK;
+}
+
+int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const float* absmax2, const float* map256,
+                         float offset, int nested_blocksize, const float* lut16, int64_t n, int blocksize, void* out,
+                         int out_dtype, void* stream) {
+    if (n < 0) return fail(NF4HIP_E_SHAPE, "nf4hip_dequantize_dq: n = %lld is negative", (long long)n);
+    if (!valid_dtype(out_dtype)) return fail(NF4HIP_E_DTYPE, "nf4hip_dequantize_dq: unknown dtype code %d", out_dtype);
+    const int bl = block_log2(blocksize);
+    if (bl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dequantize_dq: blocksize %d unsupported", blocksize);
+    if (n == 0) return NF4HIP_OK;
+    if (!packed || !lut16 || !out) return fail(NF4HIP_E_NULL, "nf4hip_dequantize_dq: null pointer");
+    int nl = 0;
+    const int rc = check_nested(absmax_q, absmax2, map256, nested_blocksize, &nl);
+    if (rc) return rc;
+    if (!aligned16(packed) || !aligned16(out))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_dequantize_dq: pointer not 16-byte aligned");
+    const nf4::NestedAbsmax nq{absmax_q, absmax2, map256, offset, nl};
+    const hipError_t e =
+        nf4::launch_dequantize(packed, nullptr, nq, lut16, n, bl, out, out_dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail("nf4hip_dequantize_dq", e);
+    return NF4HIP_OK;
+}
+
+size_t nf4hip_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) { return nf4::gemv_workspace_bytes(M, N, K); }
+size_t nf4hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return nf4::gemm_workspace_bytes(M, N, K); }
+
+int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
+                const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                size_t workspace_bytes, void* stream) {
+    return matmul_common(GEMV, x, x_dtype, M, packed, absmax, nullptr, lut16, bias_or_null, N, K, blocksize, out,
+                         workspace, workspace_bytes, stream);
+}
+
+int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,
+                   const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
+                   const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+    int nl = 0;
+    const int rc = check_nested(absmax_q, absmax2, map256, nested_blocksize, &nl);
+    if (rc) return rc;
+    const nf4::NestedAbsmax nq{absmax_q, absmax2, map256, offset, nl};
+    return matmul_common(GEMV, x, x_dtype, M, packed, nullptr, &nq, lut16, bias_or_null, N, K, blocksize, out,
+                         workspace, workspace_bytes, stream);
+}
+
+int nf4hip_gemm(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
+                const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                size_t workspace_bytes, void* stream) {
+    return matmul_common(GEMM, x, x_dtype, M, packed, absmax, nullptr, lut16, bias_or_null, N, K, blocksize, out,
+                         workspace, workspace_bytes, stream);
+}
+
+int nf4hip_gemm_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,
+                   const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
+                   const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+    int nl = 0;
+    const int rc = check_nested(absmax_q, absmax2, map256, nested_blocksize, &nl);
+    if (rc) return rc;
+    const nf4::NestedAbsmax nq{absmax_q, absmax2, map256, offset, nl};
+    return matmul_common(GEMM, x, x_dtype, M, packed, nullptr, &nq, lut16, bias_or_null, N, K, blocksize, out,
+                         workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

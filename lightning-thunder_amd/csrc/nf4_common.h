@@ -1,0 +1,79 @@
+// Internal declarations shared by the kernel files and the C-ABI front end of libnf4hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nf4 {
+
+enum : int { BF16 = 0, F16 = 1, F32 = 2 };
+
+// Nested ("double") quantisation of absmax; all NULL/0 when absmax is given directly as fp32.
+struct NestedAbsmax {
+    const uint8_t* q;      // [nblocks] 8-bit codes
+    const float* absmax2;  // [ceil(nblocks / nested_blocksize)]
+    const float* map256;   // [256] dynamic map
+    float offset;
+    int nested_log2;       // log2(nested_blocksize)
+};
+
+struct MatmulArgs {
+    const uint16_t* x;    // [M, K] bf16
+    const uint8_t* packed;  // [N*K/2]
+    const float* absmax;  // [N*K/blocksize] or NULL when nested is used
+    NestedAbsmax nested;
+    const float* lut16;
+    const uint16_t* bias;  // [N] bf16 or NULL
+    uint16_t* out;         // [M, N] bf16
+    int M, N, K;
+    int block_log2;  // log2(blocksize)
+    void* workspace;
+    size_t workspace_bytes;
+};
+
+// Launchers (defined next to their kernels).  They assume validated arguments and return the
+// hipError_t of the launch.
+hipError_t launch_quantize(const void* w, int w_dtype, int64_t n, int block_log2, uint8_t* packed, float* absmax,
+                           hipStream_t stream);
+hipError_t launch_dequantize(const uint8_t* packed, const float* absmax, const NestedAbsmax& nested,
+                             const float* lut16, int64_t n, int block_log2, void* out, int out_dtype,
+                             hipStream_t stream);
+hipError_t launch_dq_compress(const float* absmax, int64_t nblocks, int nested_log2, const float* map256,
+                              float offset, uint8_t* q, float* absmax2, hipStream_t stream);
+hipError_t launch_dq_reconstruct(const NestedAbsmax& nested, int64_t nblocks, float* absmax, hipStream_t stream);
+
+size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
+hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream);
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream);
+
+// ---------------------------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------------------------
+
+// 16-byte streaming (non-temporal) load: data that is read exactly once should not displace what
+// the caches hold for re-use.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load16_stream(const void* p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// fp32 -> bf16 bits, round to nearest even (finite inputs; NaN is quieted).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// Reconstruct one absmax value from its nested form: (map * absmax2) + offset, two roundings.
+__device__ __forceinline__ float nested_absmax(const NestedAbsmax& nq, int64_t block) {
+    float m = nq.map256[nq.q[block]];
+    float s = nq.absmax2[block >> nq.nested_log2];
+    return __fadd_rn(__fmul_rn(m, s), nq.offset);
+}
+
+}  // namespace nf4

@@ -1,0 +1,286 @@
+// NF4 blockwise quantize / dequantize kernels for gfx950 (bit-exact contract, HBM-bound).
+//
+// quantize  : bitsandbytes.functional.quantize_4bit(w, quant_type="nf4"), the call made at
+//             thunder/transforms/quantization.py:63
+// dequantize: bitsandbytes.functional.dequantize_4bit, reached through matmul_4bit from
+//             thunder/transforms/quantization.py:39
+//
+// Data layout.  The weight is a flat row-major array of n elements.  Every lane owns 8
+// consecutive elements: one 128-bit load of bf16/f16 input (two for fp32), one 32-bit word of
+// packed codes, one 128-bit store of bf16/f16 output.  A quantisation block of B elements is
+// therefore B/8 adjacent lanes, and the block maximum is a butterfly over those lanes.
+//
+// This file is compiled with -ffp-contract=off: every product and sum below is rounded once.
+#include <hip/hip_fp16.h>
+
+#include "nf4_common.h"
+
+namespace nf4 {
+namespace {
+
+// Decision thresholds of the NF4 code (midpoints of adjacent code values) as the exact fp32
+// bit patterns a C compiler produces for the literals -0.8480964004993439f ... 0.8614784181118011f.
+__device__ __forceinline__ float thr(int j) {
+    constexpr uint32_t T[15] = {0xBF591CD9u, 0xBF1C5270u, 0xBEEB8480u, 0xBEADEA76u, 0xBE703CECu,
+                                0xBE0D38BCu, 0xBD3A7871u, 0x3D22FAFFu, 0x3DF64863u, 0x3E5067E0u,
+                                0x3E9582D4u, 0x3EC753F9u, 0x3F006D03u, 0x3F248DAFu, 0x3F5C89D9u};
+    return __uint_as_float(T[j]);
+}
+
+// code = number of thresholds strictly below s (NaN -> 0), as a 4-level binary search.
+__device__ __forceinline__ uint32_t nf4_code(float s) {
+    const bool b3 = s > thr(7);
+    const float t2 = b3 ? thr(11) : thr(3);
+    const bool b2 = s > t2;
+    const float t1 = b3 ? (b2 ? thr(13) : thr(9)) : (b2 ? thr(5) : thr(1));
+    const bool b1 = s > t1;
+    const float t0 = b3 ? (b2 ? (b1 ? thr(14) : thr(12)) : (b1 ? thr(10) : thr(8)))
+                        : (b2 ? (b1 ? thr(6) : thr(4)) : (b1 ? thr(2) : thr(0)));
+    const bool b0 = s > t0;
+    return (uint32_t)b3 * 8u + (uint32_t)b2 * 4u + (uint32_t)b1 * 2u + (uint32_t)b0;
+}
+
+__device__ __forceinline__ float load_elem(const void* w, int dtype, int64_t i) {
+    if (dtype == BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(w)[i]);
+    if (dtype == F16) return __half2float(reinterpret_cast<const __half*>(w)[i]);
+    return reinterpret_cast<const float*>(w)[i];
+}
+
+// Load the 8 elements [e0, e0+8) as fp32; elements at or beyond n read as 0.
+__device__ __forceinline__ void load8(const void* w, int dtype, int64_t e0, int64_t n, float v[8]) {
+    if (e0 + 8 <= n) {
+        if (dtype == F32) {
+            const float4 a = reinterpret_cast<const float4*>(w)[e0 / 4];
+            const float4 b = reinterpret_cast<const float4*>(w)[e0 / 4 + 1];
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+            v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        } else {
+            const uint4 q = reinterpret_cast<const uint4*>(w)[e0 / 8];
+            const uint32_t d[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (dtype == BF16) {
+                    v[2 * j] = __uint_as_float(d[j] << 16);
+                    v[2 * j + 1] = __uint_as_float(d[j] & 0xffff0000u);
+                } else {
+                    v[2 * j] = __half2float(__ushort_as_half((unsigned short)(d[j] & 0xffffu)));
+                    v[2 * j + 1] = __half2float(__ushort_as_half((unsigned short)(d[j] >> 16)));
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (e0 + j < n) ? load_elem(w, dtype, e0 + j) : 0.0f;
+    }
+}
+
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void quantize_kernel(const void* __restrict__ w, int dtype, int64_t n,
+                                                           int block_log2, uint8_t* __restrict__ packed,
+                                                           float* __restrict__ absmax) {
+    __shared__ float wave_max[THREADS / 64];
+    const int tid = threadIdx.x;
+    const int64_t e0 = ((int64_t)blockIdx.x * THREADS + tid) * 8;
+    const int group = 1 << (block_log2 - 3);  // lanes per quantisation block
+
+    float v[8];
+    load8(w, dtype, e0, n, v);
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
+
+    // max over the lanes of one quantisation block
+    const int in_wave = group < 64 ? group : 64;
+    for (int off = 1; off < in_wave; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if (group > 64) {  // uniform branch: blocks of 1024, 2048 or 4096 elements span several waves
+        if ((tid & 63) == 0) wave_max[tid >> 6] = m;
+        __syncthreads();
+        const int waves = group >> 6;
+        const int first = (tid >> 6) & ~(waves - 1);
+        for (int j = 0; j < waves; ++j) m = fmaxf(m, wave_max[first + j]);
+    }
+
+    if (e0 >= n) return;
+    if ((tid & (group - 1)) == 0) absmax[e0 >> block_log2] = m;
+
+    const float inv = __fdiv_rn(1.0f, m);
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t hi = nf4_code(__fmul_rn(v[2 * j], inv));
+        const uint32_t lo = nf4_code(__fmul_rn(v[2 * j + 1], inv));
+        word |= ((hi << 4) | lo) << (8 * j);
+    }
+    if (e0 + 8 <= n) {
+        reinterpret_cast<uint32_t*>(packed)[e0 / 8] = word;
+    } else {
+        const int64_t nbytes = (n + 1) / 2;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (e0 / 2 + j < nbytes) packed[e0 / 2 + j] = (uint8_t)(word >> (8 * j));
+    }
+}
+
+template <bool NESTED>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ packed,
+                                                         const float* __restrict__ absmax, NestedAbsmax nq,
+                                                         const float* __restrict__ lut16, int64_t n, int block_log2,
+                                                         void* __restrict__ out, int out_dtype) {
+    __shared__ float lut[16];
+    const int tid = threadIdx.x;
+    if (tid < 16) lut[tid] = lut16[tid];
+    __syncthreads();
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + tid) * 8;
+    if (e0 >= n) return;
+
+    const int64_t blk = e0 >> block_log2;
+    const float s = NESTED ? nested_absmax(nq, blk) : absmax[blk];
+    const bool full = e0 + 8 <= n;
+    uint32_t word;
+    if (full) {
+        word = reinterpret_cast<const uint32_t*>(packed)[e0 / 8];
+    } else {
+        const int64_t nbytes = (n + 1) / 2;
+        word = 0;
+        for (int j = 0; j < 4; ++j)
+            if (e0 / 2 + j < nbytes) word |= (uint32_t)packed[e0 / 2 + j] << (8 * j);
+    }
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t byte = (word >> (8 * j)) & 0xffu;
+        v[2 * j] = __fmul_rn(lut[byte >> 4], s);
+        v[2 * j + 1] = __fmul_rn(lut[byte & 15u], s);
+    }
+    if (out_dtype == F32) {
+        float* o = reinterpret_cast<float*>(out);
+        if (full) {
+            reinterpret_cast<float4*>(o)[e0 / 4] = make_float4(v[0], v[1], v[2], v[3]);
+            reinterpret_cast<float4*>(o)[e0 / 4 + 1] = make_float4(v[4], v[5], v[6], v[7]);
+        } else {
+            for (int j = 0; j < 8; ++j)
+                if (e0 + j < n) o[e0 + j] = v[j];
+        }
+    } else {
+        uint32_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            h[j] = out_dtype == BF16 ? f32_to_bf16_bits(v[j]) : (uint32_t)__half_as_ushort(__float2half_rn(v[j]));
+        uint16_t* o = reinterpret_cast<uint16_t*>(out);
+        if (full) {
+            uint4 q;
+            q.x = h[0] | (h[1] << 16);
+            q.y = h[2] | (h[3] << 16);
+            q.z = h[4] | (h[5] << 16);
+            q.w = h[6] | (h[7] << 16);
+            reinterpret_cast<uint4*>(o)[e0 / 8] = q;
+        } else {
+            for (int j = 0; j < 8; ++j)
+                if (e0 + j < n) o[e0 + j] = (uint16_t)h[j];
+        }
+    }
+}
+
+// One workgroup per nested block: r = absmax - offset, absmax2 = max|r|, then the nearest entry
+// of the 256-entry map (lowest index on ties) for every r * (1/absmax2).
+__global__ __launch_bounds__(256) void dq_compress_kernel(const float* __restrict__ absmax, int64_t nblocks,
+                                                          int nested_log2, const float* __restrict__ map256,
+                                                          float offset, uint8_t* __restrict__ q,
+                                                          float* __restrict__ absmax2) {
+    __shared__ float map[256];
+    __shared__ float red[4];
+    __shared__ int zero_code;
+    const int tid = threadIdx.x;
+    const int nested = 1 << nested_log2;
+    const int64_t base = (int64_t)blockIdx.x << nested_log2;
+    map[tid] = map256[tid];
+    if (tid == 0) zero_code = 255;
+    __syncthreads();
+    if (map[tid] == 0.0f) atomicMin(&zero_code, tid);
+
+    float m = 0.0f;
+    for (int i = tid; i < nested; i += 256) {
+        const int64_t idx = base + i;
+        if (idx < nblocks) m = fmaxf(m, fabsf(__fsub_rn(absmax[idx], offset)));
+    }
+    for (int off = 1; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    if (tid == 0) absmax2[blockIdx.x] = m;
+
+    const float inv = __fdiv_rn(1.0f, m);
+    for (int i = tid; i < nested; i += 256) {
+        const int64_t idx = base + i;
+        if (idx >= nblocks) continue;
+        int best = zero_code;
+        if (m != 0.0f) {
+            const float s = __fmul_rn(__fsub_rn(absmax[idx], offset), inv);
+            float bestd = INFINITY;
+            best = 0;
+            for (int j = 0; j < 256; ++j) {
+                const float d = fabsf(__fsub_rn(s, map[j]));
+                if (d < bestd) {
+                    bestd = d;
+                    best = j;
+                }
+            }
+        }
+        q[idx] = (uint8_t)best;
+    }
+}
+
+__global__ __launch_bounds__(256) void dq_reconstruct_kernel(NestedAbsmax nq, int64_t nblocks,
+                                                             float* __restrict__ absmax) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nblocks) absmax[i] = nested_absmax(nq, i);
+}
+
+}  // namespace
+
+hipError_t launch_quantize(const void* w, int w_dtype, int64_t n, int block_log2, uint8_t* packed, float* absmax,
+                           hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    if (block_log2 == 12) {
+        const int64_t grid = (n + 4095) / 4096;
+        hipLaunchKernelGGL(quantize_kernel<512>, dim3((unsigned)grid), dim3(512), 0, stream, w, w_dtype, n, block_log2,
+                           packed, absmax);
+    } else {
+        const int64_t grid = (n + 2047) / 2048;
+        hipLaunchKernelGGL(quantize_kernel<256>, dim3((unsigned)grid), dim3(256), 0, stream, w, w_dtype, n, block_log2,
+                           packed, absmax);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize(const uint8_t* packed, const float* absmax, const NestedAbsmax& nested,
+                             const float* lut16, int64_t n, int block_log2, void* out, int out_dtype,
+                             hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    const int64_t grid = (n + 2047) / 2048;
+    if (nested.q)
+        hipLaunchKernelGGL(dequantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, stream, packed, absmax, nested,
+                           lut16, n, block_log2, out, out_dtype);
+    else
+        hipLaunchKernelGGL(dequantize_kernel<false>, dim3((unsigned)grid), dim3(256), 0, stream, packed, absmax,
+                           nested, lut16, n, block_log2, out, out_dtype);
+    return hipGetLastError();
+}
+
+hipError_t launch_dq_compress(const float* absmax, int64_t nblocks, int nested_log2, const float* map256,
+                              float offset, uint8_t* q, float* absmax2, hipStream_t stream) {
+    if (nblocks == 0) return hipSuccess;
+    const int64_t grid = (nblocks + (1 << nested_log2) - 1) >> nested_log2;
+    hipLaunchKernelGGL(dq_compress_kernel, dim3((unsigned)grid), dim3(256), 0, stream, absmax, nblocks, nested_log2,
+                       map256, offset, q, absmax2);
+    return hipGetLastError();
+}
+
+hipError_t launch_dq_reconstruct(const NestedAbsmax& nested, int64_t nblocks, float* absmax, hipStream_t stream) {
+    if (nblocks == 0) return hipSuccess;
+    const int64_t grid = (nblocks + 255) / 256;
+    hipLaunchKernelGGL(dq_reconstruct_kernel, dim3((unsigned)grid), dim3(256), 0, stream, nested, nblocks, absmax);
+    return hipGetLastError();
+}
+
+}  // namespace nf4

@@ -1,0 +1,280 @@
+"""Tensor-level NF4 ops on PyTorch-ROCm tensors, backed by ``libnf4hip.so``.
+
+These are the functions the executor registers as operators.  They mirror what the reference
+gets from bitsandbytes at thunder/transforms/quantization.py:35-39,63:
+
+* :func:`quantize_nf4`      -- ``bitsandbytes.functional.quantize_4bit(w, quant_type="nf4")``
+* :func:`dequantize_nf4`    -- ``bitsandbytes.functional.dequantize_4bit``
+* :func:`matmul_nf4`        -- ``bitsandbytes.matmul_4bit(x, qweight.t(), bias, quant_state)``
+
+All tensors must live on the GPU (``device.type == "cuda"`` on ROCm builds of torch); kernels are
+queued on ``torch.cuda.current_stream()`` and nothing synchronises.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
+
+_DTYPE_CODE = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32}
+
+# fp32 NF4 code values (QLoRA), index = 4-bit code; the table bitsandbytes stores as QuantState.code
+NF4_CODE = (
+    -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453,
+    -0.28444138169288635, -0.18477343022823334, -0.09105003625154495, 0.0,
+    0.07958029955625534, 0.16093020141124725, 0.24611230194568634, 0.33791524171829224,
+    0.44070982933044434, 0.5626170039176941, 0.7229568362236023, 1.0,
+)  # fmt: skip
+
+
+def nf4_code(device=None, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """The 16-entry code book as a tensor (``quant_map`` / ``QuantState.code``)."""
+    return torch.tensor(NF4_CODE, dtype=torch.float32, device=device).to(dtype)
+
+
+def dynamic_map(device=None) -> torch.Tensor:
+    """The 256-entry signed "dynamic" 8-bit code bitsandbytes uses for nested absmax quantisation
+    (``create_dynamic_map(signed=True, max_exponent_bits=7, total_bits=8)``)."""
+    data: list[float] = []
+    for i in range(7):
+        boundaries = torch.linspace(0.1, 1, 2**i + 1)
+        means = (boundaries[:-1] + boundaries[1:]) / 2.0
+        scale = 10 ** (-6 + i)
+        data += (scale * means).tolist()
+        data += (-scale * means).tolist()
+    data += [0.0, 1.0]
+    assert len(data) == 256
+    data.sort()
+    return torch.tensor(data, dtype=torch.float32, device=device)
+
+
+@dataclass
+class NestedAbsmax:
+    """absmax in nested ("double quantised") form: ``map256[q] * absmax2[i // blocksize] + offset``."""
+
+    q: torch.Tensor  # uint8 [nblocks]
+    absmax2: torch.Tensor  # fp32 [ceil(nblocks / blocksize)]
+    map256: torch.Tensor  # fp32 [256]
+    offset: float
+    blocksize: int = 256
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and t.device.type != "cuda":
+            raise RuntimeError(f"NF4 HIP ops need GPU tensors, got a tensor on {t.device}")
+
+
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned view or copy of ``t``."""
+    t = t.contiguous()
+    if t.data_ptr() % 16:
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
+
+
+def _check_blocksize(blocksize: int) -> None:
+    if blocksize not in SUPPORTED_BLOCKSIZES:
+        raise ValueError(f"blocksize must be one of {SUPPORTED_BLOCKSIZES}, got {blocksize}")
+
+
+# ------------------------------------------------------------------------------------------------
+# quantize / dequantize
+# ------------------------------------------------------------------------------------------------
+
+
+def quantize_nf4(w: torch.Tensor, blocksize: int = 64):
+    """Blockwise NF4 quantisation of ``w`` (bf16/f16/f32, any shape, flattened row-major).
+
+    Returns ``(qweight uint8 [(n+1)//2, 1], absmax fp32 [ceil(n/blocksize)], code fp32 [16])``,
+    the tensors the reference stores as ``<w>``, ``<w>.absmax`` and ``<w>.code``
+    (thunder/transforms/quantization.py:87-89).
+    """
+    _check_blocksize(blocksize)
+    _require_gpu(w)
+    if w.dtype not in _DTYPE_CODE:
+        raise TypeError(f"cannot quantize dtype {w.dtype}")
+    lib = _lib.load()
+    w = _aligned(w.detach())
+    n = w.numel()
+    with torch.cuda.device(w.device):
+        packed = torch.empty(((n + 1) // 2, 1), dtype=torch.uint8, device=w.device)
+        absmax = torch.empty(((n + blocksize - 1) // blocksize,), dtype=torch.float32, device=w.device)
+        _lib.check(lib.nf4hip_quantize(w.data_ptr(), _DTYPE_CODE[w.dtype], n, blocksize, packed.data_ptr(), absmax.data_ptr(), _stream()))
+    return packed, absmax, nf4_code(w.device)
+
+
+def dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape) -> torch.Tensor:
+    """``cast(quant_map[code] * absmax[block])`` reshaped to ``shape``; ``absmax`` is an fp32
+    tensor or a :class:`NestedAbsmax`."""
+    _check_blocksize(blocksize)
+    if dtype not in _DTYPE_CODE:
+        raise TypeError(f"cannot dequantize to dtype {dtype}")
+    shape = tuple(int(s) for s in shape)
+    n = math.prod(shape)
+    lib = _lib.load()
+    _require_gpu(qweight, quant_map)
+    qweight = _aligned(qweight)
+    if qweight.numel() < (n + 1) // 2:
+        raise ValueError(f"qweight holds {qweight.numel()} bytes, shape {shape} needs {(n + 1) // 2}")
+    quant_map = _aligned(quant_map.to(torch.float32))
+    nblocks = (n + blocksize - 1) // blocksize
+    with torch.cuda.device(qweight.device):
+        out = torch.empty(shape, dtype=dtype, device=qweight.device)
+        if isinstance(absmax, NestedAbsmax):
+            nq = _nested_args(absmax, nblocks)
+            _lib.check(
+                lib.nf4hip_dequantize_dq(qweight.data_ptr(), nq[0].data_ptr(), nq[1].data_ptr(), nq[2].data_ptr(), nq[3], nq[4],
+                                         quant_map.data_ptr(), n, blocksize, out.data_ptr(), _DTYPE_CODE[dtype], _stream())
+            )  # fmt: skip
+        else:
+            _require_gpu(absmax)
+            absmax = _aligned(absmax.to(torch.float32))
+            if absmax.numel() < nblocks:
+                raise ValueError(f"absmax holds {absmax.numel()} entries, need {nblocks}")
+            _lib.check(
+                lib.nf4hip_dequantize(qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(), n, blocksize,
+                                      out.data_ptr(), _DTYPE_CODE[dtype], _stream())
+            )  # fmt: skip
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# nested (double) quantisation of absmax
+# ------------------------------------------------------------------------------------------------
+
+
+def _nested_args(nq: NestedAbsmax, nblocks: int):
+    _require_gpu(nq.q, nq.absmax2, nq.map256)
+    if nq.q.numel() < nblocks:
+        raise ValueError(f"nested absmax holds {nq.q.numel()} codes, need {nblocks}")
+    return (_aligned(nq.q), _aligned(nq.absmax2.to(torch.float32)), _aligned(nq.map256.to(torch.float32)), float(nq.offset), int(nq.blocksize))
+
+
+def compress_absmax(absmax: torch.Tensor, nested_blocksize: int = 256, map256: torch.Tensor | None = None) -> NestedAbsmax:
+    """bitsandbytes' ``compress_statistics=True``: subtract the mean, then 8-bit blockwise quantise.
+    The mean is taken in float64 and rounded to fp32 once, so it does not depend on reduction order."""
+    _check_blocksize(nested_blocksize)
+    _require_gpu(absmax)
+    lib = _lib.load()
+    absmax = _aligned(absmax.to(torch.float32))
+    nb = absmax.numel()
+    offset = float(absmax.double().mean().to(torch.float32)) if nb else 0.0
+    with torch.cuda.device(absmax.device):
+        if map256 is None:
+            map256 = dynamic_map(absmax.device)
+        map256 = _aligned(map256.to(torch.float32))
+        q = torch.empty(nb, dtype=torch.uint8, device=absmax.device)
+        absmax2 = torch.empty(((nb + nested_blocksize - 1) // nested_blocksize,), dtype=torch.float32, device=absmax.device)
+        _lib.check(lib.nf4hip_dq_compress(absmax.data_ptr(), nb, nested_blocksize, map256.data_ptr(), offset, q.data_ptr(), absmax2.data_ptr(), _stream()))
+    return NestedAbsmax(q, absmax2, map256, offset, nested_blocksize)
+
+
+def reconstruct_absmax(nq: NestedAbsmax) -> torch.Tensor:
+    lib = _lib.load()
+    nb = nq.q.numel()
+    q, a2, m, off, bs = _nested_args(nq, nb)
+    with torch.cuda.device(q.device):
+        out = torch.empty(nb, dtype=torch.float32, device=q.device)
+        _lib.check(lib.nf4hip_dq_reconstruct(q.data_ptr(), a2.data_ptr(), m.data_ptr(), off, nb, bs, out.data_ptr(), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# matmul
+# ------------------------------------------------------------------------------------------------
+
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _gemv_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Zero-initialised scratch for the gemv kernel, one per (device, stream); the kernel leaves
+    its counters zeroed, so the buffer is reused without clearing."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape) -> str:
+    """Which kernel serves this call: ``"gemv"``, ``"gemm"`` or ``"dequant+linear"``.
+
+    Mirrors bitsandbytes.matmul_4bit: the fused single-row kernel when the shape allows, else
+    dequantize followed by a dense matmul.
+    """
+    N, K = shape
+    M = x.numel() // K if K else 0
+    fused = (
+        x.dtype == torch.bfloat16
+        and dtype == torch.bfloat16
+        and (bias is None or bias.dtype == torch.bfloat16)
+        and blocksize in SUPPORTED_BLOCKSIZES
+        and M > 0
+        and K % 64 == 0
+        and K % blocksize == 0
+    )
+    if not fused:
+        return "dequant+linear"
+    if M <= 16 and K % 512 == 0:
+        return "gemv"
+    return "gemm"
+
+
+def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> torch.Tensor:
+    """``x @ dequantize(qweight).T + bias`` with the signature of the reference operator
+    ``bnb_matmul_nf4`` (thunder/transforms/quantization.py:34).  ``absmax`` may be a
+    :class:`NestedAbsmax`."""
+    shape = tuple(int(s) for s in shape)
+    assert len(shape) == 2
+    N, K = shape
+    assert x.shape[-1] == K, f"{x.shape=}, rhs {shape=}"
+    _require_gpu(x, qweight, quant_map, bias)
+    route = fused_route(x, bias, blocksize, dtype, shape)
+    if route == "dequant+linear":
+        w = dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape).to(x.dtype)
+        return torch.nn.functional.linear(x, w, bias)
+
+    lib = _lib.load()
+    x2 = _aligned(x.reshape(-1, K))
+    M = x2.shape[0]
+    qweight = _aligned(qweight)
+    if qweight.numel() < N * K // 2:
+        raise ValueError(f"qweight holds {qweight.numel()} bytes, shape {shape} needs {N * K // 2}")
+    quant_map = _aligned(quant_map.to(torch.float32))
+    b = None if bias is None else bias.contiguous()
+    nblocks = N * K // blocksize
+    with torch.cuda.device(x.device):
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        if route == "gemv":
+            need = lib.nf4hip_gemv_workspace_bytes(M, N, K)
+            ws = _gemv_workspace(x.device, need)
+            ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+            fn, fn_dq = lib.nf4hip_gemv, lib.nf4hip_gemv_dq
+        else:
+            ws_ptr, ws_bytes = None, 0
+            fn, fn_dq = lib.nf4hip_gemm, lib.nf4hip_gemm_dq
+        bptr = None if b is None else b.data_ptr()
+        if isinstance(absmax, NestedAbsmax):
+            q, a2, m256, off, nbs = _nested_args(absmax, nblocks)
+            _lib.check(fn_dq(x2.data_ptr(), _lib.BF16, M, qweight.data_ptr(), q.data_ptr(), a2.data_ptr(), m256.data_ptr(), off, nbs,
+                             quant_map.data_ptr(), bptr, N, K, blocksize, out.data_ptr(), ws_ptr, ws_bytes, _stream()))  # fmt: skip
+        else:
+            _require_gpu(absmax)
+            absmax = _aligned(absmax.to(torch.float32))
+            if absmax.numel() < nblocks:
+                raise ValueError(f"absmax holds {absmax.numel()} entries, need {nblocks}")
+            _lib.check(fn(x2.data_ptr(), _lib.BF16, M, qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(), bptr,
+                          N, K, blocksize, out.data_ptr(), ws_ptr, ws_bytes, _stream()))  # fmt: skip
+    return out.reshape(*x.shape[:-1], N)

@@ -1,0 +1,296 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+quantize / dequantize: bit-exact.  matmul: rtol = atol = 2e-2 against the float64-accumulated
+dequantize-then-matmul (the tolerance the north star states for bf16).
+"""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _weights(shape, seed, dtype=torch.bfloat16, std=0.02):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * std).to(dtype)
+
+
+def _acts(shape, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype)
+
+
+def _sync_print(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------------------------------------
+# quantize
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize(
+    "shape",
+    [(2, 2), (1, 1), (3, 21), (64, 64), (64, 1376), (7, 999), (512, 4096), (1, 64 * 5 + 2)],
+)
+def test_quantize_bit_exact(ta, oracle, dtype, shape):
+    _sync_print(f"quantize {dtype} {shape}")
+    w = _weights(shape, seed=sum(shape), dtype=dtype)
+    qw, absmax, code = ta.quantize_nf4(w.to(DEV))
+    qw_o, absmax_o = oracle.C().quantize(w, 64)
+    assert qw.shape == qw_o.shape and qw.dtype == torch.uint8
+    assert torch.equal(qw.cpu(), qw_o)
+    assert torch.equal(absmax.cpu(), absmax_o)
+    assert torch.equal(code.cpu(), oracle.nf4_lut())
+
+
+@pytest.mark.parametrize("blocksize", [64, 128, 256, 512, 1024, 2048, 4096])
+def test_quantize_blocksizes(ta, oracle, blocksize):
+    _sync_print(f"quantize blocksize {blocksize}")
+    w = _weights((37, 1000), seed=blocksize)  # partial last block for every blocksize
+    qw, absmax, _ = ta.quantize_nf4(w.to(DEV), blocksize=blocksize)
+    qw_o, absmax_o = oracle.C().quantize(w, blocksize)
+    assert torch.equal(qw.cpu(), qw_o)
+    assert torch.equal(absmax.cpu(), absmax_o)
+
+
+def test_quantize_corner_cases(ta, oracle):
+    _sync_print("quantize corner cases")
+    w = torch.zeros(4, 64, dtype=torch.bfloat16)
+    w[1, 5] = 0.5  # a block with a single non-zero
+    w[2] = torch.linspace(-1, 1, 64).to(torch.bfloat16)  # contains +-absmax exactly
+    w[3, ::2] = -3.0
+    qw, absmax, _ = ta.quantize_nf4(w.to(DEV))
+    qw_o, absmax_o = oracle.C().quantize(w, 64)
+    assert torch.equal(qw.cpu(), qw_o)
+    assert torch.equal(absmax.cpu(), absmax_o)
+    codes = oracle.unpack_codes(qw.cpu(), w.numel()).view(4, 64)
+    assert (codes[0] == 0).all() and absmax[0].item() == 0.0  # zero block: 0*inf = NaN -> code 0
+    assert codes[1, 5] == 15 and (codes[1, :5] == 7).all()
+    assert codes[2, 0] == 0 and codes[2, 63] == 15
+    # zero block dequantizes to -0.0 (code 0 is -1.0, times absmax 0)
+    deq = ta.dequantize_nf4(qw, absmax, ta.nf4_code(DEV), 64, torch.bfloat16, w.shape)
+    assert (deq[0].cpu().view(torch.int16) == -32768).all()
+
+
+def test_quantize_exhaustive_bf16(ta, oracle):
+    """Every finite bf16 bit pattern, in blocks whose absmax is pinned to a chosen value."""
+    _sync_print("quantize exhaustive bf16")
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16)
+    vals = bits.view(torch.bfloat16)
+    vals = vals[torch.isfinite(vals.float())]
+    for amax in [2.0**-7, 0.025146484375, 0.0517578125, 0.10595703125, 1.0, 3.5, 65280.0]:
+        v = vals[vals.float().abs() <= amax]
+        pad = (-v.numel()) % 63
+        v = torch.cat([v, torch.zeros(pad, dtype=torch.bfloat16)]).view(-1, 63)
+        w = torch.cat([torch.full((v.shape[0], 1), amax, dtype=torch.bfloat16), v], dim=1).contiguous()
+        qw, absmax, _ = ta.quantize_nf4(w.to(DEV))
+        qw_o, absmax_o = oracle.C().quantize(w, 64)
+        assert torch.equal(qw.cpu(), qw_o), f"absmax {amax}"
+        assert torch.equal(absmax.cpu(), absmax_o)
+
+
+# ------------------------------------------------------------------------------------------------
+# dequantize
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("lut_mode", ["f32", "rounded"])
+def test_dequantize_exhaustive(ta, oracle, dtype, lut_mode):
+    """16 codes x every non-negative finite bf16 absmax."""
+    _sync_print(f"dequantize exhaustive {dtype} {lut_mode}")
+    bits = torch.arange(0, 0x7F80, dtype=torch.int32).to(torch.int16)
+    amax = bits.view(torch.bfloat16).float()  # 32640 values
+    nb = amax.numel()
+    codes = (torch.arange(64) % 16).to(torch.uint8).repeat(nb, 1)  # each block holds all 16 codes, 4 times
+    packed = ((codes[:, 0::2] << 4) | codes[:, 1::2]).reshape(-1, 1).contiguous()
+    lut = oracle.nf4_lut()
+    if lut_mode == "rounded":
+        lut = lut.to(dtype).float()
+    out = ta.dequantize_nf4(packed.to(DEV), amax.to(DEV), lut.to(DEV), 64, dtype, (nb, 64))
+    ref = oracle.C().dequantize(packed, amax, lut, 64, dtype, (nb, 64))
+    assert torch.equal(out.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       ref.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+@pytest.mark.parametrize("shape", [(2, 2), (3, 21), (64, 1376), (7, 999), (256, 4096)])
+@pytest.mark.parametrize("blocksize", [64, 256, 4096])
+def test_dequantize_shapes(ta, oracle, shape, blocksize):
+    _sync_print(f"dequantize {shape} {blocksize}")
+    w = _weights(shape, seed=3)
+    qw, absmax = oracle.C().quantize(w, blocksize)
+    out = ta.dequantize_nf4(qw.to(DEV), absmax.to(DEV), ta.nf4_code(DEV), blocksize, torch.bfloat16, shape)
+    ref = oracle.C().dequantize(qw, absmax, oracle.nf4_lut(), blocksize, torch.bfloat16, shape)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+    # round trip bound: |deq - w| <= absmax * (largest code gap)/2 (+ bf16 rounding)
+    err = (out.cpu().float() - w.float()).abs().view(-1)
+    bound = absmax.repeat_interleave(blocksize)[: err.numel()] * (0.3038072 / 2 + 2**-8)
+    assert (err <= bound).all()
+
+
+def test_nested_absmax(ta, oracle):
+    _sync_print("nested absmax")
+    w = _weights((1024, 1024), seed=11)
+    qw, absmax = oracle.C().quantize(w, 64)
+    nq = ta.compress_absmax(absmax.to(DEV))
+    D = oracle.create_dynamic_map()
+    assert torch.equal(nq.map256.cpu(), D)
+    off = oracle.C().dq_offset(absmax)
+    assert nq.offset == off
+    q_o, a2_o = oracle.C().dq_compress(absmax, D, off)
+    assert torch.equal(nq.q.cpu(), q_o)
+    assert torch.equal(nq.absmax2.cpu(), a2_o)
+    rec = ta.reconstruct_absmax(nq)
+    rec_o = oracle.C().dq_reconstruct(q_o, a2_o, D, off)
+    assert torch.equal(rec.cpu(), rec_o)
+    deq = ta.dequantize_nf4(qw.to(DEV), nq, ta.nf4_code(DEV), 64, torch.bfloat16, w.shape)
+    deq_o = oracle.C().dequantize(qw, rec_o, oracle.nf4_lut(), 64, torch.bfloat16, w.shape)
+    assert torch.equal(deq.cpu().view(torch.int16), deq_o.view(torch.int16))
+
+
+# ------------------------------------------------------------------------------------------------
+# matmul
+# ------------------------------------------------------------------------------------------------
+
+
+def _matmul_case(ta, oracle, M, N, K, blocksize=64, bias=False, nested=False, seed=0, x_shape=None):
+    w = _weights((N, K), seed=1000 + seed)
+    x = _acts(x_shape or (M, K), seed=2000 + seed)
+    b = _acts((N,), seed=3000 + seed) if bias else None
+    qw, absmax = oracle.C().quantize(w, blocksize)
+    lut = oracle.nf4_lut()
+    absmax_dev = absmax.to(DEV)
+    absmax_ref = absmax
+    if nested:
+        absmax_dev = ta.compress_absmax(absmax.to(DEV))
+        absmax_ref = ta.reconstruct_absmax(absmax_dev).cpu()
+    y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None if b is None else b.to(DEV), absmax_dev, lut.to(DEV), blocksize,
+                      torch.bfloat16, (N, K))
+    ref = oracle.matmul_4bit_f64(x, qw, b, absmax_ref, lut, blocksize, torch.bfloat16, (N, K))
+    assert y.shape == ref.shape and y.dtype == torch.bfloat16
+    torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
+    return y, ref
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 15, 16])
+def test_gemv_rows(ta, oracle, M):
+    _sync_print(f"gemv M={M}")
+    assert ta.functional.fused_route(torch.empty(M, 1024, dtype=torch.bfloat16), None, 64, torch.bfloat16, (256, 1024)) == "gemv"
+    _matmul_case(ta, oracle, M, 256, 1024, seed=M)
+
+
+@pytest.mark.parametrize(
+    "N,K",
+    [(16, 512), (48, 512), (100, 1024), (130, 2048), (1024, 4096), (4096, 4096), (1000, 14336), (2048 + 16, 8192)],
+)
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_gemv_shapes(ta, oracle, N, K, M):
+    _sync_print(f"gemv N={N} K={K} M={M}")
+    _matmul_case(ta, oracle, M, N, K, seed=N + K + M)
+
+
+@pytest.mark.parametrize("blocksize", [128, 512, 4096])
+def test_gemv_blocksizes(ta, oracle, blocksize):
+    _sync_print(f"gemv blocksize={blocksize}")
+    _matmul_case(ta, oracle, 3, 272, 4096, blocksize=blocksize, seed=blocksize)
+
+
+def test_gemv_bias_and_batch_dims(ta, oracle):
+    _sync_print("gemv bias / leading dims")
+    y, _ = _matmul_case(ta, oracle, 6, 320, 1024, bias=True, seed=5, x_shape=(2, 3, 1024))
+    assert y.shape == (2, 3, 320)
+
+
+@pytest.mark.parametrize("M", [1, 16])
+def test_gemv_nested(ta, oracle, M):
+    _sync_print(f"gemv nested M={M}")
+    _matmul_case(ta, oracle, M, 1024, 8192, nested=True, seed=70 + M)
+
+
+def test_gemv_repeatable_and_workspace_reuse(ta, oracle):
+    """Split-K partial sums are added in a fixed order: repeated calls are bit-identical, and calls
+    of different shapes can share the workspace back to back."""
+    _sync_print("gemv repeatability")
+    outs = []
+    for it in range(3):
+        y, _ = _matmul_case(ta, oracle, 4, 1024, 4096, seed=42)
+        outs.append(y.cpu())
+        _matmul_case(ta, oracle, 16, 512, 2048, seed=43)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize(
+    "M,N,K",
+    [(17, 128, 64), (32, 130, 128), (128, 128, 512), (100, 100, 1344), (300, 384, 1024), (512, 1024, 4096), (257, 4096, 1024)],
+)
+def test_gemm_shapes(ta, oracle, M, N, K):
+    _sync_print(f"gemm M={M} N={N} K={K}")
+    assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, 64, torch.bfloat16, (N, K)) == "gemm"
+    _matmul_case(ta, oracle, M, N, K, seed=M + N + K)
+
+
+def test_gemm_recovers_dequantized_weight_bit_exact(ta, oracle):
+    """x = identity makes every output a single product 1.0 * w: the fused kernel's in-LDS
+    dequantisation must equal nf4hip_dequantize bit for bit."""
+    _sync_print("gemm identity")
+    N, K = 256, 512
+    w = _weights((N, K), seed=9)
+    qw, absmax = oracle.C().quantize(w, 64)
+    x = torch.eye(K, dtype=torch.bfloat16)
+    y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None, absmax.to(DEV), ta.nf4_code(DEV), 64, torch.bfloat16, (N, K))
+    deq = oracle.C().dequantize(qw, absmax, oracle.nf4_lut(), 64, torch.bfloat16, (N, K))
+    assert torch.equal(y.cpu().t().contiguous().view(torch.int16), deq.view(torch.int16))
+
+
+def test_gemm_bias_nested_blocksize(ta, oracle):
+    _sync_print("gemm bias/nested/blocksize")
+    _matmul_case(ta, oracle, 64, 256, 1024, bias=True, seed=1)
+    _matmul_case(ta, oracle, 64, 256, 1024, nested=True, seed=2)
+    _matmul_case(ta, oracle, 64, 256, 1024, blocksize=256, seed=3)
+
+
+@pytest.mark.parametrize("case", ["fp32", "fp16", "K_not_64", "n_lt_block"])
+def test_fallback_route(ta, oracle, case):
+    """Shapes/dtypes outside the fused kernels take HIP dequantize + dense matmul, as
+    bitsandbytes.matmul_4bit does."""
+    _sync_print(f"fallback {case}")
+    dtype = {"fp32": torch.float32, "fp16": torch.float16}.get(case, torch.bfloat16)
+    N, K = {"K_not_64": (64, 1376), "n_lt_block": (2, 2)}.get(case, (96, 256))
+    w = _weights((N, K), seed=5, dtype=dtype)
+    x = _acts((3, K), seed=6, dtype=dtype)
+    b = _acts((N,), seed=7, dtype=dtype)
+    qw, absmax = oracle.C().quantize(w, 64)
+    assert ta.functional.fused_route(x, b, 64, dtype, (N, K)) == "dequant+linear"
+    y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), b.to(DEV), absmax.to(DEV), ta.nf4_code(DEV), 64, dtype, (N, K))
+    ref = oracle.matmul_4bit_f64(x, qw, b, absmax, oracle.nf4_lut(), 64, dtype, (N, K))
+    torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_full_size_properties(ta):
+    """Llama-3-8B FFN shape at full size through size-independent properties: quantize is
+    idempotent on its own dequantisation, and gemv is linear in x."""
+    _sync_print("full size properties")
+    N, K = 14336, 4096
+    g = torch.Generator(device=DEV).manual_seed(1)
+    w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    qw, absmax, code = ta.quantize_nf4(w)
+    deq = ta.dequantize_nf4(qw, absmax, code, 64, torch.bfloat16, (N, K))
+    qw2, absmax2, _ = ta.quantize_nf4(deq)
+    deq2 = ta.dequantize_nf4(qw2, absmax2, code, 64, torch.bfloat16, (N, K))
+    assert torch.equal(deq.view(torch.int16), deq2.view(torch.int16))
+    x1 = torch.randn(1, K, generator=g, device=DEV).to(torch.bfloat16)
+    x2 = torch.randn(1, K, generator=g, device=DEV).to(torch.bfloat16)
+    y1 = ta.matmul_nf4(x1, qw, None, absmax, code, 64, torch.bfloat16, (N, K)).float()
+    y2 = ta.matmul_nf4(x2, qw, None, absmax, code, 64, torch.bfloat16, (N, K)).float()
+    y12 = ta.matmul_nf4(torch.cat([x1, x2]), qw, None, absmax, code, 64, torch.bfloat16, (N, K)).float()
+    torch.testing.assert_close(y12[0], y1[0], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(y12[1], y2[0], rtol=2e-2, atol=2e-2)
+    ref = (x1.float() @ deq.float().t())
+    torch.testing.assert_close(y1, ref, rtol=2e-2, atol=2e-2)
+    big = ta.matmul_nf4(torch.cat([x1, x2]).repeat(128, 1), qw, None, absmax, code, 64, torch.bfloat16, (N, K)).float()
+    torch.testing.assert_close(big[0], ref[0], rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(big[254], ref[0], rtol=2e-2, atol=2e-2)

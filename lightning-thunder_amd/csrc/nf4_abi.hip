@@ -67,11 +67,14 @@ int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const 
     if (N > INT32_MAX || K > INT32_MAX || M > INT32_MAX) return fail(NF4HIP_E_SHAPE, "%s: dimension too large", name);
     if (kind == GEMV) {
         if (M > 16) return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: M = %lld > 16", (long long)M);
-        if (K % 512) return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: K = %lld is not a multiple of 512", (long long)K);
+        if (M <= 4 ? K % 32 : K % 512)
+            return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: K = %lld is not a multiple of %d (M = %lld)", (long long)K,
+                        M <= 4 ? 32 : 512, (long long)M);
     } else {
         if (K % 64) return fail(NF4HIP_E_SHAPE, "nf4hip_gemm: K = %lld is not a multiple of 64", (long long)K);
     }
-    if (K % blocksize) return fail(NF4HIP_E_SHAPE, "%s: blocksize %d does not divide K = %lld", name, blocksize, (long long)K);
+    if (!(kind == GEMV && M <= 4) && K % blocksize)
+        return fail(NF4HIP_E_SHAPE, "%s: blocksize %d does not divide K = %lld", name, blocksize, (long long)K);
     if (!aligned16(x) || !aligned16(packed) || !aligned16(out) || (absmax && !aligned16(absmax)) ||
         (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
         return fail(NF4HIP_E_ALIGN, "%s: pointer not 16-byte aligned", name);

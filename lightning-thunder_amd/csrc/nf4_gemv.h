@@ -1,0 +1,81 @@
+// Pieces shared by the two decode-shape kernels (row-streaming for M <= 4, MFMA tiles for M <= 16).
+#pragma once
+
+#include "nf4_common.h"
+
+namespace nf4 {
+
+constexpr int GEMV_THREADS = 512;  // 8 waves; two workgroups per CU
+constexpr int GEMV_WAVES = GEMV_THREADS / 64;
+constexpr int GEMV_TABLE_BYTES = 256 * 256;     // 256 byte values x 64 lanes x 4 B
+constexpr int GEMV_COUNTER_BYTES = 4096 * 4;    // split-K arrival counters at the head of the workspace
+
+// Byte -> (bf16, bf16) table at the start of LDS.  Entry b holds the code values of the two
+// nibbles of b as bf16, the high nibble (even element) in the low half.  It is replicated for the
+// 64 lanes with a 256-byte stride: lane l reads byte address (b << 8) | (l * 4), so every lane
+// owns one bank column and a lookup is conflict-free whatever the data.
+// `lut_lane` is lut16[lane & 15], loaded by the caller (early, so that its latency is hidden).
+__device__ __forceinline__ void build_pair_table(uint8_t* smem, float lut_lane, int lane, int wave) {
+    const uint32_t lb = f32_to_bf16_bits(lut_lane);
+    uint32_t* table = reinterpret_cast<uint32_t*>(smem);
+#pragma unroll 8
+    for (int it = 0; it < 32; ++it) {
+        const int e = wave * 32 + it;
+        const uint32_t first = __builtin_amdgcn_readlane(lb, e >> 4);   // high nibble = even element
+        const uint32_t second = __builtin_amdgcn_readlane(lb, e & 15);  // low nibble = odd element
+        table[e * 64 + lane] = first | (second << 16);
+    }
+}
+
+// fp32 variant of the table for the exact kernels: entry b = (lut[b >> 4], lut[b & 15]) as two
+// floats, replicated for 32 lane columns with a 256-byte stride; lane l reads byte address
+// (b << 8) | ((l & 31) * 8).
+__device__ __forceinline__ void build_pair_table_f32(uint8_t* smem, float lut_lane, int lane, int wave) {
+    const uint32_t lb = __float_as_uint(lut_lane);
+    float2* table = reinterpret_cast<float2*>(smem);
+    const int half = lane >> 5;
+#pragma unroll 8
+    for (int it = 0; it < 16; ++it) {
+        const int e0 = wave * 32 + 2 * it;  // lanes 0-31 write entry e0, lanes 32-63 entry e0 + 1
+        const uint32_t first = __builtin_amdgcn_readlane(lb, e0 >> 4);
+        const uint32_t s0 = __builtin_amdgcn_readlane(lb, e0 & 15);
+        const uint32_t s1 = __builtin_amdgcn_readlane(lb, (e0 & 15) + 1);
+        table[(e0 + half) * 32 + (lane & 31)] = make_float2(__uint_as_float(first), __uint_as_float(half ? s1 : s0));
+    }
+}
+
+// K beyond which the decode kernels reproduce the reference's per-weight bf16 rounding exactly.
+__host__ __device__ constexpr bool gemv_wants_exact(int64_t K) { return K > 16384; }
+
+// Read one table entry.  `addr` is an absolute LDS byte address: the table sits at LDS offset 0
+// (the gemv kernels have no static __shared__ data, so their dynamic segment starts there), which
+// saves the "+ base" VALU add the compiler emits for every access through an extern __shared__
+// array.
+__device__ __forceinline__ uint32_t lds_table_read(uint32_t addr) {
+    typedef __attribute__((address_space(3))) const uint32_t* lds_u32_ptr;
+    return *reinterpret_cast<lds_u32_ptr>((uintptr_t)addr);
+}
+
+__device__ __forceinline__ float2 lds_table_read2(uint32_t addr) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) const f32x2_t* lds_f2_ptr;
+    const f32x2_t v = *reinterpret_cast<lds_f2_ptr>((uintptr_t)addr);
+    return make_float2(v.x, v.y);
+}
+
+template <typename K>
+hipError_t gemv_allow_lds(K kern, int bytes) {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+// row-streaming kernel, 1 <= M <= 4 (nf4_gemv_rows.hip)
+size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K);
+hipError_t gemv_rows_setup();
+hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream);
+
+// MFMA tile kernel, 5 <= M <= 16 (nf4_gemv.hip)
+size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K);
+hipError_t gemv_tiles_setup();
+hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream);
+
+}  // namespace nf4

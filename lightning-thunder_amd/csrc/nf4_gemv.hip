@@ -1,4 +1,5 @@
-// Decode-shape fused NF4 dequant-matmul for gfx950, 1 <= M <= 16 rows of x.
+// Decode-shape fused NF4 dequant-matmul for gfx950, 5 <= M <= 16 rows of x (MFMA tiles), and the
+// dispatch between it and the row-streaming kernel that serves M <= 4.
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -27,7 +28,7 @@
 //  * K split.  When N alone cannot fill the chip, K is split over workgroups; partial sums go to a
 //    workspace and the last workgroup to finish a row group (device-scope counter) adds them in a
 //    fixed order, so the result does not depend on scheduling.
-#include "nf4_common.h"
+#include "nf4_gemv.h"
 
 namespace nf4 {
 namespace {
@@ -35,13 +36,13 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-constexpr int THREADS = 512;                // 8 waves
-constexpr int WAVES = THREADS / 64;
-constexpr int TABLE_BYTES = 256 * 256;      // 256 entries x 64 lanes x 4 B
+constexpr int THREADS = GEMV_THREADS;
+constexpr int WAVES = GEMV_WAVES;
+constexpr int TABLE_BYTES = GEMV_TABLE_BYTES;
 constexpr int PHASE_K = 512;                // k per phase (two steps of 256)
 constexpr int XOPS_BYTES = 16 * PHASE_K * 2;  // x operands of one phase, 16 rows
 constexpr int SMEM_BYTES = TABLE_BYTES + XOPS_BYTES;
-constexpr int COUNTER_BYTES = 4096 * 4;     // up to 4096 row groups
+constexpr int COUNTER_BYTES = GEMV_COUNTER_BYTES;
 
 struct Plan {
     int tiles;        // ceil(N / 16)
@@ -150,7 +151,7 @@ __device__ __forceinline__ void compute_phase(const MatmulArgs& a, const PhaseRe
                 for (int j = 0; j < 4; ++j) {
                     // LDS byte address = (byte j of d[aa]) << 8 | lane*4
                     const uint32_t addr = __builtin_amdgcn_perm(d[aa], lane4, 0x0c0c0400u | ((uint32_t)j << 8));
-                    p[j] = *reinterpret_cast<const uint32_t*>(smem + addr);
+                    p[j] = lds_table_read(addr);
                 }
                 const uint4 xa = xops[((s * 2 + c) * 4 + aa) * 64 + lane];
                 const uint4 wb = make_uint4(p[0], p[1], p[2], p[3]);
@@ -173,26 +174,16 @@ __device__ __forceinline__ void compute_phase(const MatmulArgs& a, const PhaseRe
 template <bool B64, bool NESTED>
 __global__ __launch_bounds__(THREADS, 4) void gemv_kernel(MatmulArgs a, Plan p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    // One word of the x-operand buffer doubles as the "last workgroup" flag: it is only written after
-    // the barrier that follows the last compute of a task, and slot 0 (row 0) is rewritten by the
-    // next phase anyway.
-    volatile int* last_flag = reinterpret_cast<volatile int*>(smem + TABLE_BYTES);
+    // The first word of the x-operand buffer doubles as the "last workgroup" flag of the split-K
+    // epilogue: it is only written after the barrier that follows the last compute of a task, and
+    // slot 0 (row 0 of x) is rewritten by the next phase anyway.
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, g = lane >> 4;
 
-    // ---- byte -> (bf16, bf16) table, replicated per lane ----
+    build_pair_table(smem, a.lut16[lane & 15], lane, wave);
     {
-        const uint32_t lb = f32_to_bf16_bits(a.lut16[lane & 15]);
-        uint32_t* table = reinterpret_cast<uint32_t*>(smem);
-#pragma unroll 8
-        for (int it = 0; it < 32; ++it) {
-            const int e = wave * 32 + it;
-            const uint32_t first = __builtin_amdgcn_readlane(lb, e >> 4);   // high nibble = even element
-            const uint32_t second = __builtin_amdgcn_readlane(lb, e & 15);  // low nibble = odd element
-            table[e * 64 + lane] = first | (second << 16);
-        }
         uint4* xops = reinterpret_cast<uint4*>(smem + TABLE_BYTES);
         xops[tid] = make_uint4(0, 0, 0, 0);
         xops[tid + THREADS] = make_uint4(0, 0, 0, 0);
@@ -244,24 +235,30 @@ __global__ __launch_bounds__(THREADS, 4) void gemv_kernel(MatmulArgs a, Plan p) 
                 }
             }
         } else {
+            // Partial sums cross workgroups (and XCDs, whose L2s are not coherent with each other)
+            // through agent-scope relaxed atomics only: such stores write through and such loads
+            // bypass stale lines, so no L2-wide write-back/invalidate fence is needed.  Ordering:
+            // every store has completed (s_waitcnt) before the workgroup bumps the counter.
             if (n < a.N) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int m = 4 * g + q;
-                    if (m < a.M) partial[((int64_t)ks * a.M + m) * a.N + n] = acc[q];
+                    if (m < a.M)
+                        __hip_atomic_store(&partial[((int64_t)ks * a.M + m) * a.N + n], acc[q], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-            __threadfence();
+            __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
+            int* flag = reinterpret_cast<int*>(smem + TABLE_BYTES);
             if (tid == 0) {
                 const unsigned prev =
-                    __hip_atomic_fetch_add(&counters[tg], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-                *last_flag = (prev == (unsigned)p.splits - 1u);
+                    __hip_atomic_fetch_add(&counters[tg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *flag = (prev == (unsigned)p.splits - 1u);
             }
             __syncthreads();
-            const bool is_last = *last_flag != 0;
+            const bool is_last = *flag != 0;
             if (is_last) {
-                __threadfence();
                 const int rows = min(WAVES * 16, a.N - tg * WAVES * 16);
                 for (int idx = tid; idx < rows * a.M; idx += THREADS) {
                     const int m = idx / rows;
@@ -279,35 +276,6 @@ __global__ __launch_bounds__(THREADS, 4) void gemv_kernel(MatmulArgs a, Plan p) 
     }
 }
 
-constexpr int MAX_DEVICES = 64;
-int g_num_cus[MAX_DEVICES] = {};  // 0 = not queried yet; set once per device (benign if set twice)
-
-template <typename K>
-hipError_t allow_big_lds(K kern) {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               SMEM_BYTES);
-}
-
-// CU count of the current device; on first use on a device also raises the kernels' LDS limit.
-hipError_t device_setup(int* cus_out) {
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
-    if (!g_num_cus[dev]) {
-        int cus = 0;
-        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        if (e != hipSuccess) return e;
-        if ((e = allow_big_lds(gemv_kernel<false, false>)) != hipSuccess) return e;
-        if ((e = allow_big_lds(gemv_kernel<true, false>)) != hipSuccess) return e;
-        if ((e = allow_big_lds(gemv_kernel<false, true>)) != hipSuccess) return e;
-        if ((e = allow_big_lds(gemv_kernel<true, true>)) != hipSuccess) return e;
-        g_num_cus[dev] = cus > 0 ? cus : 256;
-    }
-    *cus_out = g_num_cus[dev];
-    return hipSuccess;
-}
-
 // Work split.  `slots` = workgroups resident at once (two per CU).
 Plan make_plan(int64_t N, int64_t K, int slots) {
     Plan p;
@@ -323,11 +291,32 @@ Plan make_plan(int64_t N, int64_t K, int slots) {
     return p;
 }
 
+constexpr int MAX_DEVICES = 64;
+int g_num_cus[MAX_DEVICES] = {};  // 0 = not set up yet; set once per device (benign if set twice)
+
+// CU count of the current device; on first use on a device also raises the kernels' LDS limit.
+hipError_t device_setup(int* cus_out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    if (!g_num_cus[dev]) {
+        int cus = 0;
+        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return e;
+        if ((e = gemv_tiles_setup()) != hipSuccess) return e;
+        if ((e = gemv_rows_setup()) != hipSuccess) return e;
+        g_num_cus[dev] = cus > 0 ? cus : 256;
+    }
+    *cus_out = g_num_cus[dev];
+    return hipSuccess;
+}
+
 }  // namespace
 
-size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || K % PHASE_K) return COUNTER_BYTES;
-    // the largest split any device-dependent plan can choose is K / PHASE_K
+    // the largest split any device-dependent plan can choose is bounded by the slot count
     const int64_t max_splits = K / PHASE_K;
     const int64_t tile_groups = ((N + 15) / 16 + WAVES - 1) / WAVES;
     int64_t splits = 1;
@@ -336,10 +325,15 @@ size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return (size_t)COUNTER_BYTES + (splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0);
 }
 
-hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
-    int cus = 0;
-    hipError_t e = device_setup(&cus);
-    if (e != hipSuccess) return e;
+hipError_t gemv_tiles_setup() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_kernel<false, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_kernel<true, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_kernel<false, true>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_kernel<true, true>, SMEM_BYTES);
+}
+
+hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
     const int slots = 2 * cus;
     Plan p = make_plan(a.N, a.K, slots);
     if (p.tile_groups > COUNTER_BYTES / 4 && p.splits > 1) p.splits = 1, p.phases = a.K / PHASE_K, p.ntasks = p.tile_groups;
@@ -350,6 +344,19 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
                     : (nested ? gemv_kernel<false, true> : gemv_kernel<false, false>);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
+}
+
+// ---- dispatch -------------------------------------------------------------------------------
+
+size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    return M <= 4 ? gemv_rows_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
+}
+
+hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
+    int cus = 0;
+    const hipError_t e = device_setup(&cus);
+    if (e != hipSuccess) return e;
+    return a.M <= 4 ? launch_gemv_rows(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
 }
 
 }  // namespace nf4

@@ -1,0 +1,386 @@
+// Decode-shape fused NF4 dequant-matmul for gfx950, 1 <= M <= 4 rows of x: the GEMV proper.
+//
+// Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
+// bitsandbytes.matmul_4bit picks for a single-row x; call site
+// thunder/transforms/quantization.py:39.
+//
+// HBM-bound: 0.5 byte of codes + 4/blocksize bytes of absmax per weight, each read exactly once.
+//
+//  * Weight stream.  A wave reads one weight row at a time, 1 KB per load instruction: lane l takes
+//    the 16 bytes (32 codes) at k = chunk*2048 + 32*l.  Consecutive lanes read consecutive bytes, so
+//    every load is a fully coalesced 1 KB burst; U rows are kept in flight per wave.
+//  * x stays in registers.  A wave works on one 2048-wide k chunk for all its rows, so each lane
+//    keeps its 32 x values (16 dwords of bf16 pairs) per row of x for the whole task.
+//  * Code -> bf16.  A 256-entry LDS table indexed by a whole packed BYTE returns both bf16 code
+//    values of that byte as one dword (even element in the low half).  The table is replicated for
+//    all 64 lanes with a 256-byte stride, so the LDS address is (byte << 8) | (lane * 4): one
+//    v_perm_b32 per byte and no bank conflicts.
+//  * Multiply-accumulate on the matrix pipe.  v_mfma_f32_4x4x4_16b_bf16 computes 16 independent
+//    4x4x4 products, one per group of 4 lanes.  Lane i of a group supplies row i of A (4 of its own
+//    weights) and column i of B (the 4 matching x values), so the DIAGONAL element C[i][i] is lane
+//    i's own dot product; the off-diagonal 3/4 of the result is discarded.  Eight such MFMAs cover
+//    a lane's 32 weights and leave the VALU with the table addressing only.
+//  * Scale.  The 32 weights of a lane share one quantisation block, so absmax multiplies the lane's
+//    partial sum once.  This differs from the reference's dequantise-then-multiply only in where the
+//    bf16 rounding happens; the difference grows like sqrt(K), so for K > 16384 an exact variant
+//    rounds every weight as bf16(lut * absmax) before the MFMA (fp32 table, two multiplies and one
+//    convert per byte more).
+//  * Reduction.  Per-lane partial sums of 8 (row, m) pairs are reduced together by a transposing
+//    butterfly (DPP for the four in-row levels, ds_bpermute for the two cross-row levels); the
+//    result of (row, chunk, m) is parked in LDS, and after the band is done the chunks are added in
+//    a fixed order.
+//  * K > 16384 is split over two or more workgroups; partial sums cross workgroups through
+//    agent-scope relaxed atomics and a counter (no L2-wide fences), added in a fixed order by the
+//    last workgroup to arrive.
+#include "nf4_gemv.h"
+
+namespace nf4 {
+namespace {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int PART_BYTES = 16 * 1024;  // per-(row, chunk, m) partial sums of one band
+constexpr int SMEM_BYTES = GEMV_TABLE_BYTES + PART_BYTES;
+constexpr int CHUNK_K = 2048;          // k covered by one wave-wide 16-byte load
+constexpr int FLAG_OFFSET = GEMV_TABLE_BYTES + PART_BYTES - 16;
+
+struct RowsPlan {
+    int chunks;         // k chunks handled by one workgroup (waves along K)
+    int row_lanes;      // rows processed concurrently by one workgroup = 8 / chunks
+    int splits;         // K splits across workgroups
+    int rows_per_band;  // rows of one task
+    int nbands;
+    int ntasks;         // nbands * splits
+    int aligned;        // K % blocksize == 0: the block index splits into a row part and a k part
+};
+
+#define NF4_DPP(v, ctrl) \
+    __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
+
+// v[0..7] hold per-lane partial sums of 8 independent quantities.  Returns, in every lane, the
+// 64-lane total of quantity id(lane) = 4 * ((lane >> 2) & 1) ... see `reduce8_id`.
+// Stage A/B/C halve the number of registers by letting lane bit 0/1/2 choose which quantity the
+// lane keeps (the partner lane sends its share of it); the remaining three levels are plain sums.
+__device__ __forceinline__ float reduce8(const float v[8], int lane) {
+    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
+    float w[4], z[2];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const float keep = b0 ? v[2 * p + 1] : v[2 * p];
+        const float send = b0 ? v[2 * p] : v[2 * p + 1];
+        w[p] = keep + NF4_DPP(send, 0xB1);  // quad_perm [1,0,3,2]: lane ^ 1
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const float keep = b1 ? w[2 * p + 1] : w[2 * p];
+        const float send = b1 ? w[2 * p] : w[2 * p + 1];
+        z[p] = keep + NF4_DPP(send, 0x4E);  // quad_perm [2,3,0,1]: lane ^ 2
+    }
+    const float keep = b2 ? z[1] : z[0];
+    const float send = b2 ? z[0] : z[1];
+    // lane ^ 4 inside a row of 16: shift by 4 in the direction that stays inside the group of 8
+    float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x104 /*row_shl:4*/, 0xf, 0x5, false));
+    other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, other), __builtin_bit_cast(int, send), 0x114 /*row_shr:4*/, 0xf, 0xa, false));
+    float y = keep + other;
+    y += NF4_DPP(y, 0x128);  // row_ror:8: lane ^ 8
+    y += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, y)));
+    y += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, y)));
+    return y;
+}
+// quantity whose total `reduce8` leaves in `lane`: bit 0 of the lane picks v[odd], bit 1 the second
+// pair, bit 2 the second half
+__device__ __forceinline__ int reduce8_id(int lane) { return (lane & 1) | ((lane & 2) ? 2 : 0) | ((lane & 4) ? 4 : 0); }
+
+// EXACT = false: the table holds bf16(lut) pairs and absmax scales the 32-weight partial sum.
+// EXACT = true : the table holds fp32 lut pairs and every weight is rounded like the reference's
+//                dequantisation, bf16(lut * absmax), before it is multiplied (more VALU work).
+template <int M, int U, bool NESTED, bool EXACT>
+__global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a, RowsPlan p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lane4 = (uint32_t)lane * 4u;
+    const uint32_t lane8 = (uint32_t)(lane & 31) * 8u;
+
+    // the code-book entry this lane contributes to the LDS table: requested first, used last
+    const float lut_mine = a.lut16[lane & 15];
+    bool table_built = false;
+
+    float* part = reinterpret_cast<float*>(smem + GEMV_TABLE_BYTES);
+    int* flag = reinterpret_cast<int*>(smem + FLAG_OFFSET);
+    unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
+
+    const int cw = wave % p.chunks;   // this wave's chunk inside the workgroup's K range
+    const int rl = wave / p.chunks;   // this wave's row lane
+    const int64_t K = a.K;
+    const int step = p.row_lanes;
+
+    for (int task = blockIdx.x; task < p.ntasks; task += gridDim.x) {
+        const int band = task / p.splits;
+        const int ks = task - band * p.splits;
+        const int r_begin = band * p.rows_per_band;
+        const int r_end = min(a.N, r_begin + p.rows_per_band);
+        const int64_t kchunk = (int64_t)(ks * p.chunks + cw) * CHUNK_K;
+        const uint32_t klane = 32u * (uint32_t)lane;
+        const bool wave_on = rl < p.row_lanes && kchunk < K && r_begin + rl < r_end;
+        const bool lane_on = wave_on && kchunk + klane < K;
+        const int cnt = wave_on ? (r_end - r_begin - rl + step - 1) / step : 0;  // rows of this wave
+
+        // x for this lane's 32 k, all M rows
+        uint32_t xr[M][16];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (lane_on) v = *reinterpret_cast<const uint4*>(a.x + m * K + kchunk + klane + 8 * q);
+                xr[m][4 * q + 0] = v.x; xr[m][4 * q + 1] = v.y; xr[m][4 * q + 2] = v.z; xr[m][4 * q + 3] = v.w;
+            }
+
+        uint4 wq[U];
+        float sq[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            wq[u] = make_uint4(0, 0, 0, 0);
+            sq[u] = 0.0f;
+        }
+        // row i of this wave is r_begin + rl + i * step
+        auto issue = [&](int u, int i) {
+                const int row = r_begin + rl + i * step;
+                if (lane_on) {
+                    const uint8_t* rowp = a.packed + (((int64_t)row * K + kchunk) >> 1);  // uniform
+                    wq[u] = load16_stream(rowp + (klane >> 1));
+                    int64_t blk;
+                    if (p.aligned)
+                        blk = (((int64_t)row * K + kchunk) >> a.block_log2) + (klane >> a.block_log2);
+                    else
+                        blk = ((int64_t)row * K + kchunk + klane) >> a.block_log2;
+                    sq[u] = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
+                }
+            };
+        // get the weight stream going before anything else happens
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < cnt) issue(u, u);
+
+        if (!table_built) {  // first task only: overlaps with the loads above
+            if (EXACT)
+                build_pair_table_f32(smem, lut_mine, lane, wave);
+            else
+                build_pair_table(smem, lut_mine, lane, wave);
+            table_built = true;
+        }
+        __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
+
+        if (cnt > 0) {
+            for (int i0 = 0; i0 < cnt; i0 += U) {
+                float res[U * M];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t d[4] = {wq[u].x, wq[u].y, wq[u].z, wq[u].w};
+                    const float s = sq[u];
+                    if (i0 + u + U < cnt) {
+                        issue(u, i0 + u + U);
+                    } else {  // slot is dead from here on; say so, or the compiler keeps copies alive
+                        wq[u] = make_uint4(0, 0, 0, 0);
+                        sq[u] = 0.0f;
+                    }
+                    uint32_t pr[16];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const uint32_t sel = 0x0c0c0400u | ((uint32_t)j << 8);
+                            if (EXACT) {
+                                // bf16(lut[c] * absmax) per weight, the value nf4hip_dequantize produces
+                                const float2 v = lds_table_read2(__builtin_amdgcn_perm(d[q], lane8, sel));
+                                f32x2 f = {__fmul_rn(v.x, s), __fmul_rn(v.y, s)};
+                                pr[4 * q + j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+                            } else {
+                                pr[4 * q + j] = lds_table_read(__builtin_amdgcn_perm(d[q], lane4, sel));
+                            }
+                        }
+#pragma unroll
+                    for (int m = 0; m < M; ++m) {
+                        f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            const uint2 wa = make_uint2(pr[2 * t], pr[2 * t + 1]);
+                            const uint2 xb = make_uint2(xr[m][2 * t], xr[m][2 * t + 1]);
+                            c = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
+                                                                       __builtin_bit_cast(s16x4, xb), c, 0, 0, 0);
+                        }
+                        // diagonal element of this lane's 4x4 block
+                        const float c01 = (lane & 1) ? c[1] : c[0];
+                        const float c23 = (lane & 1) ? c[3] : c[2];
+                        const float diag = (lane & 2) ? c23 : c01;
+                        res[u * M + m] = EXACT ? diag : diag * s;
+                    }
+                }
+                // reduce the U*M per-lane results over the wave, 8 at a time
+#pragma unroll
+                for (int g8 = 0; g8 < (U * M + 7) / 8; ++g8) {
+                    float v8[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v8[e] = (g8 * 8 + e < U * M) ? res[g8 * 8 + e] : 0.0f;
+                    const float total = reduce8(v8, lane);
+                    const int id = g8 * 8 + reduce8_id(lane);  // = u * M + m
+                    const int u = id / M, m = id - u * M;
+                    const int i = i0 + u;
+                    if (lane < 8 && id < U * M && i < cnt)
+                        part[((rl + i * step) * p.chunks + cw) * M + m] = total;
+                }
+            }
+        }
+        __syncthreads();
+
+        // ---- band epilogue: add the chunks of every row in a fixed order ----
+        const int nrows = r_end - r_begin;
+        // the last split may own fewer chunks than the others
+        const int nchunks = min(p.chunks, (int)((K + CHUNK_K - 1) / CHUNK_K) - ks * p.chunks);
+        if (p.splits == 1) {
+            for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                const int r = idx / M, m = idx - r * M;
+                float sum = 0.0f;
+                for (int c = 0; c < nchunks; ++c) sum += part[(r * p.chunks + c) * M + m];
+                const int n = r_begin + r;
+                if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
+                a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
+            }
+        } else {
+            for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                const int r = idx / M, m = idx - r * M;
+                float sum = 0.0f;
+                for (int c = 0; c < nchunks; ++c) sum += part[(r * p.chunks + c) * M + m];
+                __hip_atomic_store(&partial[((int64_t)ks * M + m) * a.N + r_begin + r], sum, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned prev =
+                    __hip_atomic_fetch_add(&counters[band], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *flag = (prev == (unsigned)p.splits - 1u);
+            }
+            __syncthreads();
+            if (*flag != 0) {
+                for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                    const int r = idx / M, m = idx - r * M;
+                    const int n = r_begin + r;
+                    float sum = 0.0f;
+                    for (int k2 = 0; k2 < p.splits; ++k2)
+                        sum += __hip_atomic_load(&partial[((int64_t)k2 * M + m) * a.N + n], __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+                    if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
+                    a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
+                }
+                if (tid == 0) __hip_atomic_store(&counters[band], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+}
+
+int rows_splits(int64_t K) {
+    const int64_t nch = (K + CHUNK_K - 1) / CHUNK_K;
+    return (int)((nch + GEMV_WAVES - 1) / GEMV_WAVES);
+}
+
+RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots) {
+    RowsPlan p;
+    p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
+    const int nch = (int)((K + CHUNK_K - 1) / CHUNK_K);
+    p.splits = rows_splits(K);
+    p.chunks = (nch + p.splits - 1) / p.splits;
+    p.row_lanes = GEMV_WAVES / p.chunks;
+    const int cap = ((PART_BYTES - 64) / (p.chunks * M * 4)) / p.row_lanes * p.row_lanes;
+    int bands_target = slots / p.splits;
+    if (bands_target < 1) bands_target = 1;
+    int64_t rpb = (N + bands_target - 1) / bands_target;
+    rpb = (rpb + p.row_lanes - 1) / p.row_lanes * p.row_lanes;
+    if (rpb > cap) rpb = cap;
+    if (rpb < p.row_lanes) rpb = p.row_lanes;
+    p.rows_per_band = (int)rpb;
+    p.nbands = (int)((N + rpb - 1) / rpb);
+    p.ntasks = p.nbands * p.splits;
+    return p;
+}
+
+template <int M, int U, bool NESTED>
+hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
+    if (gemv_wants_exact(a.K))
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, true>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    else
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, false>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    return hipGetLastError();
+}
+
+// U = rows in flight per wave: as many as the wave has to do, within the register budget
+// (8 only for M = 1).
+template <int M, bool NESTED>
+hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
+    const int cnt = p.rows_per_band / p.row_lanes;  // rows per wave and task
+    if constexpr (M == 1)
+        if (cnt >= 8) return launch_u<1, 8, NESTED>(a, p, grid, stream);
+    if constexpr (M <= 2)
+        if (cnt >= 4) return launch_u<M, 4, NESTED>(a, p, grid, stream);
+    return launch_u<M, 2, NESTED>(a, p, grid, stream);
+}
+
+template <bool NESTED>
+hipError_t launch_n(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
+    switch (a.M) {
+        case 1: return launch_m<1, NESTED>(a, p, grid, stream);
+        case 2: return launch_m<2, NESTED>(a, p, grid, stream);
+        case 3: return launch_m<3, NESTED>(a, p, grid, stream);
+        default: return launch_m<4, NESTED>(a, p, grid, stream);
+    }
+}
+
+template <int M, int U>
+hipError_t allow_lds_mu() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, true, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, true>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_rows_kernel<M, U, true, true>, SMEM_BYTES);
+}
+
+template <int M>
+hipError_t allow_lds_m() {
+    if constexpr (M <= 2) {
+        const hipError_t e = allow_lds_mu<M, 4>();
+        if (e != hipSuccess) return e;
+    }
+    return allow_lds_mu<M, 2>();
+}
+
+}  // namespace
+
+size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int s = rows_splits(K);
+    return (size_t)GEMV_COUNTER_BYTES + (s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0);
+}
+
+hipError_t gemv_rows_setup() {
+    hipError_t e;
+    if ((e = allow_lds_mu<1, 8>()) != hipSuccess) return e;
+    if ((e = allow_lds_m<1>()) != hipSuccess) return e;
+    if ((e = allow_lds_m<2>()) != hipSuccess) return e;
+    if ((e = allow_lds_m<3>()) != hipSuccess) return e;
+    return allow_lds_m<4>();
+}
+
+hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {
+    int slots = 2 * cus;
+    if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
+    const RowsPlan p = make_rows_plan(a.M, a.N, a.K, a.block_log2, slots);
+    const int grid = p.ntasks < slots ? p.ntasks : slots;
+    return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
+}
+
+}  // namespace nf4

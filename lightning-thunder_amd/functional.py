@@ -22,6 +22,11 @@ from . import _lib
 
 SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
 
+# Beyond this K the decode kernels round every weight exactly like the reference's dequantisation
+# (the cheaper "scale the partial sum" arithmetic drifts from it like sqrt(K)); the 5..16-row tile
+# kernel has no such variant, so those calls go to the prefill kernel, which is exact by construction.
+EXACT_K = 16384
+
 _DTYPE_CODE = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32}
 
 # fp32 NF4 code values (QLoRA), index = 4-bit code; the table bitsandbytes stores as QuantState.code
@@ -222,13 +227,17 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         and (bias is None or bias.dtype == torch.bfloat16)
         and blocksize in SUPPORTED_BLOCKSIZES
         and M > 0
-        and K % 64 == 0
-        and K % blocksize == 0
+        and N > 0
+        and (N * K) % 2 == 0
     )
     if not fused:
         return "dequant+linear"
-    if M <= 16 and K % 512 == 0:
-        return "gemv"
+    if M <= 4 and K % 32 == 0:
+        return "gemv"  # row-streaming kernel: blocks may straddle rows
+    if K % 64 or K % blocksize:
+        return "dequant+linear"
+    if M <= 16 and K % 512 == 0 and K <= EXACT_K:
+        return "gemv"  # MFMA tile kernel
     return "gemm"
 
 

@@ -185,18 +185,30 @@ def test_gemv_rows(ta, oracle, M):
 
 @pytest.mark.parametrize(
     "N,K",
-    [(16, 512), (48, 512), (100, 1024), (130, 2048), (1024, 4096), (4096, 4096), (1000, 14336), (2048 + 16, 8192)],
+    [(16, 512), (48, 512), (100, 1024), (130, 2048), (1024, 4096), (4096, 4096), (1000, 14336), (2048 + 16, 8192),
+     (300, 28672), (77, 32768 + 512)],
 )
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 16])
 def test_gemv_shapes(ta, oracle, N, K, M):
     _sync_print(f"gemv N={N} K={K} M={M}")
     _matmul_case(ta, oracle, M, N, K, seed=N + K + M)
 
 
 @pytest.mark.parametrize("blocksize", [128, 512, 4096])
-def test_gemv_blocksizes(ta, oracle, blocksize):
-    _sync_print(f"gemv blocksize={blocksize}")
-    _matmul_case(ta, oracle, 3, 272, 4096, blocksize=blocksize, seed=blocksize)
+@pytest.mark.parametrize("M", [3, 7])
+def test_gemv_blocksizes(ta, oracle, blocksize, M):
+    _sync_print(f"gemv blocksize={blocksize} M={M}")
+    _matmul_case(ta, oracle, M, 272, 4096, blocksize=blocksize, seed=blocksize)
+
+
+@pytest.mark.parametrize("N,K", [(64, 1376), (2, 32), (33, 96), (5, 2048 + 32)])
+@pytest.mark.parametrize("M", [1, 4])
+def test_gemv_rows_odd_k(ta, oracle, N, K, M):
+    """The row-streaming kernel needs only K % 32 == 0: quantisation blocks may straddle rows
+    (K = 1376 is the intermediate size of the reference's own llama2-like test model)."""
+    _sync_print(f"gemv rows odd K N={N} K={K} M={M}")
+    assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, 64, torch.bfloat16, (N, K)) == "gemv"
+    _matmul_case(ta, oracle, M, N, K, seed=N + K)
 
 
 def test_gemv_bias_and_batch_dims(ta, oracle):
@@ -205,10 +217,28 @@ def test_gemv_bias_and_batch_dims(ta, oracle):
     assert y.shape == (2, 3, 320)
 
 
-@pytest.mark.parametrize("M", [1, 16])
+@pytest.mark.parametrize("M", [1, 4, 16])
 def test_gemv_nested(ta, oracle, M):
     _sync_print(f"gemv nested M={M}")
     _matmul_case(ta, oracle, M, 1024, 8192, nested=True, seed=70 + M)
+
+
+@pytest.mark.parametrize("M", [1, 4])
+def test_gemv_large_k_bit_matches_dequantize_then_matmul(ta, oracle, M):
+    """For K > 16384 the decode kernel rounds every weight as bf16(lut * absmax): with x = one-hot
+    rows the output must equal the dequantised weight column bit for bit."""
+    _sync_print(f"gemv exact M={M}")
+    N, K = 192, 16384 + 2048
+    w = _weights((N, K), seed=77)
+    qw, absmax = oracle.C().quantize(w, 64)
+    deq = oracle.C().dequantize(qw, absmax, oracle.nf4_lut(), 64, torch.bfloat16, (N, K))
+    x = torch.zeros(M, K, dtype=torch.bfloat16)
+    cols = [5, 4097, 16383 + 64, K - 1][:M]
+    for m, c in enumerate(cols):
+        x[m, c] = 1.0
+    y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None, absmax.to(DEV), ta.nf4_code(DEV), 64, torch.bfloat16, (N, K))
+    for m, c in enumerate(cols):
+        assert torch.equal(y[m].cpu().view(torch.int16), deq[:, c].contiguous().view(torch.int16))
 
 
 def test_gemv_repeatable_and_workspace_reuse(ta, oracle):
@@ -261,7 +291,7 @@ def test_fallback_route(ta, oracle, case):
     dtype = {"fp32": torch.float32, "fp16": torch.float16}.get(case, torch.bfloat16)
     N, K = {"K_not_64": (64, 1376), "n_lt_block": (2, 2)}.get(case, (96, 256))
     w = _weights((N, K), seed=5, dtype=dtype)
-    x = _acts((3, K), seed=6, dtype=dtype)
+    x = _acts((7, K), seed=6, dtype=dtype)
     b = _acts((N,), seed=7, dtype=dtype)
     qw, absmax = oracle.C().quantize(w, 64)
     assert ta.functional.fused_route(x, b, 64, dtype, (N, K)) == "dequant+linear"

@@ -1,0 +1,34 @@
+"""CPU stand-in for libnf4hip.so, for tests of the HOST logic only (executor registration, module
+surgery, state dicts, planning).  It swaps the three tensor-level ops for the oracle and lets the
+transform quantise on the CPU.  Nothing in the shipped package can reach this; a GPU run never
+uses it (the same tests run there against the real kernels)."""
+
+import contextlib
+
+import torch
+
+from oracle import nf4_oracle as O
+
+
+@contextlib.contextmanager
+def installed(ta):
+    F = ta.functional
+    Q = ta.transforms.quantization
+    saved = (F.quantize_nf4, F.dequantize_nf4, F.matmul_nf4, Q.WORK_DEVICE)
+
+    def quantize_nf4(w, blocksize=64):
+        qw, absmax = O.C().quantize(w, blocksize)
+        return qw, absmax, O.nf4_lut()
+
+    def dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape):
+        return O.C().dequantize(qweight, absmax, quant_map, blocksize, dtype, tuple(shape))
+
+    def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape):
+        assert len(shape) == 2 and x.shape[-1] == shape[1]
+        return O.matmul_4bit_eager(x, qweight, bias, absmax, quant_map, blocksize, dtype, tuple(shape))
+
+    F.quantize_nf4, F.dequantize_nf4, F.matmul_nf4, Q.WORK_DEVICE = quantize_nf4, dequantize_nf4, matmul_nf4, "cpu"
+    try:
+        yield
+    finally:
+        F.quantize_nf4, F.dequantize_nf4, F.matmul_nf4, Q.WORK_DEVICE = saved

@@ -1,0 +1,131 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol include/nf4hip.h declares, and
+every argument error is reported before any HIP call is made."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "nf4hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nf4hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(ta):
+    lib = ta._lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 13
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/nf4hip.h but not exported"
+    assert sorted(ta._lib.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
+    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 1
+
+
+def test_missing_library_fails_loudly(ta, tmp_path):
+    with pytest.raises(RuntimeError, match="not found"):
+        ta._lib.load(str(tmp_path / "libnf4hip.so"))
+
+
+def _err(ta):
+    return ta._lib.load().nf4hip_last_error().decode()
+
+
+A = 4096  # any non-null, 16-byte aligned fake device address: validation never dereferences
+
+
+def test_quantize_dequantize_argument_errors(ta):
+    L, lib = ta._lib, ta._lib.load()
+    assert lib.nf4hip_quantize(None, L.BF16, 128, 64, A, A, None) == L.E_NULL
+    assert lib.nf4hip_quantize(A, 7, 128, 64, A, A, None) == L.E_DTYPE
+    assert lib.nf4hip_quantize(A, L.BF16, 128, 48, A, A, None) == L.E_BLOCKSIZE
+    assert "48" in _err(ta)
+    assert lib.nf4hip_quantize(A, L.BF16, -1, 64, A, A, None) == L.E_SHAPE
+    assert lib.nf4hip_quantize(A + 2, L.BF16, 128, 64, A, A, None) == L.E_ALIGN
+    assert lib.nf4hip_quantize(None, L.BF16, 0, 64, None, None, None) == 0  # empty input is a no-op
+    assert lib.nf4hip_dequantize(A, A, None, 128, 64, A, L.BF16, None) == L.E_NULL
+    assert lib.nf4hip_dequantize(A, A, A, 128, 64, A, 3, None) == L.E_DTYPE
+    assert lib.nf4hip_dequantize(A, A, A, 128, 100, A, L.F16, None) == L.E_BLOCKSIZE
+    assert lib.nf4hip_dequantize(A, A, A, 128, 64, A + 8, L.F32, None) == L.E_ALIGN
+    assert lib.nf4hip_dequantize(None, None, None, 0, 64, None, L.BF16, None) == 0
+    assert lib.nf4hip_dequantize_dq(A, None, A, A, 0.0, 256, A, 128, 64, A, L.BF16, None) == L.E_NULL
+    assert lib.nf4hip_dequantize_dq(A, A, A, A, 0.0, 100, A, 128, 64, A, L.BF16, None) == L.E_BLOCKSIZE
+    assert lib.nf4hip_dq_compress(A, 10, 256, None, 0.0, A, A, None) == L.E_NULL
+    assert lib.nf4hip_dq_compress(A, -1, 256, A, 0.0, A, A, None) == L.E_SHAPE
+    assert lib.nf4hip_dq_reconstruct(A, A, A, 0.0, 10, 3, A, None) == L.E_BLOCKSIZE
+
+
+def test_matmul_argument_errors(ta):
+    L, lib = ta._lib, ta._lib.load()
+    ws = 1 << 30
+
+    def gemv(x=A, dt=L.BF16, M=1, packed=A, absmax=A, lut=A, bias=None, N=64, K=4096, bs=64, out=A, w=A, wb=ws):
+        return lib.nf4hip_gemv(x, dt, M, packed, absmax, lut, bias, N, K, bs, out, w, wb, None)
+
+    def gemm(x=A, dt=L.BF16, M=64, packed=A, absmax=A, lut=A, bias=None, N=64, K=4096, bs=64, out=A, w=None, wb=0):
+        return lib.nf4hip_gemm(x, dt, M, packed, absmax, lut, bias, N, K, bs, out, w, wb, None)
+
+    assert gemv(x=None) == L.E_NULL and gemv(absmax=None) == L.E_NULL and gemm(out=None) == L.E_NULL
+    assert gemv(dt=L.F16) == L.E_DTYPE and gemm(dt=L.F32) == L.E_DTYPE  # only bf16 x is fused
+    assert gemv(bs=96) == L.E_BLOCKSIZE
+    assert gemv(M=0) == L.E_SHAPE and gemv(M=17) == L.E_SHAPE and gemv(N=-5) == L.E_SHAPE
+    assert gemv(M=1, K=48) == L.E_SHAPE      # row-streaming kernel: K % 32
+    assert gemv(M=8, K=1376) == L.E_SHAPE    # tile kernel: K % 512
+    assert "512" in _err(ta)
+    assert gemm(K=100) == L.E_SHAPE and gemm(K=192, bs=128) == L.E_SHAPE
+    assert gemv(x=A + 4) == L.E_ALIGN and gemm(packed=A + 1) == L.E_ALIGN and gemv(bias=A + 1) == L.E_ALIGN
+    assert gemv(w=None) == L.E_WORKSPACE and gemv(wb=16) == L.E_WORKSPACE
+    assert "workspace" in _err(ta)
+    assert lib.nf4hip_gemv_dq(A, L.BF16, 1, A, None, A, A, 0.0, 256, A, None, 64, 4096, 64, A, A, ws, None) == L.E_NULL
+    assert lib.nf4hip_gemm_dq(A, L.BF16, 64, A, A, A, A, 0.0, 7, A, None, 64, 4096, 64, A, None, 0, None) == L.E_BLOCKSIZE
+    # workspace sizing is pure arithmetic
+    assert lib.nf4hip_gemv_workspace_bytes(1, 4096, 4096) == 16384
+    assert lib.nf4hip_gemv_workspace_bytes(4, 8192, 28672) == 16384 + 2 * 4 * 8192 * 4  # K split over 2 workgroups
+    assert lib.nf4hip_gemv_workspace_bytes(16, 1024, 4096) > 16384                        # tile kernel splits K
+    assert lib.nf4hip_gemm_workspace_bytes(2048, 4096, 4096) == 0
+
+
+def test_python_wrappers_refuse_cpu_tensors(ta):
+    import torch
+
+    w = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ta.quantize_nf4(w)
+    with pytest.raises(ValueError):
+        ta.quantize_nf4(w, blocksize=100)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ta.matmul_nf4(torch.zeros(1, 64, dtype=torch.bfloat16), torch.zeros(128, 1, dtype=torch.uint8), None,
+                      torch.zeros(4), ta.nf4_code(), 64, torch.bfloat16, (4, 64))
+
+
+def test_check_raises_with_message(ta):
+    lib = ta._lib.load()
+    rc = lib.nf4hip_quantize(A, 9, 1, 64, A, A, None)
+    with pytest.raises(ta._lib.NF4HipError, match="NF4HIP_E_DTYPE") as e:
+        ta._lib.check(rc)
+    assert e.value.code == ta._lib.E_DTYPE
+
+
+def test_fused_route_rules(ta):
+    import torch
+
+    F = ta.functional
+    bf = torch.bfloat16
+
+    def route(M, N, K, dtype=bf, xdtype=bf, bs=64, bias=None):
+        return F.fused_route(torch.empty(M, K, dtype=xdtype), bias, bs, dtype, (N, K))
+
+    assert route(1, 4096, 4096) == "gemv" and route(4, 64, 1376) == "gemv" and route(16, 4096, 4096) == "gemv"
+    assert route(5, 64, 1376) == "dequant+linear"        # tile kernel needs K % 512, gemm K % 64
+    assert route(8, 64, 1344) == "gemm" and route(17, 64, 4096) == "gemm" and route(2048, 4096, 4096) == "gemm"
+    assert route(16, 8192, 28672) == "gemm"              # K > 16384: exact weights wanted
+    assert route(1, 8192, 28672) == "gemv"               # row-streaming kernel has an exact variant
+    assert route(1, 64, 4096, dtype=torch.float32) == "dequant+linear"
+    assert route(1, 64, 4096, xdtype=torch.float16, dtype=torch.float16) == "dequant+linear"
+    assert route(1, 2, 2) == "dequant+linear"
+    assert route(1, 64, 4096, bias=torch.zeros(64)) == "dequant+linear"  # fp32 bias with bf16 x
+    _ = ctypes  # (imported for readers who want to poke at the library by hand)

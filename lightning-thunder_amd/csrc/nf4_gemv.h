@@ -68,10 +68,15 @@ hipError_t gemv_allow_lds(K kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-// row-streaming kernel, 1 <= M <= 4 (nf4_gemv_rows.hip)
+// row-streaming kernel, M = 1 (nf4_gemv_rows.hip)
 size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_rows_setup();
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream);
+
+// four-rows-per-quad kernel, 2 <= M <= 4 (nf4_gemv_quad.hip)
+size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K);
+hipError_t gemv_quad_setup();
+hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream);
 
 // MFMA tile kernel, 5 <= M <= 16 (nf4_gemv.hip)
 size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K);

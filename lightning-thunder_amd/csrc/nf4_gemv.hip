@@ -1,5 +1,5 @@
 // Decode-shape fused NF4 dequant-matmul for gfx950, 5 <= M <= 16 rows of x (MFMA tiles), and the
-// dispatch between it and the row-streaming kernel that serves M <= 4.
+// dispatch between it, the row-streaming kernel (M = 1) and the four-rows-per-quad kernel (M = 2..4).
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -306,6 +306,7 @@ hipError_t device_setup(int* cus_out) {
         if (e != hipSuccess) return e;
         if ((e = gemv_tiles_setup()) != hipSuccess) return e;
         if ((e = gemv_rows_setup()) != hipSuccess) return e;
+        if ((e = gemv_quad_setup()) != hipSuccess) return e;
         g_num_cus[dev] = cus > 0 ? cus : 256;
     }
     *cus_out = g_num_cus[dev];
@@ -349,14 +350,16 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
 // ---- dispatch -------------------------------------------------------------------------------
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    return M <= 4 ? gemv_rows_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
+    if (M == 1) return gemv_rows_workspace_bytes(M, N, K);
+    return M <= 4 ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
 }
 
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     int cus = 0;
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;
-    return a.M <= 4 ? launch_gemv_rows(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
+    if (a.M == 1) return launch_gemv_rows(a, cus, stream);
+    return a.M <= 4 ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
 }
 
 }  // namespace nf4

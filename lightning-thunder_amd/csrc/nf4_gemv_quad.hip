@@ -1,0 +1,373 @@
+// Decode-shape fused NF4 dequant-matmul for gfx950, 2 <= M <= 4 rows of x.
+//
+// Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
+// bitsandbytes.matmul_4bit picks for a single-row x; call site
+// thunder/transforms/quantization.py:39.
+//
+// HBM-bound: 0.5 byte of codes + 4/blocksize bytes of absmax per weight, each read exactly once.
+//
+//  * Lane mapping.  A wave works on FOUR weight rows at a time.  Lane l = 4*s + r holds row r of the
+//    group and k segment s (32 consecutive k): one 16-byte load per lane, and the 16 lanes of a row
+//    read 256 contiguous bytes.  CPW such loads (512 k each) cover the wave's k range; the 8 waves
+//    of a workgroup are (waves along K) x (row groups), so a workgroup streams whole rows.
+//  * v_mfma_f32_4x4x4_16b_bf16 computes one 4x4x4 product per group of 4 lanes: A row i comes from
+//    lane i of the quad (4 weights of weight-row i), B column j from lane j (4 values of x row j at
+//    the same k).  C[i][j] = weight-row i . x-row j, so ALL 16 results of the quad are wanted and
+//    M = 2, 3, 4 cost exactly what M = 1 costs.  Lane j keeps x row j in registers (rows >= M: 0).
+//  * Code -> bf16: 256-entry LDS table indexed by a whole packed byte, both code values as one
+//    dword, replicated per lane with a 256-byte stride: address (byte << 8) | lane*4 is one
+//    v_perm_b32 and bank-conflict free.
+//  * Scale: a lane's 32 weights share one absmax; the 8-MFMA partial of row i is scaled by the
+//    absmax lane i of the quad loaded (a DPP quad broadcast folded into the FMA).  EXACT variant
+//    (K > 16384): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA, which is
+//    the reference's dequantisation bit for bit.
+//  * Reduction over the 16 k segments: a transposing butterfly leaves the 16 (row, m) totals of the
+//    group in lanes 0..15; per-(row, wave) sums are parked in LDS and added in a fixed order.
+//  * K larger than one workgroup covers is split over workgroups; partial sums cross workgroups
+//    through agent-scope relaxed atomics and a counter (no L2-wide fences), added in a fixed order
+//    by the last workgroup to arrive.
+#include "nf4_gemv.h"
+
+namespace nf4 {
+namespace {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int PART_BYTES = 16 * 1024;  // per-(row, wave, m) partial sums of one band
+constexpr int SMEM_BYTES = GEMV_TABLE_BYTES + PART_BYTES;
+constexpr int LOAD_K = 512;            // k covered by one wave-wide 16-byte load (16 segments of 32)
+constexpr int FLAG_OFFSET = GEMV_TABLE_BYTES + PART_BYTES - 16;
+
+struct QuadPlan {
+    int waves_k;          // waves of a workgroup along K
+    int row_groups;       // 4-row groups processed concurrently by a workgroup = 8 / waves_k
+    int splits;           // K splits across workgroups
+    int groups_per_band;  // 4-row groups of one task
+    int nbands;
+    int ntasks;           // nbands * splits
+    int aligned;          // K % blocksize == 0
+};
+
+#define NF4_DPP(v, ctrl, bank, keep_old) \
+    __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep_old), __builtin_bit_cast(int, v), ctrl, 0xf, bank, false))
+
+// value of `v` in lane (lane ^ 4); DPP shifts by 4 inside a row of 16, direction chosen per bank of 4
+__device__ __forceinline__ float lane_xor4(float v) {
+    float o = NF4_DPP(v, 0x104 /*row_shl:4*/, 0x5, 0.0f);
+    return NF4_DPP(v, 0x114 /*row_shr:4*/, 0xa, o);
+}
+
+// t[0..3]: this lane's partial sums for weight rows 0..3 of the group (and x row lane & 3).
+// Returns in every lane the total over the 16 k segments of weight row 2*bit3 + bit2 (bits of lane).
+__device__ __forceinline__ float reduce_rows(const float t[4], int lane) {
+    const bool b2 = lane & 4, b3 = lane & 8;
+    float w[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {  // rows (0,1) and (2,3): lane bit 2 picks the row the lane keeps
+        const float keep = b2 ? t[2 * p + 1] : t[2 * p];
+        const float send = b2 ? t[2 * p] : t[2 * p + 1];
+        w[p] = keep + lane_xor4(send);
+    }
+    const float keep = b3 ? w[1] : w[0];
+    const float send = b3 ? w[0] : w[1];
+    float y = keep + NF4_DPP(send, 0x128 /*row_ror:8*/, 0xf, 0.0f);
+    y += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, y)));
+    y += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, y)));
+    return y;
+}
+
+template <int CPW, int U, bool NESTED, bool EXACT>
+__global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a, QuadPlan p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lane4 = (uint32_t)lane * 4u;
+    const uint32_t lane8 = (uint32_t)(lane & 31) * 8u;
+    const int ri = lane & 3;        // weight row inside the group of 4, and the x row this lane feeds
+    const uint32_t kseg = 32u * (uint32_t)(lane >> 2);
+
+    // the code-book entry this lane contributes to the LDS table: requested first, used last
+    const float lut_mine = a.lut16[lane & 15];
+    bool table_built = false;
+
+    float* part = reinterpret_cast<float*>(smem + GEMV_TABLE_BYTES);
+    int* flag = reinterpret_cast<int*>(smem + FLAG_OFFSET);
+    unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
+
+    const int cw = wave % p.waves_k;
+    const int rg = wave / p.waves_k;
+    const int64_t K = a.K;
+    const int M = a.M;
+    const int step = p.row_groups;
+
+    for (int task = blockIdx.x; task < p.ntasks; task += gridDim.x) {
+        const int band = task / p.splits;
+        const int ks = task - band * p.splits;
+        const int g_begin = band * p.groups_per_band;
+        const int g_end = min((a.N + 3) / 4, g_begin + p.groups_per_band);
+        const int64_t kw0 = (int64_t)(ks * p.waves_k + cw) * (CPW * LOAD_K);
+        const bool wave_on = rg < p.row_groups && kw0 < K && g_begin + rg < g_end;
+        const int cnt = wave_on ? (g_end - g_begin - rg + step - 1) / step : 0;  // groups of this wave
+        bool lane_on[CPW];
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) lane_on[c] = wave_on && kw0 + c * LOAD_K + kseg < K;
+
+        // x row `ri`, this lane's 32 k of every load
+        uint32_t xr[CPW][16];
+#pragma unroll
+        for (int c = 0; c < CPW; ++c)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (lane_on[c] && ri < M) v = *reinterpret_cast<const uint4*>(a.x + ri * K + kw0 + c * LOAD_K + kseg + 8 * q);
+                xr[c][4 * q + 0] = v.x; xr[c][4 * q + 1] = v.y; xr[c][4 * q + 2] = v.z; xr[c][4 * q + 3] = v.w;
+            }
+
+        uint4 wq[U][CPW];
+        float sq[U][CPW];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) {
+                wq[u][c] = make_uint4(0, 0, 0, 0);
+                sq[u][c] = 0.0f;
+            }
+        // group i of this wave is g_begin + rg + i * step; its rows are 4 * group + ri
+        auto issue = [&](int u, int i) {
+            const int row = min(4 * (g_begin + rg + i * step) + ri, a.N - 1);
+            const int64_t e0 = (int64_t)row * K + kw0 + kseg;
+#pragma unroll
+            for (int c = 0; c < CPW; ++c)
+                if (lane_on[c]) {
+                    const int64_t e = e0 + c * LOAD_K;
+                    wq[u][c] = load16_stream(a.packed + (e >> 1));
+                    const int64_t blk = e >> a.block_log2;
+                    sq[u][c] = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
+                }
+        };
+        // get the weight stream going before anything else happens
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < cnt) issue(u, u);
+
+        if (!table_built) {  // first task only: overlaps with the loads above
+            if (EXACT)
+                build_pair_table_f32(smem, lut_mine, lane, wave);
+            else
+                build_pair_table(smem, lut_mine, lane, wave);
+            table_built = true;
+        }
+        __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
+
+        for (int i0 = 0; i0 < cnt; i0 += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float tot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < CPW; ++c) {
+                    const uint32_t d[4] = {wq[u][c].x, wq[u][c].y, wq[u][c].z, wq[u][c].w};
+                    const float s = sq[u][c];
+                    uint32_t pr[16];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const uint32_t sel = 0x0c0c0400u | ((uint32_t)j << 8);
+                            if (EXACT) {
+                                // bf16(lut[c] * absmax) per weight, the value nf4hip_dequantize produces
+                                const float2 v = lds_table_read2(__builtin_amdgcn_perm(d[q], lane8, sel));
+                                f32x2 f = {__fmul_rn(v.x, s), __fmul_rn(v.y, s)};
+                                pr[4 * q + j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+                            } else {
+                                pr[4 * q + j] = lds_table_read(__builtin_amdgcn_perm(d[q], lane4, sel));
+                            }
+                        }
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const uint2 wa = make_uint2(pr[2 * t], pr[2 * t + 1]);
+                        const uint2 xb = make_uint2(xr[c][2 * t], xr[c][2 * t + 1]);
+                        acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
+                                                                     __builtin_bit_cast(s16x4, xb), acc, 0, 0, 0);
+                    }
+                    if (EXACT) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) tot[i] += acc[i];
+                    } else {
+                        // acc[i] belongs to weight row i, whose absmax lane i of this quad holds
+                        tot[0] = fmaf(acc[0], NF4_DPP(s, 0x00, 0xf, 0.0f), tot[0]);
+                        tot[1] = fmaf(acc[1], NF4_DPP(s, 0x55, 0xf, 0.0f), tot[1]);
+                        tot[2] = fmaf(acc[2], NF4_DPP(s, 0xAA, 0xf, 0.0f), tot[2]);
+                        tot[3] = fmaf(acc[3], NF4_DPP(s, 0xFF, 0xf, 0.0f), tot[3]);
+                    }
+                }
+                const int i = i0 + u;
+                if (i + U < cnt) {
+                    issue(u, i + U);
+                } else {  // slot is dead from here on; say so, or the compiler keeps copies alive
+#pragma unroll
+                    for (int c = 0; c < CPW; ++c) {
+                        wq[u][c] = make_uint4(0, 0, 0, 0);
+                        sq[u][c] = 0.0f;
+                    }
+                }
+                const float total = reduce_rows(tot, lane);  // lanes 0..15: row 2*b3+b2 of the group, x row ri
+                const int grow = 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);
+                if (lane < 16 && ri < M && i < cnt)
+                    part[(((rg + i * step) * 4 + grow) * p.waves_k + cw) * M + ri] = total;
+            }
+        }
+        __syncthreads();
+
+        // ---- band epilogue: add the waves of every row in a fixed order ----
+        const int r_begin = 4 * g_begin;
+        const int nrows = min(a.N, 4 * g_end) - r_begin;
+        // the last split may own fewer waves along K than the others
+        const int wave_k = CPW * LOAD_K;
+        const int nwk = min(p.waves_k, (int)((K + wave_k - 1) / wave_k) - ks * p.waves_k);
+        if (p.splits == 1) {
+            for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                const int r = idx / M, m = idx - r * M;
+                float sum = 0.0f;
+                for (int c = 0; c < nwk; ++c) sum += part[(r * p.waves_k + c) * M + m];
+                const int n = r_begin + r;
+                if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
+                a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
+            }
+        } else {
+            for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                const int r = idx / M, m = idx - r * M;
+                float sum = 0.0f;
+                for (int c = 0; c < nwk; ++c) sum += part[(r * p.waves_k + c) * M + m];
+                __hip_atomic_store(&partial[((int64_t)ks * M + m) * a.N + r_begin + r], sum, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned prev =
+                    __hip_atomic_fetch_add(&counters[band], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *flag = (prev == (unsigned)p.splits - 1u);
+            }
+            __syncthreads();
+            if (*flag != 0) {
+                for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                    const int r = idx / M, m = idx - r * M;
+                    const int n = r_begin + r;
+                    float sum = 0.0f;
+                    for (int k2 = 0; k2 < p.splits; ++k2)
+                        sum += __hip_atomic_load(&partial[((int64_t)k2 * M + m) * a.N + n], __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+                    if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
+                    a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
+                }
+                if (tid == 0) __hip_atomic_store(&counters[band], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+}
+
+// k per wave = 512 * CPW.  Two loads per lane and row group keep x in 32 registers; one workgroup
+// (8 waves) then covers K <= 8192, larger K is split over workgroups.
+int pick_cpw(int64_t K) { return K <= 2 * LOAD_K ? 1 : 2; }
+
+int quad_splits(int64_t K) {
+    const int64_t wave_k = (int64_t)pick_cpw(K) * LOAD_K;
+    const int64_t nwk = (K + wave_k - 1) / wave_k;
+    return (int)((nwk + GEMV_WAVES - 1) / GEMV_WAVES);
+}
+
+QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots) {
+    QuadPlan p;
+    p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
+    const int64_t wave_k = (int64_t)pick_cpw(K) * LOAD_K;
+    const int nwk = (int)((K + wave_k - 1) / wave_k);
+    p.splits = quad_splits(K);
+    p.waves_k = (nwk + p.splits - 1) / p.splits;
+    p.row_groups = GEMV_WAVES / p.waves_k;
+    const int groups = (int)((N + 3) / 4);
+    const int cap = ((PART_BYTES - 64) / (4 * p.waves_k * M * 4)) / p.row_groups * p.row_groups;
+    int bands_target = slots / p.splits;
+    if (bands_target < 1) bands_target = 1;
+    // one task per resident workgroup if its partial sums fit in LDS, else 2, 3, ... balanced rounds
+    int gpb = cap;
+    for (int rounds = 1; rounds <= 64; ++rounds) {
+        int g = (groups + rounds * bands_target - 1) / (rounds * bands_target);
+        g = (g + p.row_groups - 1) / p.row_groups * p.row_groups;
+        if (g <= cap) {
+            gpb = g;
+            break;
+        }
+    }
+    if (gpb < p.row_groups) gpb = p.row_groups;
+    p.groups_per_band = gpb;
+    p.nbands = (groups + gpb - 1) / gpb;
+    p.ntasks = p.nbands * p.splits;
+    return p;
+}
+
+template <int CPW, int U, bool NESTED>
+hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
+    if (gemv_wants_exact(a.K))
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, NESTED, true>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    else
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, NESTED, false>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    return hipGetLastError();
+}
+
+// U = row groups in flight per wave: U * CPW 16-byte loads per lane, at most 8
+template <int CPW, bool NESTED>
+hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
+    const int cnt = p.groups_per_band / p.row_groups;  // groups per wave and task
+    constexpr int UMAX = 8 / CPW;
+    if constexpr (UMAX >= 8)
+        if (cnt >= 8) return launch_u<CPW, 8, NESTED>(a, p, grid, stream);
+    if constexpr (UMAX >= 4)
+        if (cnt >= 4) return launch_u<CPW, 4, NESTED>(a, p, grid, stream);
+    return launch_u<CPW, 2, NESTED>(a, p, grid, stream);
+}
+
+template <bool NESTED>
+hipError_t launch_n(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
+    return pick_cpw(a.K) == 1 ? launch_c<1, NESTED>(a, p, grid, stream) : launch_c<2, NESTED>(a, p, grid, stream);
+}
+
+template <int CPW, int U>
+hipError_t allow_lds_cu() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, false, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, true, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, false, true>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_quad_kernel<CPW, U, true, true>, SMEM_BYTES);
+}
+
+}  // namespace
+
+size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int s = quad_splits(K);
+    return (size_t)GEMV_COUNTER_BYTES + (s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0);
+}
+
+hipError_t gemv_quad_setup() {
+    hipError_t e;
+    if ((e = allow_lds_cu<1, 8>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<1, 4>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<1, 2>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<2, 4>()) != hipSuccess) return e;
+    return allow_lds_cu<2, 2>();
+}
+
+hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {
+    int slots = 2 * cus;
+    if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
+    const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots);
+    const int grid = p.ntasks < slots ? p.ntasks : slots;
+    return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
+}
+
+}  // namespace nf4

@@ -1,4 +1,4 @@
-// Decode-shape fused NF4 dequant-matmul for gfx950, 1 <= M <= 4 rows of x: the GEMV proper.
+// Decode-shape fused NF4 dequant-matmul for gfx950, M = 1 (any M <= 4 works): the GEMV proper.
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -300,9 +300,16 @@ RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots) 
     const int cap = ((PART_BYTES - 64) / (p.chunks * M * 4)) / p.row_lanes * p.row_lanes;
     int bands_target = slots / p.splits;
     if (bands_target < 1) bands_target = 1;
-    int64_t rpb = (N + bands_target - 1) / bands_target;
-    rpb = (rpb + p.row_lanes - 1) / p.row_lanes * p.row_lanes;
-    if (rpb > cap) rpb = cap;
+    // one task per resident workgroup if its partial sums fit in LDS, else 2, 3, ... balanced rounds
+    int64_t rpb = cap;
+    for (int rounds = 1; rounds <= 64; ++rounds) {
+        int64_t r = (N + (int64_t)rounds * bands_target - 1) / ((int64_t)rounds * bands_target);
+        r = (r + p.row_lanes - 1) / p.row_lanes * p.row_lanes;
+        if (r <= cap) {
+            rpb = r;
+            break;
+        }
+    }
     if (rpb < p.row_lanes) rpb = p.row_lanes;
     p.rows_per_band = (int)rpb;
     p.nbands = (int)((N + rpb - 1) / rpb);
@@ -333,12 +340,7 @@ hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_
 
 template <bool NESTED>
 hipError_t launch_n(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
-    switch (a.M) {
-        case 1: return launch_m<1, NESTED>(a, p, grid, stream);
-        case 2: return launch_m<2, NESTED>(a, p, grid, stream);
-        case 3: return launch_m<3, NESTED>(a, p, grid, stream);
-        default: return launch_m<4, NESTED>(a, p, grid, stream);
-    }
+    return launch_m<1, NESTED>(a, p, grid, stream);  // M = 2..4 is served by the four-rows-per-quad kernel
 }
 
 template <int M, int U>
@@ -367,12 +369,8 @@ size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 hipError_t gemv_rows_setup() {
-    hipError_t e;
-    if ((e = allow_lds_mu<1, 8>()) != hipSuccess) return e;
-    if ((e = allow_lds_m<1>()) != hipSuccess) return e;
-    if ((e = allow_lds_m<2>()) != hipSuccess) return e;
-    if ((e = allow_lds_m<3>()) != hipSuccess) return e;
-    return allow_lds_m<4>();
+    const hipError_t e = allow_lds_mu<1, 8>();
+    return e != hipSuccess ? e : allow_lds_m<1>();
 }
 
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {

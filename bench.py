@@ -98,7 +98,7 @@ def main() -> int:
     groups = [
         ("gemv_rows_kernel", "M = 1, row-streaming", [(M, N, K) for M in MS if M == 1 for (N, K) in SHAPES]),
         ("gemv_quad_kernel", "M = 4, four rows per lane quad", [(M, N, K) for M in MS if 2 <= M <= 4 for (N, K) in SHAPES]),
-        ("gemv_kernel", "M = 16, MFMA tiles", [(M, N, K) for M in MS if M > 4 for (N, K) in SHAPES]),
+        ("gemv_tiles_kernel", "M = 16, MFMA tiles", [(M, N, K) for M in MS if M > 4 for (N, K) in SHAPES]),
     ]
     group_bytes = [sum(algorithmic_bytes(*c) for c in calls) for _, _, calls in groups]
     bytes_step = sum(group_bytes)

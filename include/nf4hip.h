@@ -98,7 +98,7 @@ int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const f
  *   out[m][n] = bf16( sum_k x[m][k] * lut16[code(n,k)] * absmax[(n*K+k)/blocksize] + bias[n] )
  *   x    [M, K] bf16 row-major      out  [M, N] bf16 row-major      bias [N] bf16 or NULL
  * Fast-path rules (else NF4HIP_E_SHAPE; the host side then takes dequantize + matmul):
- *   x_dtype == NF4HIP_BF16, K % 512 == 0, blocksize divides K.
+ *   x_dtype == NF4HIP_BF16; M <= 4: K % 32 == 0; M >= 5: K % 512 == 0, blocksize divides K, K <= 2^24.
  * `workspace` must hold nf4hip_gemv_workspace_bytes(M,N,K) bytes, be 16-byte aligned, and have
  * been ZEROED once before its first use; every call leaves it zeroed where that matters, so it
  * can be reused by later calls on the same stream.  Two calls that may overlap in time (different

@@ -70,6 +70,8 @@ int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const 
         if (M <= 4 ? K % 32 : K % 512)
             return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: K = %lld is not a multiple of %d (M = %lld)", (long long)K,
                         M <= 4 ? 32 : 512, (long long)M);
+        if (M > 4 && K > (1 << 24))
+            return fail(NF4HIP_E_SHAPE, "nf4hip_gemv: K = %lld > 2^24 with M > 4 (use nf4hip_gemm)", (long long)K);
     } else {
         if (K % 64) return fail(NF4HIP_E_SHAPE, "nf4hip_gemm: K = %lld is not a multiple of 64", (long long)K);
     }

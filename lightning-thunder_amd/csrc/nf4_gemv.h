@@ -8,7 +8,7 @@ namespace nf4 {
 constexpr int GEMV_THREADS = 512;  // 8 waves; two workgroups per CU
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_TABLE_BYTES = 256 * 256;     // 256 byte values x 64 lanes x 4 B
-constexpr int GEMV_COUNTER_BYTES = 4096 * 4;    // split-K arrival counters at the head of the workspace
+constexpr int GEMV_COUNTER_BYTES = 65536 * 4;   // split-K arrival counters at the head of the workspace
 
 // Byte -> (bf16, bf16) table at the start of LDS.  Entry b holds the code values of the two
 // nibbles of b as bf16, the high nibble (even element) in the low half.  It is replicated for the
@@ -16,14 +16,20 @@ constexpr int GEMV_COUNTER_BYTES = 4096 * 4;    // split-K arrival counters at t
 // owns one bank column and a lookup is conflict-free whatever the data.
 // `lut_lane` is lut16[lane & 15], loaded by the caller (early, so that its latency is hidden).
 __device__ __forceinline__ void build_pair_table(uint8_t* smem, float lut_lane, int lane, int wave) {
+    // Every entry is one dword replicated over a 256-byte row.  Sixteen lanes write one row with
+    // 16-byte stores, so a wave writes four entries per instruction and its 32 entries in eight.
     const uint32_t lb = f32_to_bf16_bits(lut_lane);
-    uint32_t* table = reinterpret_cast<uint32_t*>(smem);
-#pragma unroll 8
-    for (int it = 0; it < 32; ++it) {
-        const int e = wave * 32 + it;
-        const uint32_t first = __builtin_amdgcn_readlane(lb, e >> 4);   // high nibble = even element
-        const uint32_t second = __builtin_amdgcn_readlane(lb, e & 15);  // low nibble = odd element
-        table[e * 64 + lane] = first | (second << 16);
+    uint4* table = reinterpret_cast<uint4*>(smem);
+    const int sub = lane >> 4;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int e = wave * 32 + it * 4 + sub;
+        // high nibble = even element: wave * 2 + (it >> 2), the same for all four entries
+        const uint32_t first = __builtin_amdgcn_readlane(lb, wave * 2 + (it >> 2));
+        // low nibble = odd element: lane (it * 4 + sub) & 15 holds its code value
+        const uint32_t second = (uint32_t)__builtin_amdgcn_ds_bpermute(((it * 4 + sub) & 15) * 4, (int)lb);
+        const uint32_t v = first | (second << 16);
+        table[e * 16 + (lane & 15)] = make_uint4(v, v, v, v);
     }
 }
 
@@ -61,6 +67,25 @@ __device__ __forceinline__ float2 lds_table_read2(uint32_t addr) {
     typedef __attribute__((address_space(3))) const f32x2_t* lds_f2_ptr;
     const f32x2_t v = *reinterpret_cast<lds_f2_ptr>((uintptr_t)addr);
     return make_float2(v.x, v.y);
+}
+
+// Sum, in slice order, of the `splits` partial sums of one output (first one at p0, `stride` floats
+// apart).  The partial sums were written by other workgroups with agent-scope stores; the loads are
+// agent-scope too and are issued eight at a time before the first add, so that their latencies
+// overlap; the order of the adds is fixed.
+__device__ __forceinline__ float sum_partials(const float* p0, int64_t stride, int splits) {
+    float sum = 0.0f;
+    for (int k2 = 0; k2 < splits; k2 += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            v[j] = k2 + j < splits
+                       ? __hip_atomic_load(p0 + (int64_t)(k2 + j) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                       : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sum += v[j];
+    }
+    return sum;
 }
 
 template <typename K>

@@ -1,0 +1,552 @@
+// Decode-shape fused NF4 dequant-matmul for gfx950, 5 <= M <= 16 rows of x: MFMA tiles.
+//
+// Replaces bitsandbytes' gemv_4bit / small-batch matmul_4bit, call site
+// thunder/transforms/quantization.py:39.
+//
+// The kernel is HBM-bound: per weight it moves 4 bits of code plus 1/blocksize of an fp32 absmax.
+// One workgroup (8 waves) per CU; wave w of a workgroup owns the w-th 16-row tile of each of the
+// workgroup's 128-row tile groups.  The x operands of one K slice are resident in LDS in MFMA
+// order, so the waves run unsynchronised except when the slice changes.  Tile groups are taken
+// in batches of up to four whose accumulators all live in registers: the batch sweeps the slices
+// of the workgroup's K range one after the other, so a long K costs a re-staging of x per slice
+// and batch, not a round trip of partial sums.  Weight loads run through a four-slot register
+// ring (one 512-k phase of one tile per slot) that stays full across tile, slice and batch
+// boundaries.
+//
+//  * Weight stream.  Per phase a lane issues four 16-byte loads; in load i, lane l reads row
+//    4*((l>>2)&3) + i of the tile at byte (l>>4)*64 + (l&3)*16 of the row's 256-byte phase slice,
+//    so four ADJACENT lanes read 64 contiguous bytes (one L1 request instead of four) and one load
+//    instruction covers four rows x 256 contiguous bytes.
+//  * Into MFMA order, in registers.  A 4x4 transpose inside each lane quad (DPP quad_perm +
+//    select) exchanges "load index" with "lane & 3", after which lane l holds row l & 15; a 4x4
+//    transpose across lanes {c, c+16, c+32, c+48} (v_permlane32_swap, v_permlane16_swap) then
+//    makes every MFMA cover 32 CONSECUTIVE k, so two MFMAs = one 64-element quantisation block.
+//  * Code -> bf16.  256-entry byte -> (bf16, bf16) LDS table replicated per lane: one v_perm_b32
+//    builds the address, one ds_read_b32 returns two MFMA-ready values.
+//  * Contraction.  v_mfma_f32_16x16x32_bf16, A = x (rows m), B = W (columns n): the accumulator of
+//    a lane belongs to the lane's own weight row, so the absmax scale of a block is one the lane
+//    loaded itself (4 FMAs per block).
+//  * x.  Up to 80 KB resident: 5 phases of 16 rows, or 10 phases of 8 rows when M <= 8 (lanes of
+//    rows >= 8 then re-read rows 0..7; an MFMA output row depends on its own A row only, and rows
+//    >= M are never stored).  XOR-swizzled so that both the scattered staging writes and the
+//    linear operand reads are conflict-free.
+//  * K split.  Only when N alone cannot fill the chip is K also split over workgroups; partial
+//    sums then go to a workspace and the last WAVE to finish a tile (device-scope counter per
+//    tile) adds them in a fixed order, so the result does not depend on scheduling.
+#include "nf4_gemv.h"
+
+namespace nf4 {
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int THREADS = GEMV_THREADS;
+constexpr int WAVES = GEMV_WAVES;
+constexpr int TABLE_BYTES = GEMV_TABLE_BYTES;
+constexpr int PHASE_K = 512;                 // k per phase
+constexpr int XBYTES_MAX = 80 * 1024;        // resident x operands
+constexpr int SMEM_BYTES = TABLE_BYTES + XBYTES_MAX;
+constexpr int COUNTER_BYTES = GEMV_COUNTER_BYTES;
+constexpr int SLOTS = 4;                     // ring slots = accumulator sets = largest batch
+
+struct Plan {
+    int tile_groups;   // ceil(N / 128)
+    int splits;        // K ranges across workgroups
+    int range_phases;  // phases per K range (the last range may be shorter)
+    int total_phases;  // K / 512
+    int tg_step;       // gridDim.x / splits: distance between a workgroup's consecutive tile groups
+};
+
+struct PhaseRegs {
+    uint4 w[4];   // [load]: 32 codes each
+    float4 s[2];  // absmax of the 8 blocks of the phase (or raw data to build them)
+};
+
+// Position in the item stream of a workgroup (wave-uniform).  An item is one phase of one tile
+// group.  Order: batch, slice, phase, tile group of the batch; `slot` counts items of the batch
+// modulo 4, so that with batches of 1, 2 or 4 tile groups a slot always meets the same tile group.
+struct Cursor {
+    int bi;     // index (in the workgroup's list of tile groups) of the batch's first tile group
+    int nb;     // tile groups in the batch: 1, 2 or 4
+    int batch;  // batch number
+    int q;      // slice step within the batch (odd batches walk the slices backwards)
+    int ph;     // phase within the slice
+    int t;      // tile group within the batch
+    int slot;
+    bool valid;
+};
+
+// Lane-dependent constants of the load side.
+struct LaneLoad {
+    uint32_t woff[4];  // per load: byte offset from the tile's first byte of the phase
+    uint32_t s_off;    // absmax blocks from the tile's first row to the lane's row
+};
+
+// 4x4 dword transpose across the lanes {c, c+16, c+32, c+48}: afterwards element a of lane g holds
+// what element g of lane a held.
+__device__ __forceinline__ void transpose_g(uint32_t d[4]) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {  // lane bit 5 <-> element bit 1
+        auto r = __builtin_amdgcn_permlane32_swap(d[j], d[j + 2], false, false);
+        d[j] = r[0];
+        d[j + 2] = r[1];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j += 2) {  // lane bit 4 <-> element bit 0
+        auto r = __builtin_amdgcn_permlane16_swap(d[j], d[j + 1], false, false);
+        d[j] = r[0];
+        d[j + 1] = r[1];
+    }
+}
+
+// One stage of the in-quad transpose: lanes whose `bit` is 0 keep A and receive the partner's A
+// into B; lanes whose bit is 1 keep B and receive the partner's B into A.
+template <int DPP_CTRL>
+__device__ __forceinline__ void quad_exchange(uint32_t& A, uint32_t& B, bool bit) {
+    const uint32_t pa = (uint32_t)__builtin_amdgcn_update_dpp((int)A, (int)A, DPP_CTRL, 0xf, 0xf, true);
+    const uint32_t pb = (uint32_t)__builtin_amdgcn_update_dpp((int)B, (int)B, DPP_CTRL, 0xf, 0xf, true);
+    A = bit ? pb : A;
+    B = bit ? B : pa;
+}
+
+// 4x4 transpose of r[0..3] across the four lanes of a quad: afterwards r[i] of lane q holds what
+// r[q] of lane i (of the same quad) held.
+__device__ __forceinline__ void transpose_quad(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3, bool b0,
+                                               bool b1) {
+    quad_exchange<0xB1>(r0, r1, b0);  // quad_perm [1,0,3,2]
+    quad_exchange<0xB1>(r2, r3, b0);
+    quad_exchange<0x4E>(r0, r2, b1);  // quad_perm [2,3,0,1]
+    quad_exchange<0x4E>(r1, r3, b1);
+}
+
+template <bool B64, bool NESTED>
+__device__ __forceinline__ void load_phase(const MatmulArgs& a, PhaseRegs& r, const LaneLoad& ll, int n0c, int kabs) {
+    // n0c = first row actually read for the tile, kabs = first k of the phase (both wave-uniform)
+    const int64_t e0 = (int64_t)n0c * a.K + kabs;
+    const uint8_t* wp = a.packed + (e0 >> 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.w[i] = load16_stream(wp + ll.woff[i]);
+    if (NESTED) {
+        if (B64) {
+            const int64_t b = (e0 >> 6) + ll.s_off;
+            const uint2 q = *reinterpret_cast<const uint2*>(a.nested.q + b);
+            r.s[0].x = __uint_as_float(q.x);
+            r.s[0].y = __uint_as_float(q.y);
+            // 8 consecutive blocks starting at a multiple of 8 share one nested block (>= 64 blocks)
+            r.s[0].z = a.nested.absmax2[b >> a.nested.nested_log2];
+        } else {
+            const int64_t b = ((int64_t)n0c * a.K >> a.block_log2) + ll.s_off;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                r.s[j].x = nested_absmax(a.nested, b + ((kabs + j * 256) >> a.block_log2));
+                r.s[j].y = nested_absmax(a.nested, b + ((kabs + j * 256 + 64) >> a.block_log2));
+                r.s[j].z = nested_absmax(a.nested, b + ((kabs + j * 256 + 128) >> a.block_log2));
+                r.s[j].w = nested_absmax(a.nested, b + ((kabs + j * 256 + 192) >> a.block_log2));
+            }
+        }
+    } else if (B64) {
+        const float* sp = a.absmax + (e0 >> 6) + ll.s_off;
+        r.s[0] = *reinterpret_cast<const float4*>(sp);
+        r.s[1] = *reinterpret_cast<const float4*>(sp + 4);
+    } else {
+        const float* sp = a.absmax + ((int64_t)n0c * a.K >> a.block_log2) + ll.s_off;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            r.s[j].x = sp[(kabs + j * 256) >> a.block_log2];
+            r.s[j].y = sp[(kabs + j * 256 + 64) >> a.block_log2];
+            r.s[j].z = sp[(kabs + j * 256 + 128) >> a.block_log2];
+            r.s[j].w = sp[(kabs + j * 256 + 192) >> a.block_log2];
+        }
+    }
+}
+
+// LDS layout of the resident x operands.  One phase = 16 MFMAs (j); MFMA j reads, for lane
+// (gg = lane >> 4, m = lane & 15), the 16 bytes x[m][32 j + 8 gg .. + 8].  With R rows held
+// (R = 16, or 8 when M <= 8) a phase takes R KB and the slot of (j, gg, m) is
+//     j * 4R + gg * R + ((m ^ ((j & 1) << 2 | gg)) & (R - 1)):
+// linear in the lane up to an XOR inside each R-slot group, so operand reads are conflict-free,
+// and the XOR spreads the eight consecutive 8-k pieces that eight adjacent staging lanes write
+// (same m, piece & 7 = 0..7) over all banks.
+template <int R>
+__device__ __forceinline__ uint32_t xslot_bytes(int m, int piece) {
+    const int j = piece >> 2, gg = piece & 3;
+    return (uint32_t)(j * 4 * R + gg * R + ((m ^ (((j & 1) << 2) | gg)) & (R - 1))) * 16u;
+}
+
+// The codes of one phase in MFMA order plus the scales of its 8 blocks: what is left of a ring slot
+// once its registers have been handed back to the next load.
+struct PhaseOperands {
+    uint32_t d[4][4];  // d[q][p] = bytes [64 p + 16 q + 4 (lane >> 4), +4) of row (lane & 15)
+    float sc[8];
+};
+
+template <bool B64, bool NESTED>
+__device__ __forceinline__ void prepare_phase(const MatmulArgs& a, PhaseRegs& r, int lane, PhaseOperands& o) {
+    const bool b0 = lane & 1, b1 = lane & 2;
+    float* sc = o.sc;
+    if (NESTED && B64) {
+        const uint32_t q0 = __float_as_uint(r.s[0].x), q1 = __float_as_uint(r.s[0].y);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t code = ((j < 4 ? q0 : q1) >> (8 * (j & 3))) & 0xffu;
+            sc[j] = __fadd_rn(__fmul_rn(a.nested.map256[code], r.s[0].z), a.nested.offset);
+        }
+    } else {
+        sc[0] = r.s[0].x; sc[1] = r.s[0].y; sc[2] = r.s[0].z; sc[3] = r.s[0].w;
+        sc[4] = r.s[1].x; sc[5] = r.s[1].y; sc[6] = r.s[1].z; sc[7] = r.s[1].w;
+    }
+
+    // in-quad transpose, one dword column at a time: load index <-> lane & 3
+    transpose_quad(r.w[0].x, r.w[1].x, r.w[2].x, r.w[3].x, b0, b1);
+    transpose_quad(r.w[0].y, r.w[1].y, r.w[2].y, r.w[3].y, b0, b1);
+    transpose_quad(r.w[0].z, r.w[1].z, r.w[2].z, r.w[3].z, b0, b1);
+    transpose_quad(r.w[0].w, r.w[1].w, r.w[2].w, r.w[3].w, b0, b1);
+    // now w[q] = bytes [64 * (lane >> 4) + 16 * q, +16) of row (lane & 15)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        o.d[q][0] = r.w[q].x; o.d[q][1] = r.w[q].y; o.d[q][2] = r.w[q].z; o.d[q][3] = r.w[q].w;
+        transpose_g(o.d[q]);
+    }
+}
+
+// MFMA j = 4p + q of the phase covers k [32j, 32j + 32) and uses d[q][p].
+template <int R>
+__device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uint8_t* xph, int lane, f32x4& acc) {
+    const uint32_t lane4 = (uint32_t)lane * 4u;
+    const int gg = lane >> 4, m = lane & 15;
+    const uint32_t xoff_even = (uint32_t)(gg * R + ((m ^ gg) & (R - 1))) * 16u;
+    const uint32_t xoff_odd = (uint32_t)(gg * R + ((m ^ (4 | gg)) & (R - 1))) * 16u;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            f32x4 blk = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
+                const int q = 2 * h + qq;
+                const int j = 4 * p + q;
+                uint32_t t[4];
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    t[b] = lds_table_read(__builtin_amdgcn_perm(o.d[q][p], lane4, 0x0c0c0400u | ((uint32_t)b << 8)));
+                const uint4 xa = *reinterpret_cast<const uint4*>(xph + j * (64 * R) + (qq ? xoff_odd : xoff_even));
+                const uint4 wb = make_uint4(t[0], t[1], t[2], t[3]);
+                blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa),
+                                                              __builtin_bit_cast(bf16x8, wb), blk, 0, 0, 0);
+            }
+            const float scale = o.sc[2 * p + h];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(scale, blk[i], acc[i]);
+        }
+    }
+}
+
+// One (row, phase) of x = 64 pieces of 16 bytes = 1 KB contiguous per wave; at most 80 such units
+// per slice, ten per wave.  All loads are issued before the first LDS write.
+constexpr int XUNITS = XBYTES_MAX / 1024 / WAVES;
+
+__device__ __forceinline__ void load_x_slice(const MatmulArgs& a, uint4 (&xv)[XUNITS], int k0, int n, int lane,
+                                             int wave) {
+#pragma unroll
+    for (int i = 0; i < XUNITS; ++i) {
+        const int u = min(wave + WAVES * i, a.M * n - 1);  // past the end: re-read the last unit
+        const int m = u / n, ph = u - m * n;
+        xv[i] = *reinterpret_cast<const uint4*>(a.x + (int64_t)m * a.K + k0 + ph * PHASE_K + lane * 8);
+    }
+}
+
+template <int R>
+__device__ __forceinline__ void store_x_slice(const MatmulArgs& a, const uint4 (&xv)[XUNITS], uint8_t* xlds, int n,
+                                              int lane, int wave) {
+#pragma unroll
+    for (int i = 0; i < XUNITS; ++i) {
+        const int u = wave + WAVES * i;
+        if (u < a.M * n) {
+            const int m = u / n, ph = u - m * n;
+            *reinterpret_cast<uint4*>(xlds + ph * (R * 1024) + xslot_bytes<R>(m, lane)) = xv[i];
+        }
+    }
+}
+
+// Re-staging in the middle of the stream, four units in flight per wave.
+template <int R>
+__device__ __forceinline__ void restage_x(const MatmulArgs& a, uint8_t* xlds, int k0, int n, int lane, int wave) {
+    const int units = a.M * n;
+    for (int u0 = wave; u0 < units; u0 += 4 * WAVES) {
+        uint4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int u = min(u0 + WAVES * i, units - 1);
+            const int m = u / n, ph = u - m * n;
+            v[i] = *reinterpret_cast<const uint4*>(a.x + (int64_t)m * a.K + k0 + ph * PHASE_K + lane * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int u = u0 + WAVES * i;
+            if (u < units) {
+                const int m = u / n, ph = u - m * n;
+                *reinterpret_cast<uint4*>(xlds + ph * (R * 1024) + xslot_bytes<R>(m, lane)) = v[i];
+            }
+        }
+    }
+}
+
+template <bool B64, bool NESTED, int R>
+__global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Plan p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int CAP = XBYTES_MAX / (R * 1024);  // phases of x that fit
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 15, g = lane >> 4;
+
+    const float lut_lane = a.lut16[lane & 15];
+
+    // this workgroup's K range and tile groups
+    const int ks = (int)blockIdx.x % p.splits;
+    const int tg0 = (int)blockIdx.x / p.splits;
+    const int r0 = ks * p.range_phases;                             // first phase of the range
+    const int rph = min(p.range_phases, p.total_phases - r0);      // phases in the range
+    const int nsl = (rph + CAP - 1) / CAP;                          // x slices in the range
+    const int G = tg0 < p.tile_groups ? (p.tile_groups - 1 - tg0) / p.tg_step + 1 : 0;
+
+    LaneLoad ll;
+    {
+        // rows of a tile are read from n0c = max(min(n0, N - 16), 0) on, so only N < 16 needs a clamp
+        const uint32_t lane_bytes = (uint32_t)(lane >> 4) * 64u + (uint32_t)(lane & 3) * 16u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            ll.woff[i] = (uint32_t)min(((lane >> 2) & 3) * 4 + i, a.N - 1) * (uint32_t)(a.K >> 1) + lane_bytes;
+        ll.s_off = (uint32_t)min(col, a.N - 1) * (uint32_t)(a.K >> a.block_log2);
+    }
+
+    auto batch_size = [&](int bi) {
+        const int rem = G - bi;
+        return rem >= 4 ? 4 : (rem == 3 ? 2 : rem);
+    };
+    auto slice_of = [&](const Cursor& c) { return (c.batch & 1) ? nsl - 1 - c.q : c.q; };
+    auto slice_phases = [&](int sl) { return min(CAP, rph - sl * CAP); };
+    auto advance = [&](Cursor& c) {
+        c.slot = (c.slot + 1) & (SLOTS - 1);
+        if (++c.t < c.nb) return;
+        c.t = 0;
+        if (++c.ph < slice_phases(slice_of(c))) return;
+        c.ph = 0;
+        if (++c.q < nsl) return;
+        c.q = 0;
+        c.bi += c.nb;
+        c.batch += 1;
+        c.slot = 0;
+        c.valid = c.bi < G;
+        c.nb = batch_size(c.bi);
+    };
+    auto first_row = [&](const Cursor& c) {  // first row read for the wave's tile of the item
+        const int n0 = ((tg0 + (c.bi + c.t) * p.tg_step) * WAVES + wave) * 16;
+        return max(min(n0, a.N - 16), 0);
+    };
+    auto first_k = [&](const Cursor& c) { return (r0 + slice_of(c) * CAP + c.ph) * PHASE_K; };
+
+    Cursor lc = {0, batch_size(0), 0, 0, 0, 0, 0, G > 0};  // next item to load
+    Cursor cc = lc;                                         // next item to compute
+    PhaseRegs ring[SLOTS];
+
+    // Prologue staging of x.  Loads return in issue order, so x is requested BEFORE the ring is
+    // filled: its latency is then that of an idle memory system.
+    uint4 xv[XUNITS];
+    load_x_slice(a, xv, (r0 + slice_of(cc) * CAP) * PHASE_K, slice_phases(slice_of(cc)), lane, wave);
+
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) {
+        if (lc.valid && lc.slot == j) {
+            load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
+            advance(lc);
+        }
+    }
+    int resident = slice_of(cc);
+    store_x_slice<R>(a, xv, smem + TABLE_BYTES, slice_phases(resident), lane, wave);
+    build_pair_table(smem, lut_lane, lane, wave);
+    __syncthreads();
+
+    unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + COUNTER_BYTES);
+
+    f32x4 acc[SLOTS];
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    while (cc.valid) {
+        const int fin_bi = cc.bi, fin_nb = cc.nb, fin_batch = cc.batch;
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j) {
+            if (cc.valid && cc.batch == fin_batch && cc.slot == j) {
+                if (cc.ph == 0 && cc.t == 0 && slice_of(cc) != resident) {
+                    __syncthreads();  // every wave is done with the slice that was resident
+                    resident = slice_of(cc);
+                    restage_x<R>(a, smem + TABLE_BYTES, (r0 + resident * CAP) * PHASE_K, slice_phases(resident), lane,
+                                 wave);
+                    __syncthreads();
+                }
+                PhaseOperands o;
+                prepare_phase<B64, NESTED>(a, ring[j], lane, o);
+                // the slot's registers are free again: refill before the long part of the work
+                if (lc.valid && lc.slot == j) {
+                    load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
+                    advance(lc);
+                }
+                contract_phase<R>(o, smem + TABLE_BYTES + cc.ph * (R * 1024), lane, acc[j]);
+                advance(cc);
+            } else if (lc.valid && lc.slot == j) {
+                load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
+                advance(lc);
+            }
+        }
+        if (cc.batch == fin_batch) continue;
+
+        // ---- end of a batch: slot j holds tile group j % nb; lane holds out[m = 4g + i][row] ----
+        if (fin_nb == 1) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[0][i] = (acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i]);
+        } else if (fin_nb == 2) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[0][i] += acc[2][i], acc[1][i] += acc[3][i];
+        }
+#pragma unroll
+        for (int t = 0; t < SLOTS; ++t) {
+            if (t < fin_nb) {
+                const int tile = (tg0 + (fin_bi + t) * p.tg_step) * WAVES + wave;
+                const int n0 = tile * 16;
+                const int n = max(min(n0, a.N - 16), 0) + col;  // the lane's row
+                const bool mine = n >= n0 && n < a.N;
+                if (p.splits == 1) {
+                    if (mine) {
+                        const float b = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.0f;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int m = 4 * g + i;
+                            if (m < a.M) a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(acc[t][i] + b);
+                        }
+                    }
+                } else if (n0 < a.N) {
+                    // Partial sums cross workgroups (and XCDs, whose L2s are not coherent with each
+                    // other) through agent-scope relaxed atomics only: such stores write through
+                    // and such loads bypass stale lines, so no L2-wide write-back/invalidate is
+                    // needed.  Ordering: every store of the wave has completed (s_waitcnt) before
+                    // the wave bumps the tile's counter; the wave that finds splits - 1 there reduces.
+                    if (mine) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int m = 4 * g + i;
+                            if (m < a.M)
+                                __hip_atomic_store(&partial[((int64_t)ks * a.M + m) * a.N + n], acc[t][i],
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    }
+                    __builtin_amdgcn_s_waitcnt(0);
+                    unsigned prev = 0;
+                    if (lane == 0)
+                        prev = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    prev = __builtin_amdgcn_readfirstlane(prev);
+                    if (prev == (unsigned)p.splits - 1u) {
+                        for (int idx = lane; idx < 16 * a.M; idx += 64) {
+                            const int m = idx >> 4;
+                            const int nn = n0 + (idx & 15);
+                            if (nn < a.N) {
+                                float sum = sum_partials(&partial[(int64_t)m * a.N + nn], (int64_t)a.M * a.N, p.splits);
+                                if (a.bias) sum += bf16_bits_to_f32(a.bias[nn]);
+                                a.out[(int64_t)m * a.N + nn] = (uint16_t)f32_to_bf16_bits(sum);
+                            }
+                        }
+                        if (lane == 0)
+                            __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+            }
+            acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+}
+
+constexpr int rows_held(int64_t M) {
+    return M <= 8 ? 8 : 16;
+}
+
+// Work split.  K is split into ranges over workgroups only to fill the chip: the number of ranges
+// minimises rounds x (phases per range + fixed cost) on a device of NOMINAL_SLOTS CUs, one
+// workgroup per CU, where a split adds the partial sums' round trip to the fixed cost.  The choice
+// does not depend on the device at hand, so that the workspace size is a function of the shape
+// alone; the grid does (correctness never depends on how many workgroups are resident).
+constexpr int NOMINAL_SLOTS = 256;
+
+int grid_for(int64_t ntasks, int splits, int slots) {
+    int grid = (int)(ntasks < slots ? ntasks : slots);
+    grid -= grid % splits;
+    return grid < splits ? splits : grid;
+}
+
+Plan make_plan(int64_t M, int64_t N, int64_t K) {
+    Plan p;
+    p.tile_groups = (int)((N + 16 * WAVES - 1) / (16 * WAVES));
+    p.total_phases = (int)(K / PHASE_K);
+    const int cap = XBYTES_MAX / (rows_held(M) * 1024);
+    double best_cost = 1e30;
+    int best_rp = p.total_phases;
+    for (int rp = p.total_phases; rp >= 1; --rp) {
+        const int splits = (p.total_phases + rp - 1) / rp;
+        if ((p.total_phases + splits - 1) / splits != rp) continue;  // same split, shorter last range
+        if (splits > 1 && (int64_t)p.tile_groups * WAVES > COUNTER_BYTES / 4) break;
+        const int64_t ntasks = (int64_t)p.tile_groups * splits;
+        const int grid = grid_for(ntasks, splits, NOMINAL_SLOTS);
+        const int64_t rounds = (ntasks + grid - 1) / grid;
+        const int restages = (rp + cap - 1) / cap;
+        const double fixed = 1.0 + 0.5 * restages + (splits > 1 ? (double)M / 18.0 + 1.0 : 0.0);
+        const double cost = (double)rounds * (rp + fixed);
+        if (cost < best_cost - 1e-9) best_cost = cost, best_rp = rp;
+    }
+    p.range_phases = best_rp;
+    p.splits = (p.total_phases + best_rp - 1) / best_rp;
+    p.tg_step = 0;  // set with the grid
+    return p;
+}
+
+}  // namespace
+
+size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % PHASE_K) return COUNTER_BYTES;
+    const Plan p = make_plan(M, N, K);
+    return (size_t)COUNTER_BYTES + (p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)N * sizeof(float) : 0);
+}
+
+template <bool B64, bool NESTED>
+hipError_t allow_both() {
+    hipError_t e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8>, SMEM_BYTES);
+    if (e != hipSuccess) return e;
+    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16>, SMEM_BYTES);
+}
+
+hipError_t gemv_tiles_setup() {
+    hipError_t e;
+    if ((e = allow_both<false, false>()) != hipSuccess) return e;
+    if ((e = allow_both<true, false>()) != hipSuccess) return e;
+    if ((e = allow_both<false, true>()) != hipSuccess) return e;
+    return allow_both<true, true>();
+}
+
+template <int R>
+hipError_t launch_r(const MatmulArgs& a, const Plan& p, int grid, hipStream_t stream) {
+    const bool b64 = a.block_log2 == 6;
+    const bool nested = a.nested.q != nullptr;
+    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R> : gemv_tiles_kernel<true, false, R>)
+                    : (nested ? gemv_tiles_kernel<false, true, R> : gemv_tiles_kernel<false, false, R>);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
+    Plan p = make_plan(a.M, a.N, a.K);
+    const int grid = grid_for((int64_t)p.tile_groups * p.splits, p.splits, cus < 1024 ? cus : 1024);
+    p.tg_step = grid / p.splits;
+    return rows_held(a.M) == 8 ? launch_r<8>(a, p, grid, stream) : launch_r<16>(a, p, grid, stream);
+}
+
+}  // namespace nf4

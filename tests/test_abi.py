@@ -82,10 +82,12 @@ def test_matmul_argument_errors(ta):
     assert "workspace" in _err(ta)
     assert lib.nf4hip_gemv_dq(A, L.BF16, 1, A, None, A, A, 0.0, 256, A, None, 64, 4096, 64, A, A, ws, None) == L.E_NULL
     assert lib.nf4hip_gemm_dq(A, L.BF16, 64, A, A, A, A, 0.0, 7, A, None, 64, 4096, 64, A, None, 0, None) == L.E_BLOCKSIZE
-    # workspace sizing is pure arithmetic
-    assert lib.nf4hip_gemv_workspace_bytes(1, 4096, 4096) == 16384
-    assert lib.nf4hip_gemv_workspace_bytes(4, 8192, 28672) == 16384 + 4 * 4 * 8192 * 4  # K split over 4 workgroups
-    assert lib.nf4hip_gemv_workspace_bytes(16, 1024, 4096) > 16384                        # tile kernel splits K
+    # workspace sizing is pure arithmetic: split-K arrival counters (65536 x 4 bytes), then partial sums
+    COUNTERS = 65536 * 4
+    assert lib.nf4hip_gemv_workspace_bytes(16, 128256, 4096) == COUNTERS                  # big N: K is not split
+    assert lib.nf4hip_gemv_workspace_bytes(1, 4096, 4096) == COUNTERS
+    assert lib.nf4hip_gemv_workspace_bytes(4, 8192, 28672) == COUNTERS + 4 * 4 * 8192 * 4  # K split over 4 workgroups
+    assert lib.nf4hip_gemv_workspace_bytes(16, 1024, 4096) > COUNTERS                        # tile kernel splits K
     assert lib.nf4hip_gemm_workspace_bytes(2048, 4096, 4096) == 0
 
 

@@ -1,0 +1,275 @@
+"""Decode-step harness: the caller either side of the 4-bit linear in token generation.
+
+A Llama-architecture decoder (RMSNorm, rotary GQA attention over a static KV cache, SwiGLU) whose
+every ``nn.Linear`` is handed to ``BitsAndBytesLinearQuant4bit`` through ``jit``, and a greedy
+decoding loop whose single-token step is captured in a HIP graph, the way the reference's
+``CUDAGraphTransform`` replays a forward pass (thunder/transforms/cudagraph.py:47-226) over weights
+tagged as static inputs (thunder/transforms/quantization.py:178,186).  Everything that is not a
+linear (norms, rotary embedding, attention, sampling) is plain PyTorch: it is plumbing around the
+path, not part of it.
+
+``fused_projections=True`` builds Q/K/V and gate/up as ONE linear each ([6144, 4096] and
+[28672, 4096] for Llama-3-8B).  NF4 blocks are 64 consecutive elements of a row, so the packed
+weight of the row-concatenated matrix is the concatenation of the packed weights: fusing changes
+no value, only the number of launches and the size of each weight stream.
+"""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+
+@dataclass
+class LlamaConfig:
+    n_layer: int = 32
+    d_model: int = 4096
+    n_head: int = 32
+    n_kv_head: int = 8
+    d_ff: int = 14336
+    vocab: int = 128256
+    rope_theta: float = 500000.0
+    norm_eps: float = 1e-5
+    max_seq: int = 640
+    fused_projections: bool = False
+
+    @property
+    def head_dim(self) -> int:
+        return self.d_model // self.n_head
+
+    @classmethod
+    def llama3_8b(cls, **kw) -> "LlamaConfig":
+        return cls(**kw)
+
+    @classmethod
+    def tiny(cls, **kw) -> "LlamaConfig":
+        base = dict(n_layer=2, d_model=512, n_head=8, n_kv_head=2, d_ff=1024, vocab=1024, max_seq=64)
+        base.update(kw)
+        return cls(**base)
+
+
+def _rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    # x [B, T, heads, hd]; cos/sin [T, 1, hd] (each half repeated): x * cos + rotate_half(x) * sin, in fp32
+    xf = x.float()
+    x1, x2 = xf.chunk(2, dim=-1)
+    return torch.addcmul(xf * cos, torch.cat((-x2, x1), dim=-1), sin).to(x.dtype)
+
+
+class Attention(nn.Module):
+    def __init__(self, cfg: LlamaConfig):
+        super().__init__()
+        self.cfg = cfg
+        hd = cfg.head_dim
+        if cfg.fused_projections:
+            self.qkv_proj = nn.Linear(cfg.d_model, (cfg.n_head + 2 * cfg.n_kv_head) * hd, bias=False)
+        else:
+            self.q_proj = nn.Linear(cfg.d_model, cfg.n_head * hd, bias=False)
+            self.k_proj = nn.Linear(cfg.d_model, cfg.n_kv_head * hd, bias=False)
+            self.v_proj = nn.Linear(cfg.d_model, cfg.n_kv_head * hd, bias=False)
+        self.o_proj = nn.Linear(cfg.n_head * hd, cfg.d_model, bias=False)
+
+    def forward(self, x, pos, cos, sin, mask, kcache, vcache):
+        cfg = self.cfg
+        B, T, _ = x.shape
+        hd, H, Hkv = cfg.head_dim, cfg.n_head, cfg.n_kv_head
+        rep = H // Hkv
+        if cfg.fused_projections:
+            qkv = self.qkv_proj(x)
+            qk, v = qkv[..., : (H + Hkv) * hd], qkv[..., (H + Hkv) * hd:]
+        else:
+            qk = torch.cat((self.q_proj(x), self.k_proj(x)), dim=-1)
+            v = self.v_proj(x)
+        qk = _rope(qk.reshape(B, T, H + Hkv, hd), cos, sin)  # q and k heads rotated in one go
+        kcache.index_copy_(2, pos, qk[:, :, H:].transpose(1, 2))
+        vcache.index_copy_(2, pos, v.reshape(B, T, Hkv, hd).transpose(1, 2))
+        # grouped-query attention without expanding the cache: the `rep` query heads that share a
+        # kv head become extra query rows of that head, row index r * T + t
+        q = qk[:, :, :H].reshape(B, T, Hkv, rep, hd).permute(0, 2, 3, 1, 4).reshape(B, Hkv, rep * T, hd)
+        if T == 1:
+            # one query per head: two small batched matmuls beat a general attention kernel
+            scores = torch.matmul(q, kcache.transpose(-1, -2)).float() * (hd ** -0.5)
+            scores = scores.masked_fill(~mask, float("-inf"))
+            y = torch.matmul(torch.softmax(scores, dim=-1).to(q.dtype), vcache)
+        else:
+            y = F.scaled_dot_product_attention(q, kcache, vcache, attn_mask=mask.repeat(rep, 1))
+        y = y.reshape(B, Hkv, rep, T, hd).permute(0, 3, 1, 2, 4).reshape(B, T, H * hd)
+        return self.o_proj(y)
+
+
+class MLP(nn.Module):
+    def __init__(self, cfg: LlamaConfig):
+        super().__init__()
+        self.cfg = cfg
+        if cfg.fused_projections:
+            self.gate_up_proj = nn.Linear(cfg.d_model, 2 * cfg.d_ff, bias=False)
+        else:
+            self.gate_proj = nn.Linear(cfg.d_model, cfg.d_ff, bias=False)
+            self.up_proj = nn.Linear(cfg.d_model, cfg.d_ff, bias=False)
+        self.down_proj = nn.Linear(cfg.d_ff, cfg.d_model, bias=False)
+
+    def forward(self, x):
+        if self.cfg.fused_projections:
+            gate, up = self.gate_up_proj(x).chunk(2, dim=-1)
+        else:
+            gate, up = self.gate_proj(x), self.up_proj(x)
+        return self.down_proj(F.silu(gate) * up)
+
+
+class Block(nn.Module):
+    def __init__(self, cfg: LlamaConfig):
+        super().__init__()
+        self.norm_1 = nn.RMSNorm(cfg.d_model, eps=cfg.norm_eps)
+        self.attn = Attention(cfg)
+        self.norm_2 = nn.RMSNorm(cfg.d_model, eps=cfg.norm_eps)
+        self.mlp = MLP(cfg)
+
+    def forward(self, x, pos, cos, sin, mask, kcache, vcache):
+        x = x + self.attn(self.norm_1(x), pos, cos, sin, mask, kcache, vcache)
+        return x + self.mlp(self.norm_2(x))
+
+
+class Llama(nn.Module):
+    """``forward(idx [B, T], pos [T], kcache, vcache) -> logits [B, vocab]`` of the LAST position.
+    ``kcache`` / ``vcache``: [n_layer, B, n_kv_head, max_seq, head_dim], updated in place at ``pos``."""
+
+    def __init__(self, cfg: LlamaConfig):
+        super().__init__()
+        self.cfg = cfg
+        self.wte = nn.Embedding(cfg.vocab, cfg.d_model)
+        self.blocks = nn.ModuleList(Block(cfg) for _ in range(cfg.n_layer))
+        self.norm_f = nn.RMSNorm(cfg.d_model, eps=cfg.norm_eps)
+        self.lm_head = nn.Linear(cfg.d_model, cfg.vocab, bias=False)
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32) / cfg.head_dim))
+        ang = torch.outer(torch.arange(cfg.max_seq, dtype=torch.float32), inv).repeat(1, 2)
+        self.register_buffer("rope_cos", ang.cos(), persistent=False)
+        self.register_buffer("rope_sin", ang.sin(), persistent=False)
+        self.register_buffer("key_index", torch.arange(cfg.max_seq), persistent=False)
+
+    def forward(self, idx, pos, kcache, vcache):
+        cos = self.rope_cos.index_select(0, pos)[:, None, :]
+        sin = self.rope_sin.index_select(0, pos)[:, None, :]
+        mask = self.key_index[None, :] <= pos[:, None]  # [T, max_seq]: key s visible to query at pos[t]
+        x = self.wte(idx)
+        for i, blk in enumerate(self.blocks):
+            x = blk(x, pos, cos, sin, mask, kcache[i], vcache[i])
+        return self.lm_head(self.norm_f(x[:, -1:, :])).squeeze(1)
+
+
+def build_llama(cfg: LlamaConfig, device="cuda", dtype=torch.bfloat16, seed: int = 0) -> Llama:
+    """Random-init weights ~ N(0, 0.02), drawn on ``device`` from one seeded generator."""
+    with torch.device("meta"):
+        model = Llama(cfg)
+    model = model.to_empty(device=device)
+    g = torch.Generator(device=device).manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.ndim == 1:
+                p.data = torch.ones_like(p, dtype=dtype)
+            else:
+                w = torch.empty(p.shape, device=device, dtype=torch.float32).normal_(0.0, 0.02, generator=g)
+                p.data = w.to(dtype)
+                del w
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32, device=device) / cfg.head_dim))
+        ang = torch.outer(torch.arange(cfg.max_seq, dtype=torch.float32, device=device), inv).repeat(1, 2)
+        model.rope_cos, model.rope_sin = ang.cos(), ang.sin()
+        model.key_index = torch.arange(cfg.max_seq, device=device)
+    return model.eval().requires_grad_(False)
+
+
+def new_caches(cfg: LlamaConfig, batch: int, device="cuda", dtype=torch.bfloat16):
+    shape = (cfg.n_layer, batch, cfg.n_kv_head, cfg.max_seq, cfg.head_dim)
+    return torch.zeros(shape, device=device, dtype=dtype), torch.zeros(shape, device=device, dtype=dtype)
+
+
+@torch.no_grad()
+def greedy_decode(model, cfg: LlamaConfig, prompt: torch.Tensor, n_new: int, use_graph: bool = True):
+    """Greedy decoding of ``n_new`` tokens after ``prompt`` [B, P].  Returns ``(tokens [B, n_new],
+    stats)`` with the prefill and decode wall times (GPU-synchronised).
+
+    With ``use_graph`` one decode step -- forward, argmax, feeding the token and the position back
+    into their static buffers -- is captured in a HIP graph and replayed; the host only enqueues
+    replays and copies each step's token out, and synchronises once at the end.
+    """
+    B, P = prompt.shape
+    dev = prompt.device
+    assert P + n_new <= cfg.max_seq
+    kcache, vcache = new_caches(cfg, B, dev, model.wte.weight.dtype)
+
+    def sync():
+        if dev.type == "cuda":
+            torch.cuda.synchronize(dev)
+
+    sync()
+    t0 = time.perf_counter()
+    logits = model(prompt, torch.arange(P, device=dev), kcache, vcache)
+    first = logits.argmax(-1, keepdim=True)
+    sync()
+    t_prefill = time.perf_counter() - t0
+
+    tok = first.clone()
+    pos = torch.full((1,), P, device=dev, dtype=torch.long)
+    out = torch.empty(n_new, B, device=dev, dtype=torch.long)
+    out[0] = first[:, 0]
+
+    def step():
+        nxt = model(tok, pos, kcache, vcache).argmax(-1, keepdim=True)
+        tok.copy_(nxt)
+        pos.add_(1)
+
+    graph = None
+    if use_graph and n_new > 1 and dev.type == "cuda":
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            step()  # allocations, workspaces of this stream, lazy library state
+            step()
+            tok.copy_(first)  # roll the state back: the steps above wrote cache rows P, P+1, which
+            pos.fill_(P)      # the real steps rewrite before reading them
+            torch.cuda.synchronize(dev)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                step()
+            tok.copy_(first)  # capture does not execute, but keep the state explicit
+            pos.fill_(P)
+        torch.cuda.current_stream(dev).wait_stream(side)
+
+    sync()
+    t1 = time.perf_counter()
+    for i in range(1, n_new):
+        if graph is not None:
+            graph.replay()
+        else:
+            step()
+        out[i] = tok[:, 0]
+    sync()
+    t_decode = time.perf_counter() - t1
+    stats = {
+        "prefill_s": t_prefill,
+        "decode_s": t_decode,
+        "decode_steps": n_new - 1,
+        "decode_tok_per_s": B * (n_new - 1) / t_decode if n_new > 1 else 0.0,
+        "graph": graph is not None,
+    }
+    return out.t().contiguous(), stats
+
+
+def fuse_state_dict(sd: dict, cfg: LlamaConfig) -> dict:
+    """State dict of the ``fused_projections=True`` model from that of the unfused one: Q/K/V and
+    gate/up weights concatenated along the output dimension."""
+    out = {}
+    for k, v in sd.items():
+        if k.endswith(("k_proj.weight", "v_proj.weight", "up_proj.weight")) and "gate_up" not in k:
+            continue
+        if k.endswith("q_proj.weight"):
+            base = k[: -len("q_proj.weight")]
+            out[base + "qkv_proj.weight"] = torch.cat([v, sd[base + "k_proj.weight"], sd[base + "v_proj.weight"]], dim=0)
+        elif k.endswith("gate_proj.weight"):
+            base = k[: -len("gate_proj.weight")]
+            out[base + "gate_up_proj.weight"] = torch.cat([v, sd[base + "up_proj.weight"]], dim=0)
+        else:
+            out[k] = v
+    return out

@@ -26,6 +26,12 @@ SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
 # (the cheaper "scale the partial sum" arithmetic drifts from it like sqrt(K)); the 5..16-row tile
 # kernel has no such variant, so those calls go to the prefill kernel, which is exact by construction.
 EXACT_K = 16384
+# From this many rows of x on, HIP dequantize followed by the dense library GEMM is faster than
+# the fused GEMM kernel (measured on MI355X at every Llama-3-8B projection shape: the fused kernel
+# re-expands the weight tile once per 128 rows of x and reaches ~0.5 PFLOP/s, the library GEMM
+# 1.1-1.5 PFLOP/s and the dequantize kernel runs at HBM speed).  Raise it to force the fused,
+# allocation-free kernel.
+DENSE_ROUTE_MIN_M = 17
 
 _DTYPE_CODE = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32}
 
@@ -214,7 +220,9 @@ def _gemv_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 
 def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape) -> str:
-    """Which kernel serves this call: ``"gemv"``, ``"gemm"`` or ``"dequant+linear"``.
+    """Which kernel serves this call: ``"gemv"``, ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP
+    dequantize, then the dense library GEMM, because that is the faster of the two for many rows
+    of x) or ``"dequant+linear"`` (the same two steps, for dtypes and shapes no fused kernel takes).
 
     Mirrors bitsandbytes.matmul_4bit: the fused single-row kernel when the shape allows, else
     dequantize followed by a dense matmul.
@@ -238,7 +246,7 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "dequant+linear"
     if M <= 16 and K % 512 == 0 and K <= EXACT_K:
         return "gemv"  # MFMA tile kernel
-    return "gemm"
+    return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M else "gemm"
 
 
 def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> torch.Tensor:
@@ -251,7 +259,7 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
     assert x.shape[-1] == K, f"{x.shape=}, rhs {shape=}"
     _require_gpu(x, qweight, quant_map, bias)
     route = fused_route(x, bias, blocksize, dtype, shape)
-    if route == "dequant+linear":
+    if route in ("dequant+linear", "dequant+gemm"):
         w = dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape).to(x.dtype)
         return torch.nn.functional.linear(x, w, bias)
 

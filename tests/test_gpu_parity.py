@@ -253,17 +253,32 @@ def test_gemv_repeatable_and_workspace_reuse(ta, oracle):
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
+@pytest.fixture
+def fused_gemm(ta, monkeypatch):
+    """Route every M > 16 call to the fused GEMM kernel (the default router prefers HIP dequantize
+    + the dense library GEMM from 17 rows on)."""
+    monkeypatch.setattr(ta.functional, "DENSE_ROUTE_MIN_M", 1 << 30)
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 128, 64), (512, 1024, 4096), (2048, 4096, 4096)])
+def test_dense_route(ta, oracle, M, N, K):
+    """Default route for many rows of x: nf4hip_dequantize + dense GEMM."""
+    _sync_print(f"dequant+gemm M={M} N={N} K={K}")
+    assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, 64, torch.bfloat16, (N, K)) == "dequant+gemm"
+    _matmul_case(ta, oracle, M, N, K, seed=M + N + K + 1)
+
+
 @pytest.mark.parametrize(
     "M,N,K",
     [(17, 128, 64), (32, 130, 128), (128, 128, 512), (100, 100, 1344), (300, 384, 1024), (512, 1024, 4096), (257, 4096, 1024)],
 )
-def test_gemm_shapes(ta, oracle, M, N, K):
+def test_gemm_shapes(ta, oracle, M, N, K, fused_gemm):
     _sync_print(f"gemm M={M} N={N} K={K}")
     assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, 64, torch.bfloat16, (N, K)) == "gemm"
     _matmul_case(ta, oracle, M, N, K, seed=M + N + K)
 
 
-def test_gemm_recovers_dequantized_weight_bit_exact(ta, oracle):
+def test_gemm_recovers_dequantized_weight_bit_exact(ta, oracle, fused_gemm):
     """x = identity makes every output a single product 1.0 * w: the fused kernel's in-LDS
     dequantisation must equal nf4hip_dequantize bit for bit."""
     _sync_print("gemm identity")
@@ -276,7 +291,7 @@ def test_gemm_recovers_dequantized_weight_bit_exact(ta, oracle):
     assert torch.equal(y.cpu().t().contiguous().view(torch.int16), deq.view(torch.int16))
 
 
-def test_gemm_bias_nested_blocksize(ta, oracle):
+def test_gemm_bias_nested_blocksize(ta, oracle, fused_gemm):
     _sync_print("gemm bias/nested/blocksize")
     _matmul_case(ta, oracle, 64, 256, 1024, bias=True, seed=1)
     _matmul_case(ta, oracle, 64, 256, 1024, nested=True, seed=2)

@@ -13,6 +13,8 @@ Prints ONE JSON line:
               timed group by group): algorithmic bytes per launch / average launch duration, from
               HIP events recorded inside the timed region on the launch stream, against the
               8 TB/s HBM peak; config.kernels lists all three
+  config.decode = BASELINE config 4 (full Llama-3-8B architecture, greedy decode, batch 1 and 8)
+              run after the timed region: decode tokens/s, the second half of the metric
   cpu_baseline = the reference's CPU-side route (torch-eager dequantize + linear, restated in
               oracle/nf4_oracle.py) timed on this box's host cores on a bounded sample
 """
@@ -48,6 +50,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU baseline sample (0 disables)")
+    ap.add_argument("--decode-tokens", type=int, default=128,
+                    help="tokens of the Llama-3-8B greedy decode that follows the GEMV pass (0 disables)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only; --gpus {args.gpus} is not supported "
@@ -185,10 +189,44 @@ def main() -> int:
         },
     }
 
+    if args.decode_tokens > 1:
+        del weights, xs, outs, ws
+        torch.cuda.empty_cache()
+        result["config"]["decode"] = llama_decode(torch, ta, args.decode_tokens)
     if args.cpu_seconds > 0:
         result["cpu_baseline"] = cpu_baseline(torch, args.cpu_seconds)
     print(json.dumps(result))
     return 0
+
+
+def llama_decode(torch, ta, n_new: int) -> dict:
+    """BASELINE config 4, outside the timed region of the GEMV metric: the full Llama-3-8B
+    architecture with random-init weights, every nn.Linear NF4-quantized through the transform,
+    greedy decode from random prompts of length 512 at batch 1 and 8, decode step replayed from a
+    HIP graph, Q/K/V and gate/up as one linear each."""
+    D = importlib.import_module("lightning-thunder_amd.decode")
+    dev = torch.device("cuda:0")
+    cfg = D.LlamaConfig.llama3_8b(fused_projections=True)
+    model = D.build_llama(cfg, device=dev, seed=4000)
+    jm = ta.jit(model, transforms=[ta.BitsAndBytesLinearQuant4bit()])
+    nweights = sum(m.weight.numel() for m in model.modules() if isinstance(m, torch.nn.Linear))
+    out = {
+        "model": "Llama-3-8B architecture (32 layers, d 4096, 32q/8kv heads, FFN 14336, vocab 128256), random init, "
+                 "all 161 linears NF4 (QKV and gate/up fused), prompt 512, greedy, HIP-graph decode step",
+        "new_tokens": n_new,
+        "linear_weight_bytes_per_token": int(nweights * 0.5625),
+        "hbm_bound_tok_per_s_batch1": round(HBM_PEAK_GBS * 1e9 / (nweights * 0.5625), 1),
+    }
+    for B in (1, 8):
+        g = torch.Generator(device=dev).manual_seed(4000 + B)
+        prompt = torch.randint(0, cfg.vocab, (B, 512), generator=g, device=dev)
+        _, st = D.greedy_decode(jm, cfg, prompt, n_new=n_new, use_graph=True)
+        out[f"batch{B}"] = {
+            "decode_tok_per_s": round(st["decode_tok_per_s"], 1),
+            "ms_per_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
+            "prefill_ms": round(st["prefill_s"] * 1e3, 1),
+        }
+    return out
 
 
 def cpu_baseline(torch, budget_s: float) -> dict:

@@ -74,77 +74,74 @@ __device__ __forceinline__ void load8(const void* w, int dtype, int64_t e0, int6
     }
 }
 
+// A workgroup covers Q_SLOTS consecutive spans of THREADS * 8 elements (a span holds whole
+// quantisation blocks); a thread owns 8 consecutive elements of each span.  The loads of all spans
+// are in flight before the first reduction.
+constexpr int Q_SLOTS = 4;
+
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void quantize_kernel(const void* __restrict__ w, int dtype, int64_t n,
                                                            int block_log2, uint8_t* __restrict__ packed,
                                                            float* __restrict__ absmax) {
-    __shared__ float wave_max[THREADS / 64];
+    __shared__ float wave_max[Q_SLOTS][THREADS / 64];
     const int tid = threadIdx.x;
-    const int64_t e0 = ((int64_t)blockIdx.x * THREADS + tid) * 8;
     const int group = 1 << (block_log2 - 3);  // lanes per quantisation block
-
-    float v[8];
-    load8(w, dtype, e0, n, v);
-    float m = 0.0f;
+    float v[Q_SLOTS][8];
+    float m[Q_SLOTS];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
-
-    // max over the lanes of one quantisation block
+    for (int c = 0; c < Q_SLOTS; ++c) {
+        const int64_t e0 = (((int64_t)blockIdx.x * Q_SLOTS + c) * THREADS + tid) * 8;
+        load8(w, dtype, e0, n, v[c]);
+    }
     const int in_wave = group < 64 ? group : 64;
-    for (int off = 1; off < in_wave; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+#pragma unroll
+    for (int c = 0; c < Q_SLOTS; ++c) {
+        float mm = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mm = fmaxf(mm, fabsf(v[c][j]));
+        // max over the lanes of one quantisation block
+        for (int off = 1; off < in_wave; off <<= 1) mm = fmaxf(mm, __shfl_xor(mm, off, 64));
+        m[c] = mm;
+    }
     if (group > 64) {  // uniform branch: blocks of 1024, 2048 or 4096 elements span several waves
-        if ((tid & 63) == 0) wave_max[tid >> 6] = m;
+#pragma unroll
+        for (int c = 0; c < Q_SLOTS; ++c)
+            if ((tid & 63) == 0) wave_max[c][tid >> 6] = m[c];
         __syncthreads();
         const int waves = group >> 6;
         const int first = (tid >> 6) & ~(waves - 1);
-        for (int j = 0; j < waves; ++j) m = fmaxf(m, wave_max[first + j]);
-    }
-
-    if (e0 >= n) return;
-    if ((tid & (group - 1)) == 0) absmax[e0 >> block_log2] = m;
-
-    const float inv = __fdiv_rn(1.0f, m);
-    uint32_t word = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t hi = nf4_code(__fmul_rn(v[2 * j], inv));
-        const uint32_t lo = nf4_code(__fmul_rn(v[2 * j + 1], inv));
-        word |= ((hi << 4) | lo) << (8 * j);
+        for (int c = 0; c < Q_SLOTS; ++c)
+            for (int j = 0; j < waves; ++j) m[c] = fmaxf(m[c], wave_max[c][first + j]);
     }
-    if (e0 + 8 <= n) {
-        reinterpret_cast<uint32_t*>(packed)[e0 / 8] = word;
-    } else {
-        const int64_t nbytes = (n + 1) / 2;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (e0 / 2 + j < nbytes) packed[e0 / 2 + j] = (uint8_t)(word >> (8 * j));
+    for (int c = 0; c < Q_SLOTS; ++c) {
+        const int64_t e0 = (((int64_t)blockIdx.x * Q_SLOTS + c) * THREADS + tid) * 8;
+        if (e0 >= n) continue;
+        if ((tid & (group - 1)) == 0) absmax[e0 >> block_log2] = m[c];
+        const float inv = __fdiv_rn(1.0f, m[c]);
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t hi = nf4_code(__fmul_rn(v[c][2 * j], inv));
+            const uint32_t lo = nf4_code(__fmul_rn(v[c][2 * j + 1], inv));
+            word |= ((hi << 4) | lo) << (8 * j);
+        }
+        if (e0 + 8 <= n) {
+            reinterpret_cast<uint32_t*>(packed)[e0 / 8] = word;
+        } else {
+            const int64_t nbytes = (n + 1) / 2;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (e0 / 2 + j < nbytes) packed[e0 / 2 + j] = (uint8_t)(word >> (8 * j));
+        }
     }
 }
 
-template <bool NESTED>
-__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ packed,
-                                                         const float* __restrict__ absmax, NestedAbsmax nq,
-                                                         const float* __restrict__ lut16, int64_t n, int block_log2,
-                                                         void* __restrict__ out, int out_dtype) {
-    __shared__ float lut[16];
-    const int tid = threadIdx.x;
-    if (tid < 16) lut[tid] = lut16[tid];
-    __syncthreads();
-    const int64_t e0 = ((int64_t)blockIdx.x * 256 + tid) * 8;
-    if (e0 >= n) return;
-
-    const int64_t blk = e0 >> block_log2;
-    const float s = NESTED ? nested_absmax(nq, blk) : absmax[blk];
+// Eight elements of output from one 32-bit word of codes.
+__device__ __forceinline__ void dequant8_store(uint32_t word, float s, const float* lut, void* out, int out_dtype,
+                                               int64_t e0, int64_t n) {
     const bool full = e0 + 8 <= n;
-    uint32_t word;
-    if (full) {
-        word = reinterpret_cast<const uint32_t*>(packed)[e0 / 8];
-    } else {
-        const int64_t nbytes = (n + 1) / 2;
-        word = 0;
-        for (int j = 0; j < 4; ++j)
-            if (e0 / 2 + j < nbytes) word |= (uint32_t)packed[e0 / 2 + j] << (8 * j);
-    }
     float v[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -178,6 +175,45 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
             for (int j = 0; j < 8; ++j)
                 if (e0 + j < n) o[e0 + j] = (uint16_t)h[j];
         }
+    }
+}
+
+// A workgroup covers DQ_SLOTS consecutive spans of 2048 elements; a thread owns 8 consecutive
+// elements of each span, so every load and store of a wave is contiguous, and the loads of all
+// spans are in flight before the first store.
+constexpr int DQ_SLOTS = 4;
+
+template <bool NESTED>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ packed,
+                                                         const float* __restrict__ absmax, NestedAbsmax nq,
+                                                         const float* __restrict__ lut16, int64_t n, int block_log2,
+                                                         void* __restrict__ out, int out_dtype) {
+    __shared__ float lut[16];
+    const int tid = threadIdx.x;
+    if (tid < 16) lut[tid] = lut16[tid];
+    uint32_t word[DQ_SLOTS];
+    float s[DQ_SLOTS];
+#pragma unroll
+    for (int c = 0; c < DQ_SLOTS; ++c) {
+        const int64_t e0 = (((int64_t)blockIdx.x * DQ_SLOTS + c) * 256 + tid) * 8;
+        word[c] = 0;
+        s[c] = 0.0f;
+        if (e0 >= n) continue;
+        const int64_t blk = e0 >> block_log2;
+        s[c] = NESTED ? nested_absmax(nq, blk) : absmax[blk];
+        if (e0 + 8 <= n) {
+            word[c] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(packed) + e0 / 8);
+        } else {
+            const int64_t nbytes = (n + 1) / 2;
+            for (int j = 0; j < 4; ++j)
+                if (e0 / 2 + j < nbytes) word[c] |= (uint32_t)packed[e0 / 2 + j] << (8 * j);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < DQ_SLOTS; ++c) {
+        const int64_t e0 = (((int64_t)blockIdx.x * DQ_SLOTS + c) * 256 + tid) * 8;
+        if (e0 < n) dequant8_store(word[c], s[c], lut, out, out_dtype, e0, n);
     }
 }
 
@@ -242,11 +278,11 @@ hipError_t launch_quantize(const void* w, int w_dtype, int64_t n, int block_log2
                            hipStream_t stream) {
     if (n == 0) return hipSuccess;
     if (block_log2 == 12) {
-        const int64_t grid = (n + 4095) / 4096;
+        const int64_t grid = (n + 4096 * Q_SLOTS - 1) / (4096 * Q_SLOTS);
         hipLaunchKernelGGL(quantize_kernel<512>, dim3((unsigned)grid), dim3(512), 0, stream, w, w_dtype, n, block_log2,
                            packed, absmax);
     } else {
-        const int64_t grid = (n + 2047) / 2048;
+        const int64_t grid = (n + 2048 * Q_SLOTS - 1) / (2048 * Q_SLOTS);
         hipLaunchKernelGGL(quantize_kernel<256>, dim3((unsigned)grid), dim3(256), 0, stream, w, w_dtype, n, block_log2,
                            packed, absmax);
     }
@@ -257,7 +293,7 @@ hipError_t launch_dequantize(const uint8_t* packed, const float* absmax, const N
                              const float* lut16, int64_t n, int block_log2, void* out, int out_dtype,
                              hipStream_t stream) {
     if (n == 0) return hipSuccess;
-    const int64_t grid = (n + 2047) / 2048;
+    const int64_t grid = (n + 2048 * DQ_SLOTS - 1) / (2048 * DQ_SLOTS);
     if (nested.q)
         hipLaunchKernelGGL(dequantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, stream, packed, absmax, nested,
                            lut16, n, block_log2, out, out_dtype);

@@ -30,16 +30,18 @@ class HIPGraphRunner:
         entry = self.cache.get(key)
         if entry is None:
             static_in = [a.clone() if isinstance(a, torch.Tensor) else a for a in args]
+            # warm-up and capture run on ONE side stream: per-stream state (the gemv workspace of
+            # that stream, library handles) exists before the capture and is the one the graph uses
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 for _ in range(self.warmup):  # allocations, lazy library state, workspaces
                     self.fn(*static_in)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    static_out = self.fn(*static_in)
             torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                static_out = self.fn(*static_in)
             entry = (graph, static_in, static_out)
             self.cache[key] = entry
         graph, static_in, static_out = entry

@@ -339,3 +339,28 @@ def test_full_size_properties(ta):
     big = ta.matmul_nf4(torch.cat([x1, x2]).repeat(128, 1), qw, None, absmax, code, 64, torch.bfloat16, (N, K)).float()
     torch.testing.assert_close(big[0], ref[0], rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(big[254], ref[0], rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("N,K", [(8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672)])
+def test_llama70b_shapes_double_quant(ta, N, K):
+    """Llama-3-70B projection shapes with 8-bit double-quantized absmax (nested blocksize 256 plus
+    offset), M in {1, 16, 2048}, at full size: every route against a float64-accumulated matmul over
+    the HIP-dequantized weight (itself pinned bit-exact against the oracle at small sizes), and the
+    fused kernels' nested path against their fp32-absmax path on the reconstructed absmax."""
+    _sync_print(f"70B double-quant N={N} K={K}")
+    g = torch.Generator(device=DEV).manual_seed(5000 + N + K)
+    w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    qw, absmax, code = ta.quantize_nf4(w)
+    nested = ta.compress_absmax(absmax)
+    absmax_rec = ta.reconstruct_absmax(nested)
+    deq = ta.dequantize_nf4(qw, nested, code, 64, torch.bfloat16, (N, K))
+    assert torch.equal(deq, ta.dequantize_nf4(qw, absmax_rec, code, 64, torch.bfloat16, (N, K)))
+    rows = torch.randint(0, N, (64,), generator=g, device=DEV)
+    for M in (1, 16, 2048):
+        x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+        y = ta.matmul_nf4(x, qw, None, nested, code, 64, torch.bfloat16, (N, K))
+        ref = x.double() @ deq[rows].double().t()
+        torch.testing.assert_close(y[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
+        if M <= 16:
+            y2 = ta.matmul_nf4(x, qw, None, absmax_rec, code, 64, torch.bfloat16, (N, K))
+            assert torch.equal(y, y2)

@@ -406,3 +406,30 @@ def test_lut_rounding_option(ta, dev, oracle):
     jm = ta.jit(mlp, transforms=[ta.BitsAndBytesLinearQuant4bit(lut_rounding="dtype")], executors=(ta.get_hip_nf4_executor(),))
     code = jm.get_parameter("0.weight.code").cpu()
     assert torch.equal(code, oracle.nf4_lut().to(torch.bfloat16).float()) and not torch.equal(code, oracle.nf4_lut())
+
+
+@pytest.mark.gpu
+def test_reduce_overhead_plugin_graph_replay_equals_eager(ta):
+    """``compile(model, plugins=["quantize-int4", "reduce-overhead"])``: the forward pass replays from
+    a HIP graph.  Every replay (with eager work and synchronisations in between) must reproduce the
+    eager result of the same jitted module for the input of that call."""
+    import torch
+
+    print("graph replay of a quantized MLP", flush=True)
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(512, 1024, bias=False), torch.nn.GELU(), torch.nn.Linear(1024, 512, bias=True))
+    model = model.to(dev, torch.bfloat16).requires_grad_(False)
+    eager = ta.compile(model, plugins="quantize-int4")
+    graphed = ta.compile(model, plugins=["quantize-int4", "reduce-overhead"])
+    for i in range(6):
+        g = torch.Generator(device=dev).manual_seed(100 + i)
+        x = torch.randn(4, 512, generator=g, device=dev).to(torch.bfloat16)
+        want = eager(x)
+        got = graphed(x).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(want, got), f"replay {i}"
+        _ = (want.float() @ want.float().t()).sum().item()  # unrelated eager work between replays
+    # a new input signature is a new capture
+    x = torch.randn(1, 512, device=dev).to(torch.bfloat16)
+    assert torch.equal(eager(x), graphed(x))

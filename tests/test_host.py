@@ -433,3 +433,19 @@ def test_reduce_overhead_plugin_graph_replay_equals_eager(ta):
     # a new input signature is a new capture
     x = torch.randn(1, 512, device=dev).to(torch.bfloat16)
     assert torch.equal(eager(x), graphed(x))
+
+
+def test_thunder_adapter_is_import_guarded():
+    """Where Thunder is not installed the adapter module imports fine and ``install()`` says what is
+    missing; where it is installed, the returned class derives from the reference's transform."""
+    import importlib
+
+    adapter = importlib.import_module("lightning-thunder_amd.thunder_adapter")
+    try:
+        import thunder  # noqa: F401
+    except ImportError:
+        with pytest.raises(ImportError, match="lightning-thunder"):
+            adapter.install()
+    else:
+        cls = adapter.install()
+        assert cls.executor.name == adapter.EXECUTOR_NAME

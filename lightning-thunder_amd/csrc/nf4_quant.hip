@@ -18,26 +18,37 @@
 namespace nf4 {
 namespace {
 
-// Decision thresholds of the NF4 code (midpoints of adjacent code values) as the exact fp32
-// bit patterns a C compiler produces for the literals -0.8480964004993439f ... 0.8614784181118011f.
-__device__ __forceinline__ float thr(int j) {
-    constexpr uint32_t T[15] = {0xBF591CD9u, 0xBF1C5270u, 0xBEEB8480u, 0xBEADEA76u, 0xBE703CECu,
-                                0xBE0D38BCu, 0xBD3A7871u, 0x3D22FAFFu, 0x3DF64863u, 0x3E5067E0u,
-                                0x3E9582D4u, 0x3EC753F9u, 0x3F006D03u, 0x3F248DAFu, 0x3F5C89D9u};
-    return __uint_as_float(T[j]);
-}
+// The decision thresholds of the NF4 code (midpoints of adjacent code values) appear below as the
+// exact fp32 bit patterns a C compiler produces for the literals -0.8480964004993439f ...
+// 0.8614784181118011f (four of the midpoints are exact ties in fp32).
+// code = number of thresholds strictly below s (NaN -> 0).
+//
+// [-1, 1] is cut into 32 cells of width 1/16; adjacent thresholds are at least 0.08 apart, so a cell
+// holds at most one of them, and code = (thresholds below the cell) + (s > the cell's threshold).
+// Lane c of a wave keeps cell c & 31 in two registers and every lane fetches its cell with
+// ds_bpermute: 6 VALU operations per element instead of a 4-level tree of compares and selects.
+// The cell index comes from fma(s, 16, 16) rounded to fp32; a value within rounding distance of a
+// cell boundary may land in the neighbouring cell, which gives the same code because no threshold
+// is closer than 1.6e-3 to a boundary.
+__device__ __constant__ const uint32_t CELL_THR[32] = {
+    0x7F800000u, 0x7F800000u, 0xBF591CD9u, 0x7F800000u, 0x7F800000u, 0x7F800000u, 0xBF1C5270u, 0x7F800000u,
+    0xBEEB8480u, 0x7F800000u, 0xBEADEA76u, 0x7F800000u, 0xBE703CECu, 0xBE0D38BCu, 0x7F800000u, 0xBD3A7871u,
+    0x3D22FAFFu, 0x3DF64863u, 0x7F800000u, 0x3E5067E0u, 0x3E9582D4u, 0x7F800000u, 0x3EC753F9u, 0x7F800000u,
+    0x3F006D03u, 0x7F800000u, 0x3F248DAFu, 0x7F800000u, 0x7F800000u, 0x3F5C89D9u, 0x7F800000u, 0x7F800000u};
+__device__ __constant__ const uint32_t CELL_BASE[32] = {0, 0, 0,  1,  1,  1,  1,  2,  2,  3,  3,  4,  4,  5,  6,  6,
+                                                        7, 8, 9,  9,  10, 11, 11, 12, 12, 13, 13, 14, 14, 14, 15, 15};
 
-// code = number of thresholds strictly below s (NaN -> 0), as a 4-level binary search.
-__device__ __forceinline__ uint32_t nf4_code(float s) {
-    const bool b3 = s > thr(7);
-    const float t2 = b3 ? thr(11) : thr(3);
-    const bool b2 = s > t2;
-    const float t1 = b3 ? (b2 ? thr(13) : thr(9)) : (b2 ? thr(5) : thr(1));
-    const bool b1 = s > t1;
-    const float t0 = b3 ? (b2 ? (b1 ? thr(14) : thr(12)) : (b1 ? thr(10) : thr(8)))
-                        : (b2 ? (b1 ? thr(6) : thr(4)) : (b1 ? thr(2) : thr(0)));
-    const bool b0 = s > t0;
-    return (uint32_t)b3 * 8u + (uint32_t)b2 * 4u + (uint32_t)b1 * 2u + (uint32_t)b0;
+struct CodeCells {
+    uint32_t thr;   // CELL_THR[lane & 31]
+    uint32_t base;  // CELL_BASE[lane & 31]
+};
+
+__device__ __forceinline__ uint32_t nf4_code(float s, const CodeCells& cc) {
+    // NaN and negatives convert to 0, values above 31 are clamped
+    const uint32_t cell = min((uint32_t)__builtin_fmaf(s, 16.0f, 16.0f), 31u);
+    const float t = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute((int)(cell << 2), (int)cc.thr));
+    const uint32_t b = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(cell << 2), (int)cc.base);
+    return b + (s > t ? 1u : 0u);
 }
 
 __device__ __forceinline__ float load_elem(const void* w, int dtype, int64_t i) {
@@ -86,6 +97,7 @@ __global__ __launch_bounds__(THREADS) void quantize_kernel(const void* __restric
     __shared__ float wave_max[Q_SLOTS][THREADS / 64];
     const int tid = threadIdx.x;
     const int group = 1 << (block_log2 - 3);  // lanes per quantisation block
+    const CodeCells cc = {CELL_THR[tid & 31], CELL_BASE[tid & 31]};
     float v[Q_SLOTS][8];
     float m[Q_SLOTS];
 #pragma unroll
@@ -117,16 +129,18 @@ __global__ __launch_bounds__(THREADS) void quantize_kernel(const void* __restric
 #pragma unroll
     for (int c = 0; c < Q_SLOTS; ++c) {
         const int64_t e0 = (((int64_t)blockIdx.x * Q_SLOTS + c) * THREADS + tid) * 8;
-        if (e0 >= n) continue;
-        if ((tid & (group - 1)) == 0) absmax[e0 >> block_log2] = m[c];
+        // every lane computes its codes (the cell lookup reads other lanes' registers, so no lane
+        // may drop out before it); lanes past the end hold zeros and store nothing
         const float inv = __fdiv_rn(1.0f, m[c]);
         uint32_t word = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const uint32_t hi = nf4_code(__fmul_rn(v[c][2 * j], inv));
-            const uint32_t lo = nf4_code(__fmul_rn(v[c][2 * j + 1], inv));
+            const uint32_t hi = nf4_code(__fmul_rn(v[c][2 * j], inv), cc);
+            const uint32_t lo = nf4_code(__fmul_rn(v[c][2 * j + 1], inv), cc);
             word |= ((hi << 4) | lo) << (8 * j);
         }
+        if (e0 >= n) continue;
+        if ((tid & (group - 1)) == 0) absmax[e0 >> block_log2] = m[c];
         if (e0 + 8 <= n) {
             reinterpret_cast<uint32_t*>(packed)[e0 / 8] = word;
         } else {

@@ -40,6 +40,8 @@ constexpr int PART_BYTES = 16 * 1024;  // per-(row, wave, m) partial sums of one
 constexpr int SMEM_BYTES = GEMV_TABLE_BYTES + PART_BYTES;
 constexpr int LOAD_K = 512;            // k covered by one wave-wide 16-byte load (16 segments of 32)
 constexpr int FLAG_OFFSET = GEMV_TABLE_BYTES + PART_BYTES - 16;
+constexpr int MAP_BYTES = 1024;         // nested absmax only: the 256-entry map, taken from the end of the partial sums
+constexpr int MAP_OFFSET = FLAG_OFFSET - MAP_BYTES;
 
 struct QuadPlan {
     int waves_k;          // waves of a workgroup along K
@@ -128,14 +130,19 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 xr[c][4 * q + 0] = v.x; xr[c][4 * q + 1] = v.y; xr[c][4 * q + 2] = v.z; xr[c][4 * q + 3] = v.w;
             }
 
+        // sq: absmax of the lane's block; nested: its 8-bit code (resolved through the LDS copy of
+        // the map when the slot is consumed, so that issuing a load never waits for another) and
+        // s2 the second-level absmax
         uint4 wq[U][CPW];
         float sq[U][CPW];
+        float s2[NESTED ? U : 1][CPW];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int c = 0; c < CPW; ++c) {
                 wq[u][c] = make_uint4(0, 0, 0, 0);
                 sq[u][c] = 0.0f;
+                if (NESTED) s2[u][c] = 0.0f;
             }
         // group i of this wave is g_begin + rg + i * step; its rows are 4 * group + ri
         auto issue = [&](int u, int i) {
@@ -147,7 +154,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                     const int64_t e = e0 + c * LOAD_K;
                     wq[u][c] = load16_stream(a.packed + (e >> 1));
                     const int64_t blk = e >> a.block_log2;
-                    sq[u][c] = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
+                    if (NESTED) {
+                        sq[u][c] = __uint_as_float((uint32_t)a.nested.q[blk]);
+                        s2[u][c] = a.nested.absmax2[blk >> a.nested.nested_log2];
+                    } else {
+                        sq[u][c] = a.absmax[blk];
+                    }
                 }
         };
         // get the weight stream going before anything else happens
@@ -160,6 +172,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 build_pair_table_f32(smem, lut_mine, lane, wave);
             else
                 build_pair_table(smem, lut_mine, lane, wave);
+            if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
             table_built = true;
         }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
@@ -171,7 +184,10 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
 #pragma unroll
                 for (int c = 0; c < CPW; ++c) {
                     const uint32_t d[4] = {wq[u][c].x, wq[u][c].y, wq[u][c].z, wq[u][c].w};
-                    const float s = sq[u][c];
+                    float s = sq[u][c];
+                    if (NESTED)
+                        s = __fadd_rn(__fmul_rn(reinterpret_cast<const float*>(smem + MAP_OFFSET)[__float_as_uint(s)], s2[u][c]),
+                                      a.nested.offset);
                     uint32_t pr[16];
 #pragma unroll
                     for (int q = 0; q < 4; ++q)
@@ -214,6 +230,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                     for (int c = 0; c < CPW; ++c) {
                         wq[u][c] = make_uint4(0, 0, 0, 0);
                         sq[u][c] = 0.0f;
+                        if (NESTED) s2[u][c] = 0.0f;
                     }
                 }
                 const float total = reduce_rows(tot, lane);  // lanes 0..15: row 2*b3+b2 of the group, x row ri
@@ -282,7 +299,7 @@ int quad_splits(int64_t K) {
     return (int)((nwk + GEMV_WAVES - 1) / GEMV_WAVES);
 }
 
-QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots) {
+QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested) {
     QuadPlan p;
     p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
     const int64_t wave_k = (int64_t)pick_cpw(K) * LOAD_K;
@@ -291,7 +308,8 @@ QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots) 
     p.waves_k = (nwk + p.splits - 1) / p.splits;
     p.row_groups = GEMV_WAVES / p.waves_k;
     const int groups = (int)((N + 3) / 4);
-    const int cap = ((PART_BYTES - 64) / (4 * p.waves_k * M * 4)) / p.row_groups * p.row_groups;
+    const int part_bytes = PART_BYTES - 64 - (nested ? MAP_BYTES : 0);
+    const int cap = (part_bytes / (4 * p.waves_k * M * 4)) / p.row_groups * p.row_groups;
     int bands_target = slots / p.splits;
     if (bands_target < 1) bands_target = 1;
     // one task per resident workgroup if its partial sums fit in LDS, else 2, 3, ... balanced rounds
@@ -327,7 +345,7 @@ hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_
     constexpr int UMAX = 8 / CPW;
     if constexpr (UMAX >= 8)
         if (cnt >= 8) return launch_u<CPW, 8, NESTED>(a, p, grid, stream);
-    if constexpr (UMAX >= 4)
+    if constexpr (UMAX >= 4 && !(NESTED && CPW == 2))  // nested: one more register per load in flight
         if (cnt >= 4) return launch_u<CPW, 4, NESTED>(a, p, grid, stream);
     return launch_u<CPW, 2, NESTED>(a, p, grid, stream);
 }
@@ -365,7 +383,7 @@ hipError_t gemv_quad_setup() {
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {
     int slots = 2 * cus;
     if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
-    const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots);
+    const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
     const int grid = p.ntasks < slots ? p.ntasks : slots;
     return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
 }

@@ -46,6 +46,8 @@ constexpr int PART_BYTES = 16 * 1024;  // per-(row, chunk, m) partial sums of on
 constexpr int SMEM_BYTES = GEMV_TABLE_BYTES + PART_BYTES;
 constexpr int CHUNK_K = 2048;          // k covered by one wave-wide 16-byte load
 constexpr int FLAG_OFFSET = GEMV_TABLE_BYTES + PART_BYTES - 16;
+constexpr int MAP_BYTES = 1024;         // nested absmax only: the 256-entry map, taken from the end of the partial sums
+constexpr int MAP_OFFSET = FLAG_OFFSET - MAP_BYTES;
 
 struct RowsPlan {
     int chunks;         // k chunks handled by one workgroup (waves along K)
@@ -142,12 +144,17 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                 xr[m][4 * q + 0] = v.x; xr[m][4 * q + 1] = v.y; xr[m][4 * q + 2] = v.z; xr[m][4 * q + 3] = v.w;
             }
 
+        // sq: absmax of the lane's block; nested: its 8-bit code (resolved through the LDS copy of
+        // the map when the slot is consumed, so that issuing a load never waits for another) and
+        // s2 the second-level absmax
         uint4 wq[U];
         float sq[U];
+        float s2[NESTED ? U : 1];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             wq[u] = make_uint4(0, 0, 0, 0);
             sq[u] = 0.0f;
+            if (NESTED) s2[u] = 0.0f;
         }
         // row i of this wave is r_begin + rl + i * step
         auto issue = [&](int u, int i) {
@@ -160,7 +167,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                         blk = (((int64_t)row * K + kchunk) >> a.block_log2) + (klane >> a.block_log2);
                     else
                         blk = ((int64_t)row * K + kchunk + klane) >> a.block_log2;
-                    sq[u] = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
+                    if (NESTED) {
+                        sq[u] = __uint_as_float((uint32_t)a.nested.q[blk]);
+                        s2[u] = a.nested.absmax2[blk >> a.nested.nested_log2];
+                    } else {
+                        sq[u] = a.absmax[blk];
+                    }
                 }
             };
         // get the weight stream going before anything else happens
@@ -173,6 +185,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                 build_pair_table_f32(smem, lut_mine, lane, wave);
             else
                 build_pair_table(smem, lut_mine, lane, wave);
+            if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
             table_built = true;
         }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
@@ -183,12 +196,16 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const uint32_t d[4] = {wq[u].x, wq[u].y, wq[u].z, wq[u].w};
-                    const float s = sq[u];
+                    float s = sq[u];
+                    if (NESTED)
+                        s = __fadd_rn(__fmul_rn(reinterpret_cast<const float*>(smem + MAP_OFFSET)[__float_as_uint(s)], s2[u]),
+                                      a.nested.offset);
                     if (i0 + u + U < cnt) {
                         issue(u, i0 + u + U);
                     } else {  // slot is dead from here on; say so, or the compiler keeps copies alive
                         wq[u] = make_uint4(0, 0, 0, 0);
                         sq[u] = 0.0f;
+                        if (NESTED) s2[u] = 0.0f;
                     }
                     uint32_t pr[16];
 #pragma unroll
@@ -290,14 +307,15 @@ int rows_splits(int64_t K) {
     return (int)((nch + GEMV_WAVES - 1) / GEMV_WAVES);
 }
 
-RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots) {
+RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested) {
     RowsPlan p;
     p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
     const int nch = (int)((K + CHUNK_K - 1) / CHUNK_K);
     p.splits = rows_splits(K);
     p.chunks = (nch + p.splits - 1) / p.splits;
     p.row_lanes = GEMV_WAVES / p.chunks;
-    const int cap = ((PART_BYTES - 64) / (p.chunks * M * 4)) / p.row_lanes * p.row_lanes;
+    const int part_bytes = PART_BYTES - 64 - (nested ? MAP_BYTES : 0);
+    const int cap = (part_bytes / (p.chunks * M * 4)) / p.row_lanes * p.row_lanes;
     int bands_target = slots / p.splits;
     if (bands_target < 1) bands_target = 1;
     // one task per resident workgroup if its partial sums fit in LDS, else 2, 3, ... balanced rounds
@@ -332,7 +350,7 @@ template <int M, bool NESTED>
 hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int cnt = p.rows_per_band / p.row_lanes;  // rows per wave and task
     if constexpr (M == 1)
-        if (cnt >= 8) return launch_u<1, 8, NESTED>(a, p, grid, stream);
+        if (!NESTED && cnt >= 8) return launch_u<1, 8, NESTED>(a, p, grid, stream);  // nested: one more register per slot
     if constexpr (M <= 2)
         if (cnt >= 4) return launch_u<M, 4, NESTED>(a, p, grid, stream);
     return launch_u<M, 2, NESTED>(a, p, grid, stream);
@@ -376,7 +394,7 @@ hipError_t gemv_rows_setup() {
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {
     int slots = 2 * cus;
     if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
-    const RowsPlan p = make_rows_plan(a.M, a.N, a.K, a.block_log2, slots);
+    const RowsPlan p = make_rows_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
     const int grid = p.ntasks < slots ? p.ntasks : slots;
     return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
 }

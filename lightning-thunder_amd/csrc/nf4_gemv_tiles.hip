@@ -211,9 +211,14 @@ __device__ __forceinline__ void prepare_phase(const MatmulArgs& a, PhaseRegs& r,
 }
 
 // MFMA j = 4p + q of the phase covers k [32j, 32j + 32) and uses d[q][p].
-template <int R>
+// EXACT (K > 16384): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA -- the
+// reference's dequantisation bit for bit -- and the MFMAs accumulate straight into acc.
+template <int R, bool EXACT>
 __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uint8_t* xph, int lane, f32x4& acc) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     const uint32_t lane4 = (uint32_t)lane * 4u;
+    const uint32_t lane8 = (uint32_t)(lane & 31) * 8u;
     const int gg = lane >> 4, m = lane & 15;
     const uint32_t xoff_even = (uint32_t)(gg * R + ((m ^ gg) & (R - 1))) * 16u;
     const uint32_t xoff_odd = (uint32_t)(gg * R + ((m ^ (4 | gg)) & (R - 1))) * 16u;
@@ -221,6 +226,7 @@ __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uin
     for (int p = 0; p < 4; ++p) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
+            const float scale = o.sc[2 * p + h];
             f32x4 blk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int qq = 0; qq < 2; ++qq) {
@@ -228,16 +234,29 @@ __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uin
                 const int j = 4 * p + q;
                 uint32_t t[4];
 #pragma unroll
-                for (int b = 0; b < 4; ++b)
-                    t[b] = lds_table_read(__builtin_amdgcn_perm(o.d[q][p], lane4, 0x0c0c0400u | ((uint32_t)b << 8)));
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t sel = 0x0c0c0400u | ((uint32_t)b << 8);
+                    if (EXACT) {
+                        const float2 v = lds_table_read2(__builtin_amdgcn_perm(o.d[q][p], lane8, sel));
+                        const f32x2_t f = {__fmul_rn(v.x, scale), __fmul_rn(v.y, scale)};
+                        t[b] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+                    } else {
+                        t[b] = lds_table_read(__builtin_amdgcn_perm(o.d[q][p], lane4, sel));
+                    }
+                }
                 const uint4 xa = *reinterpret_cast<const uint4*>(xph + j * (64 * R) + (qq ? xoff_odd : xoff_even));
                 const uint4 wb = make_uint4(t[0], t[1], t[2], t[3]);
-                blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa),
-                                                              __builtin_bit_cast(bf16x8, wb), blk, 0, 0, 0);
+                if (EXACT)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa),
+                                                                  __builtin_bit_cast(bf16x8, wb), acc, 0, 0, 0);
+                else
+                    blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa),
+                                                                  __builtin_bit_cast(bf16x8, wb), blk, 0, 0, 0);
             }
-            const float scale = o.sc[2 * p + h];
+            if (!EXACT) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] = fmaf(scale, blk[i], acc[i]);
+                for (int i = 0; i < 4; ++i) acc[i] = fmaf(scale, blk[i], acc[i]);
+            }
         }
     }
 }
@@ -292,7 +311,7 @@ __device__ __forceinline__ void restage_x(const MatmulArgs& a, uint8_t* xlds, in
     }
 }
 
-template <bool B64, bool NESTED, int R>
+template <bool B64, bool NESTED, int R, bool EXACT>
 __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Plan p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int CAP = XBYTES_MAX / (R * 1024);  // phases of x that fit
@@ -365,7 +384,10 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
     }
     int resident = slice_of(cc);
     store_x_slice<R>(a, xv, smem + TABLE_BYTES, slice_phases(resident), lane, wave);
-    build_pair_table(smem, lut_lane, lane, wave);
+    if (EXACT)
+        build_pair_table_f32(smem, lut_lane, lane, wave);
+    else
+        build_pair_table(smem, lut_lane, lane, wave);
     __syncthreads();
 
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
@@ -394,7 +416,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                     load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
                     advance(lc);
                 }
-                contract_phase<R>(o, smem + TABLE_BYTES + cc.ph * (R * 1024), lane, acc[j]);
+                contract_phase<R, EXACT>(o, smem + TABLE_BYTES + cc.ph * (R * 1024), lane, acc[j]);
                 advance(cc);
             } else if (lc.valid && lc.slot == j) {
                 load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
@@ -519,9 +541,11 @@ size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 template <bool B64, bool NESTED>
 hipError_t allow_both() {
-    hipError_t e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8>, SMEM_BYTES);
-    if (e != hipSuccess) return e;
-    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16>, SMEM_BYTES);
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, true>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, true>, SMEM_BYTES);
 }
 
 hipError_t gemv_tiles_setup() {
@@ -532,12 +556,12 @@ hipError_t gemv_tiles_setup() {
     return allow_both<true, true>();
 }
 
-template <int R>
+template <int R, bool EXACT>
 hipError_t launch_r(const MatmulArgs& a, const Plan& p, int grid, hipStream_t stream) {
     const bool b64 = a.block_log2 == 6;
     const bool nested = a.nested.q != nullptr;
-    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R> : gemv_tiles_kernel<true, false, R>)
-                    : (nested ? gemv_tiles_kernel<false, true, R> : gemv_tiles_kernel<false, false, R>);
+    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R, EXACT> : gemv_tiles_kernel<true, false, R, EXACT>)
+                    : (nested ? gemv_tiles_kernel<false, true, R, EXACT> : gemv_tiles_kernel<false, false, R, EXACT>);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
@@ -546,7 +570,9 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
     Plan p = make_plan(a.M, a.N, a.K);
     const int grid = grid_for((int64_t)p.tile_groups * p.splits, p.splits, cus < 1024 ? cus : 1024);
     p.tg_step = grid / p.splits;
-    return rows_held(a.M) == 8 ? launch_r<8>(a, p, grid, stream) : launch_r<16>(a, p, grid, stream);
+    if (gemv_wants_exact(a.K))
+        return rows_held(a.M) == 8 ? launch_r<8, true>(a, p, grid, stream) : launch_r<16, true>(a, p, grid, stream);
+    return rows_held(a.M) == 8 ? launch_r<8, false>(a, p, grid, stream) : launch_r<16, false>(a, p, grid, stream);
 }
 
 }  // namespace nf4

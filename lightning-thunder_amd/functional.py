@@ -244,9 +244,11 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "gemv"  # row-streaming kernel: blocks may straddle rows
     if K % 64 or K % blocksize:
         return "dequant+linear"
-    if M <= 16 and K % 512 == 0 and K <= EXACT_K:
-        return "gemv"  # MFMA tile kernel
-    return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M else "gemm"
+    if M <= 16 and K % 512 == 0:
+        return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
+    # the fused GEMM kernel streams K sequentially per tile: beyond EXACT_K even a few rows of x are
+    # served faster by dequantize + dense GEMM
+    return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M or K > EXACT_K else "gemm"
 
 
 def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> torch.Tensor:

@@ -125,7 +125,8 @@ def test_fused_route_rules(ta):
     assert route(5, 64, 1376) == "dequant+linear"        # tile kernel needs K % 512, gemm K % 64
     assert route(8, 64, 1344) == "gemm"                   # fused GEMM kernel below DENSE_ROUTE_MIN_M rows
     assert route(17, 64, 4096) == "dequant+gemm" and route(2048, 4096, 4096) == "dequant+gemm"
-    assert route(16, 8192, 28672) == "gemm"              # K > 16384: exact weights wanted
+    assert route(16, 8192, 28672) == "gemv"              # K > 16384: the tile kernel's exact-weights variant
+    assert route(17, 8192, 28672) == "dequant+gemm"
     assert route(1, 8192, 28672) == "gemv"               # row-streaming kernel has an exact variant
     assert route(1, 64, 4096, dtype=torch.float32) == "dequant+linear"
     assert route(1, 64, 4096, xdtype=torch.float16, dtype=torch.float16) == "dequant+linear"

@@ -364,3 +364,21 @@ def test_llama70b_shapes_double_quant(ta, N, K):
         if M <= 16:
             y2 = ta.matmul_nf4(x, qw, None, absmax_rec, code, 64, torch.bfloat16, (N, K))
             assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+def test_gemv_exact_variants_recover_dequantized_weights(ta, oracle, M):
+    """K > 16384 selects the decode kernels' exact-weights variants: with one-hot rows of x every
+    output is a single product 1.0 * w, so it must equal nf4hip_dequantize's value bit for bit."""
+    _sync_print(f"gemv exact one-hot M={M}")
+    N, K = 272, 32768
+    w = _weights((N, K), seed=77)
+    qw, absmax = oracle.C().quantize(w, 64)
+    lut = oracle.nf4_lut()
+    cols = torch.randint(0, K, (M,), generator=torch.Generator().manual_seed(M))
+    x = torch.zeros(M, K, dtype=torch.bfloat16)
+    x[torch.arange(M), cols] = 1.0
+    assert ta.functional.fused_route(x, None, 64, torch.bfloat16, (N, K)) == "gemv"
+    y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None, absmax.to(DEV), lut.to(DEV), 64, torch.bfloat16, (N, K))
+    deq = oracle.C().dequantize(qw, absmax, lut, 64, torch.bfloat16, (N, K))
+    assert torch.equal(y.cpu().view(torch.int16), deq[:, cols].t().contiguous().view(torch.int16))

@@ -382,3 +382,24 @@ def test_gemv_exact_variants_recover_dequantized_weights(ta, oracle, M):
     y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None, absmax.to(DEV), lut.to(DEV), 64, torch.bfloat16, (N, K))
     deq = oracle.C().dequantize(qw, absmax, lut, 64, torch.bfloat16, (N, K))
     assert torch.equal(y.cpu().view(torch.int16), deq[:, cols].t().contiguous().view(torch.int16))
+
+
+def test_gemv_randomized_sweep(ta, oracle):
+    """Seeded sweep over the decode kernels' planning space: ragged N (tile, band and batch tails),
+    K from one phase to several slices, every M, bias, nested absmax and larger blocksizes, each
+    against the float64 oracle."""
+    rng = torch.Generator().manual_seed(1234)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rng))]
+
+    for case in range(48):
+        M = pick([1, 2, 3, 4, 5, 7, 8, 9, 12, 16])
+        K = pick([512, 1024, 1536, 2048, 3072, 4096, 5120, 6144, 8192, 11264])
+        N = pick([1, 3, 15, 16, 17, 100, 127, 128, 129, 257, 400, 515, 1000, 2049])
+        blocksize = pick([64, 64, 64, 128, 256, 512])
+        bias = pick([False, False, True])
+        nested = pick([False, False, True]) and (N * K // blocksize) >= 1
+        _sync_print(f"sweep {case}: M={M} N={N} K={K} bs={blocksize} bias={bias} nested={nested}")
+        assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, blocksize, torch.bfloat16, (N, K)) == "gemv"
+        _matmul_case(ta, oracle, M, N, K, blocksize=blocksize, bias=bias, nested=nested, seed=10 * case)

@@ -55,7 +55,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only; --gpus {args.gpus} is not supported "
-              "(the path would shard by rows/columns of W, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard like a dense linear: by rows of W for q/k/v/gate/up/lm_head, by columns for o/down)", file=sys.stderr)
         return 2
 
     import torch

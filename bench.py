@@ -13,6 +13,8 @@ Prints ONE JSON line:
               timed group by group): algorithmic bytes per launch / average launch duration, from
               HIP events recorded inside the timed region on the launch stream, against the
               8 TB/s HBM peak; config.kernels lists all three
+  config.prefill = BASELINE config 3 (M in {512, 2048, 8192}) run after the timed region: TFLOP/s of the
+              default route (HIP dequantize + dense GEMM) and of the fused GEMM kernel, vs the bf16 MFMA peak
   config.decode = BASELINE config 4 (full Llama-3-8B architecture, greedy decode, batch 1 and 8)
               run after the timed region: decode tokens/s, the second half of the metric
   cpu_baseline = the reference's CPU-side route (torch-eager dequantize + linear, restated in
@@ -50,6 +52,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU baseline sample (0 disables)")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-regime section (BASELINE config 3)")
     ap.add_argument("--decode-tokens", type=int, default=128,
                     help="tokens of the Llama-3-8B greedy decode that follows the GEMV pass (0 disables)")
     args = ap.parse_args()
@@ -189,14 +192,67 @@ def main() -> int:
         },
     }
 
+    del weights, xs, outs, ws
+    torch.cuda.empty_cache()
+    if not args.no_prefill:
+        result["config"]["prefill"] = prefill_section(torch, ta)
     if args.decode_tokens > 1:
-        del weights, xs, outs, ws
-        torch.cuda.empty_cache()
         result["config"]["decode"] = llama_decode(torch, ta, args.decode_tokens)
     if args.cpu_seconds > 0:
         result["cpu_baseline"] = cpu_baseline(torch, args.cpu_seconds)
     print(json.dumps(result))
     return 0
+
+
+MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CUs x 2.4 GHz x 4096 flop/clk/CU
+
+
+def prefill_section(torch, ta) -> dict:
+    """BASELINE config 3, outside the timed region of the GEMV metric: the Llama-3-8B projection
+    shapes with M in {512, 2048, 8192} rows of x through ``matmul_nf4`` (which routes them to
+    nf4hip_dequantize + the dense library GEMM), and the fused NF4 GEMM kernel (nf4hip_gemm) at
+    M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events around 10 calls (3 for the fused kernel) after 3 warm-up calls."""
+    dev = torch.device("cuda:0")
+    F = ta.functional
+    code = ta.nf4_code(dev)
+
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    rows = []
+    for si, (N, K) in enumerate([(4096, 4096), (14336, 4096), (4096, 14336)]):
+        g = torch.Generator(device=dev).manual_seed(3000 + si)
+        w = (torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+        qw, absmax, _ = ta.quantize_nf4(w, BLOCKSIZE)
+        del w
+        for M in (512, 2048, 8192):
+            x = torch.randn(M, K, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            assert F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K)) == "dequant+gemm"
+            t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 10)
+            row = {"N": N, "K": K, "M": M, "route": "nf4hip_dequantize + dense GEMM", "us": round(t * 1e6, 1),
+                   "tflops": round(2.0 * M * N * K / t / 1e12, 1),
+                   "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+            rows.append(row)
+            if M == 2048:
+                saved, F.DENSE_ROUTE_MIN_M = F.DENSE_ROUTE_MIN_M, 1 << 30
+                try:
+                    assert F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K)) == "gemm"
+                    t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 3)
+                finally:
+                    F.DENSE_ROUTE_MIN_M = saved
+                rows.append({"N": N, "K": K, "M": M, "route": "nf4hip_gemm (fused)", "us": round(t * 1e6, 1),
+                             "tflops": round(2.0 * M * N * K / t / 1e12, 1),
+                             "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows}
 
 
 def llama_decode(torch, ta, n_new: int) -> dict:

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void dq_compress_kernel(const float* __restric
     const int nested = 1 << nested_log2;
     const int64_t base = (int64_t)blockIdx.x << nested_log2;
     map[tid] = map256[tid];
-    if (tid == 0) zero_code = 255;
+    if (tid == 0) zero_code = 256;  // sentinel: the map holds no 0.0 (then an all-zero block stores code 0)
     __syncthreads();
     if (map[tid] == 0.0f) atomicMin(&zero_code, tid);
 
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void dq_compress_kernel(const float* __restric
     for (int i = tid; i < nested; i += 256) {
         const int64_t idx = base + i;
         if (idx >= nblocks) continue;
-        int best = zero_code;
+        int best = zero_code == 256 ? 0 : zero_code;
         if (m != 0.0f) {
             const float s = __fmul_rn(__fsub_rn(absmax[idx], offset), inv);
             float bestd = INFINITY;

@@ -152,6 +152,28 @@ def test_nested_absmax(ta, oracle):
     assert torch.equal(deq.cpu().view(torch.int16), deq_o.view(torch.int16))
 
 
+@pytest.mark.parametrize("map_has_zero", [True, False])
+def test_nested_absmax_all_equal_block(ta, oracle, map_has_zero):
+    """A nested block whose absmax values all equal the offset has residual 0 everywhere: it stores
+    the code of 0.0, or code 0 when the map holds no 0.0 -- as the oracle does."""
+    _sync_print(f"nested absmax, zero block, map_has_zero={map_has_zero}")
+    absmax = torch.full((512,), 0.25)
+    absmax[256:] = torch.linspace(0.1, 0.4, 256)  # second nested block: ordinary
+    D = oracle.create_dynamic_map()
+    if not map_has_zero:
+        D = torch.where(D == 0, torch.full_like(D, 1e-6), D)
+    off = 0.25
+    q_o, a2_o = oracle.C().dq_compress(absmax, D, off)
+    lib = ta._lib.load()
+    q = torch.empty(512, dtype=torch.uint8, device=DEV)
+    a2 = torch.empty(2, dtype=torch.float32, device=DEV)
+    a_dev, D_dev = absmax.to(DEV), D.to(DEV)
+    ta._lib.check(lib.nf4hip_dq_compress(a_dev.data_ptr(), 512, 256, D_dev.data_ptr(), off, q.data_ptr(), a2.data_ptr(),
+                                         torch.cuda.current_stream().cuda_stream))
+    assert torch.equal(q.cpu(), q_o) and torch.equal(a2.cpu(), a2_o)
+    assert a2_o[0] == 0 and len(set(q_o[:256].tolist())) == 1
+
+
 # ------------------------------------------------------------------------------------------------
 # matmul
 # ------------------------------------------------------------------------------------------------

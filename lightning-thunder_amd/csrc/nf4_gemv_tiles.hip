@@ -222,40 +222,63 @@ __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uin
     const int gg = lane >> 4, m = lane & 15;
     const uint32_t xoff_even = (uint32_t)(gg * R + ((m ^ gg) & (R - 1))) * 16u;
     const uint32_t xoff_odd = (uint32_t)(gg * R + ((m ^ (4 | gg)) & (R - 1))) * 16u;
+
+    // The 16 MFMAs of a phase in the order s = 0..15: p = s >> 2, then the two blocks of p interleaved
+    // (block h = s & 1, MFMA qq = (s >> 1) & 1 of the block), so that consecutive MFMAs never depend on
+    // each other.  Operands are fetched from LDS one MFMA ahead of their use.
+    struct Ops {
+        uint32_t t[4];
+        float2 tf[4];
+        uint4 xa;
+    };
+    auto fetch = [&](int s, Ops& f) __attribute__((always_inline)) {
+        const int p = s >> 2, h = s & 1, qq = (s >> 1) & 1;
+        const int q = 2 * h + qq;
+        const int j = 4 * p + q;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t sel = 0x0c0c0400u | ((uint32_t)b << 8);
+            if (EXACT)
+                f.tf[b] = lds_table_read2(__builtin_amdgcn_perm(o.d[q][p], lane8, sel));
+            else
+                f.t[b] = lds_table_read(__builtin_amdgcn_perm(o.d[q][p], lane4, sel));
+        }
+        f.xa = *reinterpret_cast<const uint4*>(xph + j * (64 * R) + (qq ? xoff_odd : xoff_even));
+    };
+    constexpr int AHEAD = 1;  // MFMAs between the fetch of an operand set and its use
+    Ops ops[AHEAD + 1];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const float scale = o.sc[2 * p + h];
-            f32x4 blk = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < AHEAD; ++s) fetch(s, ops[s]);
+    f32x4 blk[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-            for (int qq = 0; qq < 2; ++qq) {
-                const int q = 2 * h + qq;
-                const int j = 4 * p + q;
-                uint32_t t[4];
+    for (int s = 0; s < 16; ++s) {
+        if (s + AHEAD < 16) fetch(s + AHEAD, ops[(s + AHEAD) % (AHEAD + 1)]);
+        const int p = s >> 2, h = s & 1, qq = (s >> 1) & 1;
+        const float scale = o.sc[2 * p + h];
+        Ops& f = ops[s % (AHEAD + 1)];
+        if (EXACT) {
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const uint32_t sel = 0x0c0c0400u | ((uint32_t)b << 8);
-                    if (EXACT) {
-                        const float2 v = lds_table_read2(__builtin_amdgcn_perm(o.d[q][p], lane8, sel));
-                        const f32x2_t f = {__fmul_rn(v.x, scale), __fmul_rn(v.y, scale)};
-                        t[b] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-                    } else {
-                        t[b] = lds_table_read(__builtin_amdgcn_perm(o.d[q][p], lane4, sel));
-                    }
-                }
-                const uint4 xa = *reinterpret_cast<const uint4*>(xph + j * (64 * R) + (qq ? xoff_odd : xoff_even));
-                const uint4 wb = make_uint4(t[0], t[1], t[2], t[3]);
-                if (EXACT)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa),
-                                                                  __builtin_bit_cast(bf16x8, wb), acc, 0, 0, 0);
-                else
-                    blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa),
-                                                                  __builtin_bit_cast(bf16x8, wb), blk, 0, 0, 0);
+            for (int b = 0; b < 4; ++b) {
+                const f32x2_t v = {__fmul_rn(f.tf[b].x, scale), __fmul_rn(f.tf[b].y, scale)};
+                f.t[b] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
             }
-            if (!EXACT) {
+        }
+        const uint4 wb = make_uint4(f.t[0], f.t[1], f.t[2], f.t[3]);
+        if (EXACT) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f.xa), __builtin_bit_cast(bf16x8, wb),
+                                                          acc, 0, 0, 0);
+        } else {
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            blk[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f.xa),
+                                                             __builtin_bit_cast(bf16x8, wb), qq ? blk[h] : zero, 0, 0, 0);
+            // the block of the PREVIOUS pair that just completed is scaled here, one MFMA later
+            if (qq == 1 && h == 1) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] = fmaf(scale, blk[i], acc[i]);
+                for (int hh = 0; hh < 2; ++hh) {
+                    const float sc = o.sc[2 * p + hh];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[i] = fmaf(sc, blk[hh][i], acc[i]);
+                }
             }
         }
     }

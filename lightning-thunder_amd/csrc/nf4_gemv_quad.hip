@@ -181,13 +181,33 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 float tot[4] = {0.f, 0.f, 0.f, 0.f};
+                // take the slot's contents, then refill it at once: the load is in flight while the
+                // table lookups and MFMAs below run
+                uint32_t dd[CPW][4];
+                float ss[CPW];
 #pragma unroll
                 for (int c = 0; c < CPW; ++c) {
-                    const uint32_t d[4] = {wq[u][c].x, wq[u][c].y, wq[u][c].z, wq[u][c].w};
-                    float s = sq[u][c];
+                    dd[c][0] = wq[u][c].x; dd[c][1] = wq[u][c].y; dd[c][2] = wq[u][c].z; dd[c][3] = wq[u][c].w;
+                    ss[c] = sq[u][c];
                     if (NESTED)
-                        s = __fadd_rn(__fmul_rn(reinterpret_cast<const float*>(smem + MAP_OFFSET)[__float_as_uint(s)], s2[u][c]),
-                                      a.nested.offset);
+                        ss[c] = __fadd_rn(__fmul_rn(reinterpret_cast<const float*>(smem + MAP_OFFSET)[__float_as_uint(ss[c])], s2[u][c]),
+                                          a.nested.offset);
+                }
+                const int i = i0 + u;
+                if (i + U < cnt) {
+                    issue(u, i + U);
+                } else {  // slot is dead from here on; say so, or the compiler keeps copies alive
+#pragma unroll
+                    for (int c = 0; c < CPW; ++c) {
+                        wq[u][c] = make_uint4(0, 0, 0, 0);
+                        sq[u][c] = 0.0f;
+                        if (NESTED) s2[u][c] = 0.0f;
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < CPW; ++c) {
+                    const uint32_t* d = dd[c];
+                    const float s = ss[c];
                     uint32_t pr[16];
 #pragma unroll
                     for (int q = 0; q < 4; ++q)
@@ -220,17 +240,6 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                         tot[1] = fmaf(acc[1], NF4_DPP(s, 0x55, 0xf, 0.0f), tot[1]);
                         tot[2] = fmaf(acc[2], NF4_DPP(s, 0xAA, 0xf, 0.0f), tot[2]);
                         tot[3] = fmaf(acc[3], NF4_DPP(s, 0xFF, 0xf, 0.0f), tot[3]);
-                    }
-                }
-                const int i = i0 + u;
-                if (i + U < cnt) {
-                    issue(u, i + U);
-                } else {  // slot is dead from here on; say so, or the compiler keeps copies alive
-#pragma unroll
-                    for (int c = 0; c < CPW; ++c) {
-                        wq[u][c] = make_uint4(0, 0, 0, 0);
-                        sq[u][c] = 0.0f;
-                        if (NESTED) s2[u][c] = 0.0f;
                     }
                 }
                 const float total = reduce_rows(tot, lane);  // lanes 0..15: row 2*b3+b2 of the group, x row ri

@@ -55,10 +55,14 @@ struct QuadPlan {
 
 #define NF4_DPP(v, ctrl, bank, keep_old) \
     __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep_old), __builtin_bit_cast(int, v), ctrl, 0xf, bank, false))
+// every lane of the quad reads a valid lane: no "old" value is needed, which lets the compiler fold
+// the DPP into the instruction that uses the result
+#define NF4_QUAD_BCAST(v, ctrl) \
+    __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
 
 // value of `v` in lane (lane ^ 4); DPP shifts by 4 inside a row of 16, direction chosen per bank of 4
 __device__ __forceinline__ float lane_xor4(float v) {
-    float o = NF4_DPP(v, 0x104 /*row_shl:4*/, 0x5, 0.0f);
+    float o = NF4_DPP(v, 0x104 /*row_shl:4*/, 0x5, v);  // banks 1, 3 are overwritten below
     return NF4_DPP(v, 0x114 /*row_shr:4*/, 0xa, o);
 }
 
@@ -75,7 +79,7 @@ __device__ __forceinline__ float reduce_rows(const float t[4], int lane) {
     }
     const float keep = b3 ? w[1] : w[0];
     const float send = b3 ? w[0] : w[1];
-    float y = keep + NF4_DPP(send, 0x128 /*row_ror:8*/, 0xf, 0.0f);
+    float y = keep + NF4_DPP(send, 0x128 /*row_ror:8*/, 0xf, send);
     y += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, y)));
     y += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, y)));
     return y;
@@ -194,16 +198,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                                           a.nested.offset);
                 }
                 const int i = i0 + u;
-                if (i + U < cnt) {
-                    issue(u, i + U);
-                } else {  // slot is dead from here on; say so, or the compiler keeps copies alive
-#pragma unroll
-                    for (int c = 0; c < CPW; ++c) {
-                        wq[u][c] = make_uint4(0, 0, 0, 0);
-                        sq[u][c] = 0.0f;
-                        if (NESTED) s2[u][c] = 0.0f;
-                    }
-                }
+                if (i + U < cnt) issue(u, i + U);  // else the slot keeps its stale contents: its results are dropped
 #pragma unroll
                 for (int c = 0; c < CPW; ++c) {
                     const uint32_t* d = dd[c];
@@ -236,10 +231,10 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                         for (int i = 0; i < 4; ++i) tot[i] += acc[i];
                     } else {
                         // acc[i] belongs to weight row i, whose absmax lane i of this quad holds
-                        tot[0] = fmaf(acc[0], NF4_DPP(s, 0x00, 0xf, 0.0f), tot[0]);
-                        tot[1] = fmaf(acc[1], NF4_DPP(s, 0x55, 0xf, 0.0f), tot[1]);
-                        tot[2] = fmaf(acc[2], NF4_DPP(s, 0xAA, 0xf, 0.0f), tot[2]);
-                        tot[3] = fmaf(acc[3], NF4_DPP(s, 0xFF, 0xf, 0.0f), tot[3]);
+                        tot[0] = fmaf(NF4_QUAD_BCAST(s, 0x00), acc[0], tot[0]);
+                        tot[1] = fmaf(NF4_QUAD_BCAST(s, 0x55), acc[1], tot[1]);
+                        tot[2] = fmaf(NF4_QUAD_BCAST(s, 0xAA), acc[2], tot[2]);
+                        tot[3] = fmaf(NF4_QUAD_BCAST(s, 0xFF), acc[3], tot[3]);
                     }
                 }
                 const float total = reduce_rows(tot, lane);  // lanes 0..15: row 2*b3+b2 of the group, x row ri

@@ -59,6 +59,13 @@ __device__ __forceinline__ uint4 load16_stream(const void* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// 16-byte load as a value (a struct-typed `uint4` copy from global memory becomes a memcpy that keeps
+// its destination array in scratch memory).
+__device__ __forceinline__ uint4 load16(const void* p) {
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // fp32 -> bf16 bits, round to nearest even (finite inputs; NaN is quieted).
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);

@@ -46,7 +46,9 @@ constexpr int WAVES = GEMV_WAVES;
 constexpr int TABLE_BYTES = GEMV_TABLE_BYTES;
 constexpr int PHASE_K = 512;                 // k per phase
 constexpr int XBYTES_MAX = 80 * 1024;        // resident x operands
-constexpr int SMEM_BYTES = TABLE_BYTES + XBYTES_MAX;
+constexpr int ITEMS_MAX = 512;               // longest work list of a workgroup (one entry per thread)
+constexpr int ITEMS_OFFSET = TABLE_BYTES + XBYTES_MAX;
+constexpr int SMEM_BYTES = ITEMS_OFFSET + ITEMS_MAX * 16;
 constexpr int COUNTER_BYTES = GEMV_COUNTER_BYTES;
 constexpr int SLOTS = 4;                     // ring slots = accumulator sets = largest batch
 
@@ -63,19 +65,118 @@ struct PhaseRegs {
     float4 s[2];  // absmax of the 8 blocks of the phase (or raw data to build them)
 };
 
-// Position in the item stream of a workgroup (wave-uniform).  An item is one phase of one tile
-// group.  Order: batch, slice, phase, tile group of the batch; `slot` counts items of the batch
-// modulo 4, so that with batches of 1, 2 or 4 tile groups a slot always meets the same tile group.
-struct Cursor {
-    int bi;     // index (in the workgroup's list of tile groups) of the batch's first tile group
-    int nb;     // tile groups in the batch: 1, 2 or 4
-    int batch;  // batch number
-    int q;      // slice step within the batch (odd batches walk the slices backwards)
-    int ph;     // phase within the slice
-    int t;      // tile group within the batch
-    int slot;
-    bool valid;
+// One entry of a workgroup's work list: one 512-k phase of one tile group, or a gap.
+//
+// Order of the list: batch, slice, phase, tile group of the batch.  Tile groups are taken in batches of
+// 4, then 2, then 1; entry i uses ring slot and accumulator set i & 3, so with batches of 1, 2 or 4
+// tile groups a slot always meets the same tile group.  Every slice of a batch starts at a multiple
+// of 4 (gaps pad the previous one), so a change of slice is only ever met at slot 0.  Odd batches
+// walk the slices backwards, so the slice a batch ends with is the one the next batch starts with.
+// The list is a pure function of the entry index: every workgroup writes its own into LDS once, one
+// entry per thread, and the waves then read it instead of carrying cursors through the loop.
+struct Item {
+    int tg;    // tile group
+    int kabs;  // first k of the phase
+    int info;  // see below
+    int k0;    // first k of the phase's slice
 };
+constexpr int ITEM_PHS_MASK = 0xf;      // bits 0-3: phase within its slice
+constexpr int ITEM_NB_SHIFT = 4;        // bits 4-6: tile groups in the batch (1, 2, 4)
+constexpr int ITEM_GAP = 1 << 7;        // nothing to do in this slot
+constexpr int ITEM_RESTAGE = 1 << 8;    // first entry of a slice that is not resident yet (always at slot 0)
+constexpr int ITEM_END = 1 << 9;        // last entry of its batch
+constexpr int ITEM_NPH_SHIFT = 12;      // bits 12-15: phases of the slice
+
+struct ListShape {
+    int G;         // tile groups of this workgroup
+    int rph;       // phases of its K range
+    int nsl;       // slices of the range
+    int last;      // phases of the last slice
+    int r0;        // first phase of the range
+    int tg0;       // first tile group
+    int tg_step;   // distance between consecutive tile groups
+    int nitems;    // entries, gaps included (a multiple of 4)
+};
+
+__device__ __host__ constexpr int ceil4(int v) { return (v + 3) & ~3; }
+
+// entries of one batch of nb tile groups
+template <int CAP>
+__device__ __host__ constexpr int batch_length(int nsl, int last, int nb) {
+    return (nsl - 1) * ceil4(CAP * nb) + ceil4(last * nb);
+}
+
+template <int CAP>
+__device__ __host__ constexpr int list_length(int G, int nsl, int last) {
+    const int full = G >> 2, rem = G & 3;
+    int n = full * batch_length<CAP>(nsl, last, 4);
+    if (rem == 1) n += batch_length<CAP>(nsl, last, 1);
+    if (rem >= 2) n += batch_length<CAP>(nsl, last, 2);
+    if (rem == 3) n += batch_length<CAP>(nsl, last, 1);
+    return n;
+}
+
+template <int CAP>
+__device__ __forceinline__ Item make_item(const ListShape& ls, int i) {
+    const int LB4 = batch_length<CAP>(ls.nsl, ls.last, 4);
+    const int full = ls.G >> 2, rem = ls.G & 3;
+    int batch, k, nb, bi;
+    if (i < full * LB4) {
+        batch = i / LB4;
+        k = i - batch * LB4;
+        nb = 4;
+        bi = 4 * batch;
+    } else {
+        const int j = i - full * LB4;
+        const int nb0 = rem == 1 ? 1 : 2;
+        const int L0 = batch_length<CAP>(ls.nsl, ls.last, nb0);
+        batch = full;
+        bi = 4 * full;
+        if (j < L0) {
+            nb = nb0;
+            k = j;
+        } else {  // rem == 3: the single tile group after the pair
+            nb = 1;
+            k = j - L0;
+            batch += 1;
+            bi += 2;
+        }
+    }
+    const int Lf = ceil4(CAP * nb), Ll = ceil4(ls.last * nb);
+    int sl, kk;
+    if (!(batch & 1)) {  // forwards: the full slices, then the last one
+        const int head = (ls.nsl - 1) * Lf;
+        if (k < head) {
+            sl = k / Lf;
+            kk = k - sl * Lf;
+        } else {
+            sl = ls.nsl - 1;
+            kk = k - head;
+        }
+    } else {  // backwards: the last slice first
+        if (k < Ll) {
+            sl = ls.nsl - 1;
+            kk = k;
+        } else {
+            const int q = (k - Ll) / Lf;
+            sl = ls.nsl - 2 - q;
+            kk = k - Ll - q * Lf;
+        }
+    }
+    const int nph = sl == ls.nsl - 1 ? ls.last : CAP;
+    const int t = kk & (nb - 1);
+    const int phs = kk >> (nb >> 1);  // nb = 1, 2, 4 -> shift 0, 1, 2
+    const bool final_slice = (batch & 1) ? sl == 0 : sl == ls.nsl - 1;
+    Item it;
+    it.tg = ls.tg0 + (bi + t) * ls.tg_step;
+    it.kabs = (ls.r0 + sl * CAP + phs) * PHASE_K;
+    it.k0 = (ls.r0 + sl * CAP) * PHASE_K;
+    it.info = (phs & ITEM_PHS_MASK) | (nb << ITEM_NB_SHIFT) | ((nph & 0xf) << ITEM_NPH_SHIFT);
+    if (kk >= nph * nb) it.info |= ITEM_GAP;
+    if (kk == 0 && k != 0) it.info |= ITEM_RESTAGE;
+    if (final_slice && kk == nph * nb - 1) it.info |= ITEM_END;
+    return it;
+}
 
 // Lane-dependent constants of the load side.
 struct LaneLoad {
@@ -284,53 +385,32 @@ __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uin
     }
 }
 
-// One (row, phase) of x = 64 pieces of 16 bytes = 1 KB contiguous per wave; at most 80 such units
-// per slice, ten per wave.  All loads are issued before the first LDS write.
-constexpr int XUNITS = XBYTES_MAX / 1024 / WAVES;
+// Staging of one slice of x.  One (row, phase) of x = 64 pieces of 16 bytes = 1 KB contiguous,
+// handled by one wave: wave w takes rows w and w + 8 (the latter only exists in the 16-row layout),
+// all phases of the slice, i.e. at most ten units.  All loads are issued before the first LDS
+// write.
+constexpr int XUNITS = XBYTES_MAX / 1024 / WAVES;  // units per wave: 10 in both layouts
 
-__device__ __forceinline__ void load_x_slice(const MatmulArgs& a, uint4 (&xv)[XUNITS], int k0, int n, int lane,
-                                             int wave) {
+template <int R>
+__device__ __forceinline__ void load_x_slice(const MatmulArgs& a, uint4 (&v)[XUNITS], int k0, int n, int lane, int wave) {
+    constexpr int CAP = XBYTES_MAX / (R * 1024);
 #pragma unroll
-    for (int i = 0; i < XUNITS; ++i) {
-        const int u = min(wave + WAVES * i, a.M * n - 1);  // past the end: re-read the last unit
-        const int m = u / n, ph = u - m * n;
-        xv[i] = *reinterpret_cast<const uint4*>(a.x + (int64_t)m * a.K + k0 + ph * PHASE_K + lane * 8);
+    for (int u = 0; u < XUNITS; ++u) {
+        // outside the slice or the matrix: re-read a valid unit, the value is dropped
+        const int m = min(wave + 8 * (u / CAP), a.M - 1);
+        const int pp = min(u % CAP, n - 1);
+        v[u] = load16(a.x + (int64_t)m * a.K + k0 + pp * PHASE_K + lane * 8);
     }
 }
 
 template <int R>
-__device__ __forceinline__ void store_x_slice(const MatmulArgs& a, const uint4 (&xv)[XUNITS], uint8_t* xlds, int n,
+__device__ __forceinline__ void store_x_slice(const MatmulArgs& a, const uint4 (&v)[XUNITS], uint8_t* xlds, int n,
                                               int lane, int wave) {
+    constexpr int CAP = XBYTES_MAX / (R * 1024);
 #pragma unroll
-    for (int i = 0; i < XUNITS; ++i) {
-        const int u = wave + WAVES * i;
-        if (u < a.M * n) {
-            const int m = u / n, ph = u - m * n;
-            *reinterpret_cast<uint4*>(xlds + ph * (R * 1024) + xslot_bytes<R>(m, lane)) = xv[i];
-        }
-    }
-}
-
-// Re-staging in the middle of the stream, four units in flight per wave.
-template <int R>
-__device__ __forceinline__ void restage_x(const MatmulArgs& a, uint8_t* xlds, int k0, int n, int lane, int wave) {
-    const int units = a.M * n;
-    for (int u0 = wave; u0 < units; u0 += 4 * WAVES) {
-        uint4 v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int u = min(u0 + WAVES * i, units - 1);
-            const int m = u / n, ph = u - m * n;
-            v[i] = *reinterpret_cast<const uint4*>(a.x + (int64_t)m * a.K + k0 + ph * PHASE_K + lane * 8);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int u = u0 + WAVES * i;
-            if (u < units) {
-                const int m = u / n, ph = u - m * n;
-                *reinterpret_cast<uint4*>(xlds + ph * (R * 1024) + xslot_bytes<R>(m, lane)) = v[i];
-            }
-        }
+    for (int u = 0; u < XUNITS; ++u) {
+        const int m = wave + 8 * (u / CAP), ph = u % CAP;
+        if (m < a.M && ph < n) *reinterpret_cast<uint4*>(xlds + ph * (R * 1024) + xslot_bytes<R>(m, lane)) = v[u];
     }
 }
 
@@ -347,11 +427,15 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
 
     // this workgroup's K range and tile groups
     const int ks = (int)blockIdx.x % p.splits;
-    const int tg0 = (int)blockIdx.x / p.splits;
-    const int r0 = ks * p.range_phases;                             // first phase of the range
-    const int rph = min(p.range_phases, p.total_phases - r0);      // phases in the range
-    const int nsl = (rph + CAP - 1) / CAP;                          // x slices in the range
-    const int G = tg0 < p.tile_groups ? (p.tile_groups - 1 - tg0) / p.tg_step + 1 : 0;
+    ListShape ls;
+    ls.tg0 = (int)blockIdx.x / p.splits;
+    ls.tg_step = p.tg_step;
+    ls.r0 = ks * p.range_phases;                             // first phase of the range
+    ls.rph = min(p.range_phases, p.total_phases - ls.r0);    // phases in the range
+    ls.nsl = (ls.rph + CAP - 1) / CAP;                       // x slices in the range
+    ls.last = ls.rph - (ls.nsl - 1) * CAP;                   // phases of the last slice
+    ls.G = ls.tg0 < p.tile_groups ? (p.tile_groups - 1 - ls.tg0) / p.tg_step + 1 : 0;
+    ls.nitems = list_length<CAP>(ls.G, ls.nsl, ls.last);
 
     LaneLoad ll;
     {
@@ -362,56 +446,50 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
             ll.woff[i] = (uint32_t)min(((lane >> 2) & 3) * 4 + i, a.N - 1) * (uint32_t)(a.K >> 1) + lane_bytes;
         ll.s_off = (uint32_t)min(col, a.N - 1) * (uint32_t)(a.K >> a.block_log2);
     }
-
-    auto batch_size = [&](int bi) {
-        const int rem = G - bi;
-        return rem >= 4 ? 4 : (rem == 3 ? 2 : rem);
-    };
-    auto slice_of = [&](const Cursor& c) { return (c.batch & 1) ? nsl - 1 - c.q : c.q; };
-    auto slice_phases = [&](int sl) { return min(CAP, rph - sl * CAP); };
-    auto advance = [&](Cursor& c) {
-        c.slot = (c.slot + 1) & (SLOTS - 1);
-        if (++c.t < c.nb) return;
-        c.t = 0;
-        if (++c.ph < slice_phases(slice_of(c))) return;
-        c.ph = 0;
-        if (++c.q < nsl) return;
-        c.q = 0;
-        c.bi += c.nb;
-        c.batch += 1;
-        c.slot = 0;
-        c.valid = c.bi < G;
-        c.nb = batch_size(c.bi);
-    };
-    auto first_row = [&](const Cursor& c) {  // first row read for the wave's tile of the item
-        const int n0 = ((tg0 + (c.bi + c.t) * p.tg_step) * WAVES + wave) * 16;
+    auto first_row = [&](int tg) {  // first row read for the wave's tile of a tile group
+        const int n0 = (tg * WAVES + wave) * 16;
         return max(min(n0, a.N - 16), 0);
     };
-    auto first_k = [&](const Cursor& c) { return (r0 + slice_of(c) * CAP + c.ph) * PHASE_K; };
+    const Item* items = reinterpret_cast<const Item*>(smem + ITEMS_OFFSET);
+    auto read_item = [&](int i) {  // wave-uniform LDS read, moved to scalar registers
+        const int4 v = *reinterpret_cast<const int4*>(items + i);
+        Item it;
+        it.tg = __builtin_amdgcn_readfirstlane(v.x);
+        it.kabs = __builtin_amdgcn_readfirstlane(v.y);
+        it.info = __builtin_amdgcn_readfirstlane(v.z);
+        it.k0 = __builtin_amdgcn_readfirstlane(v.w);
+        return it;
+    };
 
-    Cursor lc = {0, batch_size(0), 0, 0, 0, 0, 0, G > 0};  // next item to load
-    Cursor cc = lc;                                         // next item to compute
     PhaseRegs ring[SLOTS];
 
-    // Prologue staging of x.  Loads return in issue order, so x is requested BEFORE the ring is
-    // filled: its latency is then that of an idle memory system.
-    uint4 xv[XUNITS];
-    load_x_slice(a, xv, (r0 + slice_of(cc) * CAP) * PHASE_K, slice_phases(slice_of(cc)), lane, wave);
-
-#pragma unroll
-    for (int j = 0; j < SLOTS; ++j) {
-        if (lc.valid && lc.slot == j) {
-            load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
-            advance(lc);
+    // Prologue.  Loads return in issue order, so x (slice 0 of the range) is requested BEFORE the
+    // ring is filled: its latency is then that of an idle memory system.  The work list is written
+    // next (one entry per thread), and the ring is filled from it while the table is built.
+    const int cn = ls.nitems;  // <= ITEMS_MAX, guaranteed by the launcher
+    {
+        uint4 xv[XUNITS];
+        const int nph0 = ls.nsl == 1 ? ls.last : CAP;
+        load_x_slice<R>(a, xv, ls.r0 * PHASE_K, nph0, lane, wave);
+        if (tid < cn) {
+            const Item it = make_item<CAP>(ls, tid);
+            reinterpret_cast<int4*>(smem + ITEMS_OFFSET)[tid] = make_int4(it.tg, it.kabs, it.info, it.k0);
         }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j) {
+            if (j < cn) {
+                const Item it = read_item(j);
+                if (!(it.info & ITEM_GAP)) load_phase<B64, NESTED>(a, ring[j], ll, first_row(it.tg), it.kabs);
+            }
+        }
+        if (EXACT)
+            build_pair_table_f32(smem, lut_lane, lane, wave);
+        else
+            build_pair_table(smem, lut_lane, lane, wave);
+        store_x_slice<R>(a, xv, smem + TABLE_BYTES, nph0, lane, wave);
+        __syncthreads();
     }
-    int resident = slice_of(cc);
-    store_x_slice<R>(a, xv, smem + TABLE_BYTES, slice_phases(resident), lane, wave);
-    if (EXACT)
-        build_pair_table_f32(smem, lut_lane, lane, wave);
-    else
-        build_pair_table(smem, lut_lane, lane, wave);
-    __syncthreads();
 
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + COUNTER_BYTES);
@@ -420,33 +498,44 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    while (cc.valid) {
-        const int fin_bi = cc.bi, fin_nb = cc.nb, fin_batch = cc.batch;
-#pragma unroll
-        for (int j = 0; j < SLOTS; ++j) {
-            if (cc.valid && cc.batch == fin_batch && cc.slot == j) {
-                if (cc.ph == 0 && cc.t == 0 && slice_of(cc) != resident) {
+    {
+        for (int base = 0; base < cn; base += SLOTS) {
+            int end_info = 0, end_tg = 0;
+            {
+                // a new slice always starts at slot 0
+                const Item it0 = read_item(base);
+                if (it0.info & ITEM_RESTAGE) {
+                    uint4 xv[XUNITS];
+                    const int n = (it0.info >> ITEM_NPH_SHIFT) & 0xf;
+                    load_x_slice<R>(a, xv, it0.k0, n, lane, wave);
                     __syncthreads();  // every wave is done with the slice that was resident
-                    resident = slice_of(cc);
-                    restage_x<R>(a, smem + TABLE_BYTES, (r0 + resident * CAP) * PHASE_K, slice_phases(resident), lane,
-                                 wave);
+                    store_x_slice<R>(a, xv, smem + TABLE_BYTES, n, lane, wave);
                     __syncthreads();
                 }
-                PhaseOperands o;
-                prepare_phase<B64, NESTED>(a, ring[j], lane, o);
-                // the slot's registers are free again: refill before the long part of the work
-                if (lc.valid && lc.slot == j) {
-                    load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
-                    advance(lc);
-                }
-                contract_phase<R, EXACT>(o, smem + TABLE_BYTES + cc.ph * (R * 1024), lane, acc[j]);
-                advance(cc);
-            } else if (lc.valid && lc.slot == j) {
-                load_phase<B64, NESTED>(a, ring[j], ll, first_row(lc), first_k(lc));
-                advance(lc);
             }
-        }
-        if (cc.batch == fin_batch) continue;
+#pragma unroll
+            for (int j = 0; j < SLOTS; ++j) {
+                const Item it = read_item(base + j);
+                Item nx;
+                nx.info = ITEM_GAP;
+                if (base + j + SLOTS < cn) nx = read_item(base + j + SLOTS);
+                if (!(it.info & ITEM_GAP)) {
+                    PhaseOperands o;
+                    prepare_phase<B64, NESTED>(a, ring[j], lane, o);
+                    // the slot's registers are free again: refill before the long part of the work
+                    if (!(nx.info & ITEM_GAP)) load_phase<B64, NESTED>(a, ring[j], ll, first_row(nx.tg), nx.kabs);
+                    contract_phase<R, EXACT>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane, acc[j]);
+                    if (it.info & ITEM_END) {
+                        end_info = it.info;
+                        end_tg = it.tg;
+                    }
+                } else if (!(nx.info & ITEM_GAP)) {
+                    load_phase<B64, NESTED>(a, ring[j], ll, first_row(nx.tg), nx.kabs);
+                }
+            }
+            if (!(end_info & ITEM_END)) continue;
+            const int fin_nb = (end_info >> ITEM_NB_SHIFT) & 7;
+            const int fin_tg0 = end_tg - (fin_nb - 1) * ls.tg_step;  // the batch's first tile group
 
         // ---- end of a batch: slot j holds tile group j % nb; lane holds out[m = 4g + i][row] ----
         if (fin_nb == 1) {
@@ -459,7 +548,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
 #pragma unroll
         for (int t = 0; t < SLOTS; ++t) {
             if (t < fin_nb) {
-                const int tile = (tg0 + (fin_bi + t) * p.tg_step) * WAVES + wave;
+                const int tile = (fin_tg0 + t * ls.tg_step) * WAVES + wave;
                 const int n0 = tile * 16;
                 const int n = max(min(n0, a.N - 16), 0) + col;  // the lane's row
                 const bool mine = n >= n0 && n < a.N;
@@ -507,7 +596,8 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                     }
                 }
             }
-            acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+                acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
         }
     }
 }
@@ -593,6 +683,16 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
     Plan p = make_plan(a.M, a.N, a.K);
     const int grid = grid_for((int64_t)p.tile_groups * p.splits, p.splits, cus < 1024 ? cus : 1024);
     p.tg_step = grid / p.splits;
+    // the longest work list of a workgroup (the one that owns the most tile groups and a full K range)
+    // must fit in LDS
+    {
+        const int cap = XBYTES_MAX / (rows_held(a.M) * 1024);
+        const int G = (p.tile_groups + p.tg_step - 1) / p.tg_step;
+        const int nsl = (p.range_phases + cap - 1) / cap;
+        const int last = p.range_phases - (nsl - 1) * cap;
+        const int n = rows_held(a.M) == 8 ? list_length<10>(G, nsl, last) : list_length<5>(G, nsl, last);
+        if (n > ITEMS_MAX) return hipErrorInvalidValue;
+    }
     if (gemv_wants_exact(a.K))
         return rows_held(a.M) == 8 ? launch_r<8, true>(a, p, grid, stream) : launch_r<16, true>(a, p, grid, stream);
     return rows_held(a.M) == 8 ? launch_r<8, false>(a, p, grid, stream) : launch_r<16, false>(a, p, grid, stream);

@@ -53,10 +53,9 @@ class LlamaConfig:
 
 
 def _rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    # x [B, T, heads, hd]; cos/sin [T, 1, hd] (each half repeated): x * cos + rotate_half(x) * sin, in fp32
-    xf = x.float()
-    x1, x2 = xf.chunk(2, dim=-1)
-    return torch.addcmul(xf * cos, torch.cat((-x2, x1), dim=-1), sin).to(x.dtype)
+    # x [B, T, heads, hd]; cos/sin [T, 1, hd] in x's dtype (each half repeated): x * cos + rotate_half(x) * sin
+    x1, x2 = x.chunk(2, dim=-1)
+    return torch.addcmul(x * cos, torch.cat((-x2, x1), dim=-1), sin)
 
 
 class Attention(nn.Module):
@@ -72,7 +71,7 @@ class Attention(nn.Module):
             self.v_proj = nn.Linear(cfg.d_model, cfg.n_kv_head * hd, bias=False)
         self.o_proj = nn.Linear(cfg.n_head * hd, cfg.d_model, bias=False)
 
-    def forward(self, x, pos, cos, sin, mask, kcache, vcache):
+    def forward(self, x, pos, cos, sin, bias, kcache, vcache):
         cfg = self.cfg
         B, T, _ = x.shape
         hd, H, Hkv = cfg.head_dim, cfg.n_head, cfg.n_kv_head
@@ -90,12 +89,14 @@ class Attention(nn.Module):
         # kv head become extra query rows of that head, row index r * T + t
         q = qk[:, :, :H].reshape(B, T, Hkv, rep, hd).permute(0, 2, 3, 1, 4).reshape(B, Hkv, rep * T, hd)
         if T == 1:
-            # one query per head: two small batched matmuls beat a general attention kernel
-            scores = torch.matmul(q, kcache.transpose(-1, -2)).float() * (hd ** -0.5)
-            scores = scores.masked_fill(~mask, float("-inf"))
-            y = torch.matmul(torch.softmax(scores, dim=-1).to(q.dtype), vcache)
+            # one query per head: two small batched matmuls beat a general attention kernel; the first
+            # one also applies the scale and the additive mask (0 / -inf)
+            scores = torch.baddbmm(bias.expand(B * Hkv, rep, -1), q.reshape(B * Hkv, rep, hd),
+                                   kcache.reshape(B * Hkv, -1, hd).transpose(1, 2), alpha=hd ** -0.5)
+            probs = torch.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
+            y = torch.bmm(probs, vcache.reshape(B * Hkv, -1, hd)).reshape(B, Hkv, rep, hd)
         else:
-            y = F.scaled_dot_product_attention(q, kcache, vcache, attn_mask=mask.repeat(rep, 1))
+            y = F.scaled_dot_product_attention(q, kcache, vcache, attn_mask=bias.repeat(rep, 1))
         y = y.reshape(B, Hkv, rep, T, hd).permute(0, 3, 1, 2, 4).reshape(B, T, H * hd)
         return self.o_proj(y)
 
@@ -127,8 +128,8 @@ class Block(nn.Module):
         self.norm_2 = nn.RMSNorm(cfg.d_model, eps=cfg.norm_eps)
         self.mlp = MLP(cfg)
 
-    def forward(self, x, pos, cos, sin, mask, kcache, vcache):
-        x = x + self.attn(self.norm_1(x), pos, cos, sin, mask, kcache, vcache)
+    def forward(self, x, pos, cos, sin, bias, kcache, vcache):
+        x = x + self.attn(self.norm_1(x), pos, cos, sin, bias, kcache, vcache)
         return x + self.mlp(self.norm_2(x))
 
 
@@ -150,12 +151,14 @@ class Llama(nn.Module):
         self.register_buffer("key_index", torch.arange(cfg.max_seq), persistent=False)
 
     def forward(self, idx, pos, kcache, vcache):
-        cos = self.rope_cos.index_select(0, pos)[:, None, :]
-        sin = self.rope_sin.index_select(0, pos)[:, None, :]
-        mask = self.key_index[None, :] <= pos[:, None]  # [T, max_seq]: key s visible to query at pos[t]
         x = self.wte(idx)
+        cos = self.rope_cos.index_select(0, pos)[:, None, :].to(x.dtype)
+        sin = self.rope_sin.index_select(0, pos)[:, None, :].to(x.dtype)
+        # additive attention mask [T, max_seq]: 0 where key s is visible to the query at pos[t], else -inf
+        visible = self.key_index[None, :] <= pos[:, None]
+        bias = torch.zeros(visible.shape, dtype=x.dtype, device=x.device).masked_fill(~visible, float("-inf"))
         for i, blk in enumerate(self.blocks):
-            x = blk(x, pos, cos, sin, mask, kcache[i], vcache[i])
+            x = blk(x, pos, cos, sin, bias, kcache[i], vcache[i])
         return self.lm_head(self.norm_f(x[:, -1:, :])).squeeze(1)
 
 

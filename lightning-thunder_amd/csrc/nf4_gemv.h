@@ -69,25 +69,6 @@ __device__ __forceinline__ float2 lds_table_read2(uint32_t addr) {
     return make_float2(v.x, v.y);
 }
 
-// Sum, in slice order, of the `splits` partial sums of one output (first one at p0, `stride` floats
-// apart).  The partial sums were written by other workgroups with agent-scope stores; the loads are
-// agent-scope too and are issued eight at a time before the first add, so that their latencies
-// overlap; the order of the adds is fixed.
-__device__ __forceinline__ float sum_partials(const float* p0, int64_t stride, int splits) {
-    float sum = 0.0f;
-    for (int k2 = 0; k2 < splits; k2 += 8) {
-        float v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            v[j] = k2 + j < splits
-                       ? __hip_atomic_load(p0 + (int64_t)(k2 + j) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                       : 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) sum += v[j];
-    }
-    return sum;
-}
-
 template <typename K>
 hipError_t gemv_allow_lds(K kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);

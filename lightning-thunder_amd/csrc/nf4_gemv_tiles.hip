@@ -431,11 +431,6 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
     ls.tg0 = (int)blockIdx.x / p.splits;
     ls.tg_step = p.tg_step;
     ls.r0 = ks * p.range_phases;                             // first phase of the range
-    ls.rph = min(p.range_phases, p.total_phases - ls.r0);    // phases in the range
-    ls.nsl = (ls.rph + CAP - 1) / CAP;                       // x slices in the range
-    ls.last = ls.rph - (ls.nsl - 1) * CAP;                   // phases of the last slice
-    ls.G = ls.tg0 < p.tile_groups ? (p.tile_groups - 1 - ls.tg0) / p.tg_step + 1 : 0;
-    ls.nitems = list_length<CAP>(ls.G, ls.nsl, ls.last);
 
     LaneLoad ll;
     {
@@ -466,6 +461,11 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
     // Prologue.  Loads return in issue order, so x (slice 0 of the range) is requested BEFORE the
     // ring is filled: its latency is then that of an idle memory system.  The work list is written
     // next (one entry per thread), and the ring is filled from it while the table is built.
+    ls.rph = min(p.range_phases, p.total_phases - ls.r0);    // phases in the range
+    ls.nsl = (ls.rph + CAP - 1) / CAP;                       // x slices in the range
+    ls.last = ls.rph - (ls.nsl - 1) * CAP;                   // phases of the last slice
+    ls.G = ls.tg0 < p.tile_groups ? (p.tile_groups - 1 - ls.tg0) / p.tg_step + 1 : 0;
+    ls.nitems = list_length<CAP>(ls.G, ls.nsl, ls.last);
     const int cn = ls.nitems;  // <= ITEMS_MAX, guaranteed by the launcher
     {
         uint4 xv[XUNITS];
@@ -582,13 +582,39 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                         prev = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     prev = __builtin_amdgcn_readfirstlane(prev);
                     if (prev == (unsigned)p.splits - 1u) {
-                        for (int idx = lane; idx < 16 * a.M; idx += 64) {
-                            const int m = idx >> 4;
-                            const int nn = n0 + (idx & 15);
-                            if (nn < a.N) {
-                                float sum = sum_partials(&partial[(int64_t)m * a.N + nn], (int64_t)a.M * a.N, p.splits);
-                                if (a.bias) sum += bf16_bits_to_f32(a.bias[nn]);
-                                a.out[(int64_t)m * a.N + nn] = (uint16_t)f32_to_bf16_bits(sum);
+                        // the lane's R / 4 outputs of the 16 x M tile; the loads of eight slices of all
+                        // of them are in flight together, the adds run in slice order
+                        constexpr int OUTS = R / 4;
+                        const int nn = n0 + col;
+                        const float* p0[OUTS];
+                        float sum[OUTS];
+#pragma unroll
+                        for (int o = 0; o < OUTS; ++o) {
+                            const int m = min(g + 4 * o, a.M - 1);
+                            p0[o] = &partial[(int64_t)m * a.N + min(nn, a.N - 1)];
+                            sum[o] = 0.0f;
+                        }
+                        const int64_t stride = (int64_t)a.M * a.N;
+                        for (int k2 = 0; k2 < p.splits; k2 += 8) {
+                            float v[OUTS][8];
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                const int64_t off = (int64_t)min(k2 + j, p.splits - 1) * stride;
+#pragma unroll
+                                for (int o = 0; o < OUTS; ++o)
+                                    v[o][j] = __hip_atomic_load(p0[o] + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+#pragma unroll
+                            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                                for (int o = 0; o < OUTS; ++o) sum[o] += k2 + j < p.splits ? v[o][j] : 0.0f;
+                        }
+                        if (nn < a.N) {
+                            const float b = a.bias ? bf16_bits_to_f32(a.bias[nn]) : 0.0f;
+#pragma unroll
+                            for (int o = 0; o < OUTS; ++o) {
+                                const int m = g + 4 * o;
+                                if (m < a.M) a.out[(int64_t)m * a.N + nn] = (uint16_t)f32_to_bf16_bits(sum[o] + b);
                             }
                         }
                         if (lane == 0)

@@ -69,6 +69,26 @@ __device__ __forceinline__ float2 lds_table_read2(uint32_t addr) {
     return make_float2(v.x, v.y);
 }
 
+// One stage of the in-quad transpose: lanes whose `bit` is 0 keep A and receive the partner's A
+// into B; lanes whose bit is 1 keep B and receive the partner's B into A.
+template <int DPP_CTRL>
+__device__ __forceinline__ void quad_exchange(uint32_t& A, uint32_t& B, bool bit) {
+    const uint32_t pa = (uint32_t)__builtin_amdgcn_update_dpp((int)A, (int)A, DPP_CTRL, 0xf, 0xf, true);
+    const uint32_t pb = (uint32_t)__builtin_amdgcn_update_dpp((int)B, (int)B, DPP_CTRL, 0xf, 0xf, true);
+    A = bit ? pb : A;
+    B = bit ? B : pa;
+}
+
+// 4x4 transpose of r[0..3] across the four lanes of a quad: afterwards r[i] of lane q holds what
+// r[q] of lane i (of the same quad) held.
+__device__ __forceinline__ void transpose_quad(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3, bool b0,
+                                               bool b1) {
+    quad_exchange<0xB1>(r0, r1, b0);  // quad_perm [1,0,3,2]
+    quad_exchange<0xB1>(r2, r3, b0);
+    quad_exchange<0x4E>(r0, r2, b1);  // quad_perm [2,3,0,1]
+    quad_exchange<0x4E>(r1, r3, b1);
+}
+
 template <typename K>
 hipError_t gemv_allow_lds(K kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);

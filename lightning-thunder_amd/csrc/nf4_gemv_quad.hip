@@ -13,7 +13,9 @@
 //  * v_mfma_f32_4x4x4_16b_bf16 computes one 4x4x4 product per group of 4 lanes: A row i comes from
 //    lane i of the quad (4 weights of weight-row i), B column j from lane j (4 values of x row j at
 //    the same k).  C[i][j] = weight-row i . x-row j, so ALL 16 results of the quad are wanted and
-//    M = 2, 3, 4 cost exactly what M = 1 costs.  Lane j keeps x row j in registers (rows >= M: 0).
+//    M = 2, 3, 4 cost exactly what M = 1 costs.  Lane j keeps x row j in registers (rows >= M: 0);
+//    a workgroup keeps one K split for all its tasks, so x is read once per kernel, in contiguous
+//    1 KB requests, and put into that layout by a 4x4 transpose inside every quad.
 //  * Code -> bf16: 256-entry LDS table indexed by a whole packed byte, both code values as one
 //    dword, replicated per lane with a 256-byte stride: address (byte << 8) | lane*4 is one
 //    v_perm_b32 and bank-conflict free.
@@ -26,6 +28,8 @@
 //  * K larger than one workgroup covers is split over workgroups; partial sums cross workgroups
 //    through agent-scope relaxed atomics and a counter (no L2-wide fences), added in a fixed order
 //    by the last workgroup to arrive.
+#include <type_traits>
+
 #include "nf4_gemv.h"
 
 namespace nf4 {
@@ -98,7 +102,6 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
 
     // the code-book entry this lane contributes to the LDS table: requested first, used last
     const float lut_mine = a.lut16[lane & 15];
-    bool table_built = false;
 
     float* part = reinterpret_cast<float*>(smem + GEMV_TABLE_BYTES);
     int* flag = reinterpret_cast<int*>(smem + FLAG_OFFSET);
@@ -111,28 +114,22 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
     const int M = a.M;
     const int step = p.row_groups;
 
-    for (int task = blockIdx.x; task < p.ntasks; task += gridDim.x) {
+    // The grid is a multiple of the number of K splits, so every task of this workgroup has the same
+    // split and x is read once, with the first task.
+    const int ks = (int)blockIdx.x % p.splits;
+    const int64_t kw0 = (int64_t)(ks * p.waves_k + cw) * (CPW * LOAD_K);
+    uint32_t xr[CPW][16];  // x row `ri`, this lane's 32 k of every load
+
+    auto run_task = [&](const int task, auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
         const int band = task / p.splits;
-        const int ks = task - band * p.splits;
         const int g_begin = band * p.groups_per_band;
         const int g_end = min((a.N + 3) / 4, g_begin + p.groups_per_band);
-        const int64_t kw0 = (int64_t)(ks * p.waves_k + cw) * (CPW * LOAD_K);
         const bool wave_on = rg < p.row_groups && kw0 < K && g_begin + rg < g_end;
         const int cnt = wave_on ? (g_end - g_begin - rg + step - 1) / step : 0;  // groups of this wave
         bool lane_on[CPW];
 #pragma unroll
         for (int c = 0; c < CPW; ++c) lane_on[c] = wave_on && kw0 + c * LOAD_K + kseg < K;
-
-        // x row `ri`, this lane's 32 k of every load
-        uint32_t xr[CPW][16];
-#pragma unroll
-        for (int c = 0; c < CPW; ++c)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (lane_on[c] && ri < M) v = *reinterpret_cast<const uint4*>(a.x + ri * K + kw0 + c * LOAD_K + kseg + 8 * q);
-                xr[c][4 * q + 0] = v.x; xr[c][4 * q + 1] = v.y; xr[c][4 * q + 2] = v.z; xr[c][4 * q + 3] = v.w;
-            }
 
         // sq: absmax of the lane's block; nested: its 8-bit code (resolved through the LDS copy of
         // the map when the slot is consumed, so that issuing a load never waits for another) and
@@ -166,20 +163,70 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                     }
                 }
         };
+        // First task: x.  Row by row, lane l takes elements [8 l, 8 l + 8) of the load's 512: one
+        // contiguous 1 KB per request.  (Every lane reading its own 64 bytes would touch 64 cache lines
+        // per request instead of 16, and with 16 waves per CU the address unit would then pace the
+        // whole kernel.)  These requests go out ahead of the weights: they are served by the L2 while
+        // the first weights are on their way from HBM.
+        // With two rows of x the transpose costs more than it saves: every lane then reads its own 64
+        // bytes (piece q of row `ri` lands in xraw[c][q]).
+        const bool direct_x = M <= 2;
+        uint4 xraw[CPW][4];
+        float lut = lut_mine;
+        if constexpr (FIRST) {
+            // The wait for the code-book entry belongs here, where nothing else is in flight: the
+            // loads below sit under branches, so a wait placed after them would be for all of them,
+            // and the table is to be built while they are in flight.
+            asm volatile("" : "+v"(lut));
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) {
+                // a lane beyond K (or an idle wave) reads the end of the row; the value is dropped below
+                const int64_t kc = kw0 + c * LOAD_K + (direct_x ? (int64_t)kseg : (int64_t)(8 * lane));
+                const uint16_t* xb = a.x + min(kc, K - (direct_x ? 32 : 8));
+                if (direct_x) xb += (int64_t)min(ri, M - 1) * K;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)  // transposed path, rows >= M: every lane reads x[0]
+                    xraw[c][r] = load16(direct_x ? xb + 8 * r : (r < M ? xb + (int64_t)r * K : a.x));
+            }
+        }
         // get the weight stream going before anything else happens
 #pragma unroll
         for (int u = 0; u < U; ++u)
             if (u < cnt) issue(u, u);
 
-        if (!table_built) {  // first task only: overlaps with the loads above
+        // first task: the table is built while the loads are in flight
+        if constexpr (FIRST) {
             if (EXACT)
-                build_pair_table_f32(smem, lut_mine, lane, wave);
+                build_pair_table_f32(smem, lut, lane, wave);
             else
-                build_pair_table(smem, lut_mine, lane, wave);
+                build_pair_table(smem, lut, lane, wave);
             if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
-            table_built = true;
         }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
+        if constexpr (FIRST) {
+            // The four lanes of a quad hold the quad's 32 k of rows 0..3 in four pieces each; a 4x4
+            // transpose inside the quad hands lane `ri` the four pieces of row `ri`.
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) {
+                const bool in = rg < p.row_groups && kw0 + c * LOAD_K + (direct_x ? (int64_t)kseg : (int64_t)(8 * lane)) < K;
+                uint32_t v[4][4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool keep = in && (direct_x ? ri < M : r < M);
+                    v[r][0] = keep ? xraw[c][r].x : 0u; v[r][1] = keep ? xraw[c][r].y : 0u;
+                    v[r][2] = keep ? xraw[c][r].z : 0u; v[r][3] = keep ? xraw[c][r].w : 0u;
+                }
+                if (!direct_x) {
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        transpose_quad(v[0][d], v[1][d], v[2][d], v[3][d], lane & 1, lane & 2);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) xr[c][4 * j + d] = v[j][d];
+            }
+        }
 
         for (int i0 = 0; i0 < cnt; i0 += U) {
 #pragma unroll
@@ -290,6 +337,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 if (tid == 0) __hip_atomic_store(&counters[band], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+    };
+
+    int task = blockIdx.x;
+    if (task < p.ntasks) {
+        run_task(task, std::true_type{});
+        for (task += gridDim.x; task < p.ntasks; task += gridDim.x) run_task(task, std::false_type{});
     }
 }
 
@@ -388,7 +441,9 @@ hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {
     int slots = 2 * cus;
     if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
     const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
-    const int grid = p.ntasks < slots ? p.ntasks : slots;
+    int grid = p.ntasks < slots ? p.ntasks : slots;
+    grid -= grid % p.splits;  // every workgroup keeps one K split (ntasks is a multiple of splits)
+    if (grid < p.splits) grid = p.splits;
     return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
 }
 

@@ -1,4 +1,4 @@
-// Pieces shared by the two decode-shape kernels (row-streaming for M <= 4, MFMA tiles for M <= 16).
+// Pieces shared by the three decode-shape kernels (row-streaming, four weight rows per lane quad, MFMA tiles).
 #pragma once
 
 #include "nf4_common.h"
@@ -99,12 +99,12 @@ size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_rows_setup();
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream);
 
-// four-rows-per-quad kernel, 2 <= M <= 4 (nf4_gemv_quad.hip)
+// four-weight-rows-per-quad kernel, 2 <= M <= 8 (nf4_gemv_quad.hip)
 size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_quad_setup();
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream);
 
-// MFMA tile kernel, 5 <= M <= 16 (nf4_gemv.hip)
+// MFMA tile kernel, 5 <= M <= 16 (nf4_gemv_tiles.hip)
 size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_tiles_setup();
 hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream);

@@ -1,6 +1,7 @@
 // Dispatch of the decode-shape fused NF4 dequant-matmul (M <= 16) between its three kernels:
-// row-streaming (M = 1, nf4_gemv_rows.hip), four rows per lane quad (M = 2..4,
-// nf4_gemv_quad.hip) and MFMA tiles (M = 5..16, nf4_gemv_tiles.hip).
+// row-streaming (M = 1, nf4_gemv_rows.hip), four weight rows per lane quad (M = 2..4, and M = 5..8
+// on weights of at most 2^26 elements, nf4_gemv_quad.hip) and MFMA tiles (the rest up to M = 16,
+// nf4_gemv_tiles.hip).
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -32,13 +33,17 @@ hipError_t device_setup(int* cus_out) {
     return hipSuccess;
 }
 
+// Five to eight rows of x: the quad kernel starts faster (no x staging, no global split of K below
+// 8192), the tile kernel streams faster once the weights are large; they cross near 2^26 weights.
+bool quad_serves(int64_t M, int64_t N, int64_t K) { return M <= 4 || (M <= 8 && N * K <= ((int64_t)1 << 26)); }
+
 }  // namespace
 
 // ---- dispatch -------------------------------------------------------------------------------
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M == 1) return gemv_rows_workspace_bytes(M, N, K);
-    return M <= 4 ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
+    return quad_serves(M, N, K) ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
 }
 
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
@@ -46,7 +51,7 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;
     if (a.M == 1) return launch_gemv_rows(a, cus, stream);
-    return a.M <= 4 ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
+    return quad_serves(a.M, a.N, a.K) ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
 }
 
 }  // namespace nf4

@@ -1,4 +1,4 @@
-// Decode-shape fused NF4 dequant-matmul for gfx950, 2 <= M <= 4 rows of x.
+// Decode-shape fused NF4 dequant-matmul for gfx950, 2 <= M <= 8 rows of x.
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -16,6 +16,8 @@
 //    M = 2, 3, 4 cost exactly what M = 1 costs.  Lane j keeps x row j in registers (rows >= M: 0);
 //    a workgroup keeps one K split for all its tasks, so x is read once per kernel, in contiguous
 //    1 KB requests, and put into that layout by a 4x4 transpose inside every quad.
+//    M = 5..8 (XS = 2): lane j also keeps x row j + 4, and every dequantised weight fragment feeds a
+//    second MFMA; a wave then covers 512 k instead of 1024 to stay within 128 registers.
 //  * Code -> bf16: 256-entry LDS table indexed by a whole packed byte, both code values as one
 //    dword, replicated per lane with a 256-byte stride: address (byte << 8) | lane*4 is one
 //    v_perm_b32 and bank-conflict free.
@@ -89,7 +91,7 @@ __device__ __forceinline__ float reduce_rows(const float t[4], int lane) {
     return y;
 }
 
-template <int CPW, int U, bool NESTED, bool EXACT>
+template <int CPW, int U, int XS, bool NESTED, bool EXACT>
 __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a, QuadPlan p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
     // split and x is read once, with the first task.
     const int ks = (int)blockIdx.x % p.splits;
     const int64_t kw0 = (int64_t)(ks * p.waves_k + cw) * (CPW * LOAD_K);
-    uint32_t xr[CPW][16];  // x row `ri`, this lane's 32 k of every load
+    uint32_t xr[XS][CPW][16];  // x rows `ri`, `ri + 4`, ...: this lane's 32 k of every load
 
     auto run_task = [&](const int task, auto first_tag) {
         constexpr bool FIRST = decltype(first_tag)::value;
@@ -169,9 +171,9 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
         // whole kernel.)  These requests go out ahead of the weights: they are served by the L2 while
         // the first weights are on their way from HBM.
         // With two rows of x the transpose costs more than it saves: every lane then reads its own 64
-        // bytes (piece q of row `ri` lands in xraw[c][q]).
-        const bool direct_x = M <= 2;
-        uint4 xraw[CPW][4];
+        // bytes (piece q of row `ri` lands in xraw[0][c][q]).
+        const bool direct_x = XS == 1 && M <= 2;
+        uint4 xraw[XS][CPW][4];
         float lut = lut_mine;
         if constexpr (FIRST) {
             // The wait for the code-book entry belongs here, where nothing else is in flight: the
@@ -185,8 +187,11 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 const uint16_t* xb = a.x + min(kc, K - (direct_x ? 32 : 8));
                 if (direct_x) xb += (int64_t)min(ri, M - 1) * K;
 #pragma unroll
-                for (int r = 0; r < 4; ++r)  // transposed path, rows >= M: every lane reads x[0]
-                    xraw[c][r] = load16(direct_x ? xb + 8 * r : (r < M ? xb + (int64_t)r * K : a.x));
+                for (int h = 0; h < XS; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)  // transposed path, rows >= M: every lane reads x[0]
+                        xraw[h][c][r] =
+                            load16(direct_x ? xb + 8 * r : (4 * h + r < M ? xb + (int64_t)(4 * h + r) * K : a.x));
             }
         }
         // get the weight stream going before anything else happens
@@ -204,34 +209,41 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
         }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
         if constexpr (FIRST) {
-            // The four lanes of a quad hold the quad's 32 k of rows 0..3 in four pieces each; a 4x4
-            // transpose inside the quad hands lane `ri` the four pieces of row `ri`.
+            // The four lanes of a quad hold the quad's 32 k of rows 4h..4h+3 in four pieces each; a 4x4
+            // transpose inside the quad hands lane `ri` the four pieces of row 4h + `ri`.
 #pragma unroll
-            for (int c = 0; c < CPW; ++c) {
-                const bool in = rg < p.row_groups && kw0 + c * LOAD_K + (direct_x ? (int64_t)kseg : (int64_t)(8 * lane)) < K;
-                uint32_t v[4][4];
+            for (int h = 0; h < XS; ++h)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const bool keep = in && (direct_x ? ri < M : r < M);
-                    v[r][0] = keep ? xraw[c][r].x : 0u; v[r][1] = keep ? xraw[c][r].y : 0u;
-                    v[r][2] = keep ? xraw[c][r].z : 0u; v[r][3] = keep ? xraw[c][r].w : 0u;
+                for (int c = 0; c < CPW; ++c) {
+                    const bool in =
+                        rg < p.row_groups && kw0 + c * LOAD_K + (direct_x ? (int64_t)kseg : (int64_t)(8 * lane)) < K;
+                    uint32_t v[4][4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const bool keep = in && (direct_x ? ri < M : 4 * h + r < M);
+                        v[r][0] = keep ? xraw[h][c][r].x : 0u; v[r][1] = keep ? xraw[h][c][r].y : 0u;
+                        v[r][2] = keep ? xraw[h][c][r].z : 0u; v[r][3] = keep ? xraw[h][c][r].w : 0u;
+                    }
+                    if (!direct_x) {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d)
+                            transpose_quad(v[0][d], v[1][d], v[2][d], v[3][d], lane & 1, lane & 2);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) xr[h][c][4 * j + d] = v[j][d];
                 }
-                if (!direct_x) {
-#pragma unroll
-                    for (int d = 0; d < 4; ++d)
-                        transpose_quad(v[0][d], v[1][d], v[2][d], v[3][d], lane & 1, lane & 2);
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int d = 0; d < 4; ++d) xr[c][4 * j + d] = v[j][d];
-            }
         }
 
         for (int i0 = 0; i0 < cnt; i0 += U) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                float tot[4] = {0.f, 0.f, 0.f, 0.f};
+                float tot[XS][4];
+#pragma unroll
+                for (int h = 0; h < XS; ++h)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) tot[h][i] = 0.0f;
                 // take the slot's contents, then refill it at once: the load is in flight while the
                 // table lookups and MFMAs below run
                 uint32_t dd[CPW][4];
@@ -265,29 +277,36 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                                 pr[4 * q + j] = lds_table_read(__builtin_amdgcn_perm(d[q], lane4, sel));
                             }
                         }
-                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const uint2 wa = make_uint2(pr[2 * t], pr[2 * t + 1]);
-                        const uint2 xb = make_uint2(xr[c][2 * t], xr[c][2 * t + 1]);
-                        acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
-                                                                     __builtin_bit_cast(s16x4, xb), acc, 0, 0, 0);
-                    }
-                    if (EXACT) {
+                    for (int h = 0; h < XS; ++h) {  // the dequantised weights serve every set of four x rows
+                        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) tot[i] += acc[i];
-                    } else {
-                        // acc[i] belongs to weight row i, whose absmax lane i of this quad holds
-                        tot[0] = fmaf(NF4_QUAD_BCAST(s, 0x00), acc[0], tot[0]);
-                        tot[1] = fmaf(NF4_QUAD_BCAST(s, 0x55), acc[1], tot[1]);
-                        tot[2] = fmaf(NF4_QUAD_BCAST(s, 0xAA), acc[2], tot[2]);
-                        tot[3] = fmaf(NF4_QUAD_BCAST(s, 0xFF), acc[3], tot[3]);
+                        for (int t = 0; t < 8; ++t) {
+                            const uint2 wa = make_uint2(pr[2 * t], pr[2 * t + 1]);
+                            const uint2 xb = make_uint2(xr[h][c][2 * t], xr[h][c][2 * t + 1]);
+                            acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
+                                                                         __builtin_bit_cast(s16x4, xb), acc, 0, 0, 0);
+                        }
+                        if (EXACT) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) tot[h][i] += acc[i];
+                        } else {
+                            // acc[i] belongs to weight row i, whose absmax lane i of this quad holds
+                            tot[h][0] = fmaf(NF4_QUAD_BCAST(s, 0x00), acc[0], tot[h][0]);
+                            tot[h][1] = fmaf(NF4_QUAD_BCAST(s, 0x55), acc[1], tot[h][1]);
+                            tot[h][2] = fmaf(NF4_QUAD_BCAST(s, 0xAA), acc[2], tot[h][2]);
+                            tot[h][3] = fmaf(NF4_QUAD_BCAST(s, 0xFF), acc[3], tot[h][3]);
+                        }
                     }
                 }
-                const float total = reduce_rows(tot, lane);  // lanes 0..15: row 2*b3+b2 of the group, x row ri
                 const int grow = 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);
-                if (lane < 16 && ri < M && i < cnt)
-                    part[(((rg + i * step) * 4 + grow) * p.waves_k + cw) * M + ri] = total;
+#pragma unroll
+                for (int h = 0; h < XS; ++h) {
+                    // lanes 0..15: row 2*b3+b2 of the group, x row 4h + ri
+                    const float total = reduce_rows(tot[h], lane);
+                    if (lane < 16 && 4 * h + ri < M && i < cnt)
+                        part[(((rg + i * step) * 4 + grow) * p.waves_k + cw) * M + 4 * h + ri] = total;
+                }
             }
         }
         __syncthreads();
@@ -348,10 +367,11 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
 
 // k per wave = 512 * CPW.  Two loads per lane and row group keep x in 32 registers; one workgroup
 // (8 waves) then covers K <= 8192, larger K is split over workgroups.
-int pick_cpw(int64_t K) { return K <= 2 * LOAD_K ? 1 : 2; }
+// Five to eight rows of x take twice the registers per load, so a wave then keeps one load's worth.
+int pick_cpw(int64_t M, int64_t K) { return (M > 4 || K <= 2 * LOAD_K) ? 1 : 2; }
 
-int quad_splits(int64_t K) {
-    const int64_t wave_k = (int64_t)pick_cpw(K) * LOAD_K;
+int quad_splits(int64_t M, int64_t K) {
+    const int64_t wave_k = (int64_t)pick_cpw(M, K) * LOAD_K;
     const int64_t nwk = (K + wave_k - 1) / wave_k;
     return (int)((nwk + GEMV_WAVES - 1) / GEMV_WAVES);
 }
@@ -359,9 +379,9 @@ int quad_splits(int64_t K) {
 QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested) {
     QuadPlan p;
     p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
-    const int64_t wave_k = (int64_t)pick_cpw(K) * LOAD_K;
+    const int64_t wave_k = (int64_t)pick_cpw(M, K) * LOAD_K;
     const int nwk = (int)((K + wave_k - 1) / wave_k);
-    p.splits = quad_splits(K);
+    p.splits = quad_splits(M, K);
     p.waves_k = (nwk + p.splits - 1) / p.splits;
     p.row_groups = GEMV_WAVES / p.waves_k;
     const int groups = (int)((N + 3) / 4);
@@ -386,55 +406,58 @@ QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
     return p;
 }
 
-template <int CPW, int U, bool NESTED>
+template <int CPW, int U, int XS, bool NESTED>
 hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
     if (gemv_wants_exact(a.K))
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, NESTED, true>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, true>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, NESTED, false>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, false>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
-// U = row groups in flight per wave: U * CPW 16-byte loads per lane, at most 8
-template <int CPW, bool NESTED>
+// U = row groups in flight per wave: U * CPW 16-byte loads per lane, at most 8 (4 with eight rows of x)
+template <int CPW, int XS, bool NESTED>
 hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
     const int cnt = p.groups_per_band / p.row_groups;  // groups per wave and task
-    constexpr int UMAX = 8 / CPW;
+    constexpr int UMAX = 8 / (CPW * XS);
     if constexpr (UMAX >= 8)
-        if (cnt >= 8) return launch_u<CPW, 8, NESTED>(a, p, grid, stream);
+        if (cnt >= 8) return launch_u<CPW, 8, XS, NESTED>(a, p, grid, stream);
     if constexpr (UMAX >= 4 && !(NESTED && CPW == 2))  // nested: one more register per load in flight
-        if (cnt >= 4) return launch_u<CPW, 4, NESTED>(a, p, grid, stream);
-    return launch_u<CPW, 2, NESTED>(a, p, grid, stream);
+        if (cnt >= 4) return launch_u<CPW, 4, XS, NESTED>(a, p, grid, stream);
+    return launch_u<CPW, 2, XS, NESTED>(a, p, grid, stream);
 }
 
 template <bool NESTED>
 hipError_t launch_n(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
-    return pick_cpw(a.K) == 1 ? launch_c<1, NESTED>(a, p, grid, stream) : launch_c<2, NESTED>(a, p, grid, stream);
+    if (a.M > 4) return launch_c<1, 2, NESTED>(a, p, grid, stream);
+    return pick_cpw(a.M, a.K) == 1 ? launch_c<1, 1, NESTED>(a, p, grid, stream) : launch_c<2, 1, NESTED>(a, p, grid, stream);
 }
 
-template <int CPW, int U>
+template <int CPW, int U, int XS>
 hipError_t allow_lds_cu() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, false, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, true, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, false, true>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_quad_kernel<CPW, U, true, true>, SMEM_BYTES);
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, true>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, true>, SMEM_BYTES);
 }
 
 }  // namespace
 
 size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    const int s = quad_splits(K);
+    const int s = quad_splits(M, K);
     return (size_t)GEMV_COUNTER_BYTES + (s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0);
 }
 
 hipError_t gemv_quad_setup() {
     hipError_t e;
-    if ((e = allow_lds_cu<1, 8>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<1, 4>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<1, 2>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<2, 4>()) != hipSuccess) return e;
-    return allow_lds_cu<2, 2>();
+    if ((e = allow_lds_cu<1, 8, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<1, 4, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<1, 2, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<2, 4, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<2, 2, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<1, 4, 2>()) != hipSuccess) return e;
+    return allow_lds_cu<1, 2, 2>();
 }
 
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {

@@ -366,7 +366,7 @@ def test_full_size_properties(ta):
 @pytest.mark.parametrize("N,K", [(8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672)])
 def test_llama70b_shapes_double_quant(ta, N, K):
     """Llama-3-70B projection shapes with 8-bit double-quantized absmax (nested blocksize 256 plus
-    offset), M in {1, 16, 2048}, at full size: every route against a float64-accumulated matmul over
+    offset), M in {1, 4, 8, 16, 2048}, at full size: every route against a float64-accumulated matmul over
     the HIP-dequantized weight (itself pinned bit-exact against the oracle at small sizes), and the
     fused kernels' nested path against their fp32-absmax path on the reconstructed absmax."""
     _sync_print(f"70B double-quant N={N} K={K}")
@@ -378,7 +378,7 @@ def test_llama70b_shapes_double_quant(ta, N, K):
     deq = ta.dequantize_nf4(qw, nested, code, 64, torch.bfloat16, (N, K))
     assert torch.equal(deq, ta.dequantize_nf4(qw, absmax_rec, code, 64, torch.bfloat16, (N, K)))
     rows = torch.randint(0, N, (64,), generator=g, device=DEV)
-    for M in (1, 16, 2048):
+    for M in (1, 4, 8, 16, 2048):
         x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
         y = ta.matmul_nf4(x, qw, None, nested, code, 64, torch.bfloat16, (N, K))
         ref = x.double() @ deq[rows].double().t()
@@ -386,6 +386,27 @@ def test_llama70b_shapes_double_quant(ta, N, K):
         if M <= 16:
             y2 = ta.matmul_nf4(x, qw, None, absmax_rec, code, 64, torch.bfloat16, (N, K))
             assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("N,K", [(28672, 4096), (128256, 4096), (16384 + 16, 4096)])
+def test_gemv_five_to_eight_rows_on_large_weights(ta, N, K):
+    """M = 5..8 is served by the quad kernel up to 2^26 weights and by the MFMA tile kernel beyond
+    (fused gate/up projection, lm_head, and a shape just past the switch with a ragged last tile):
+    at full size against a float64-accumulated matmul over sampled rows of the HIP-dequantized weight,
+    which is itself pinned bit-exact against the oracle at small sizes."""
+    _sync_print(f"gemv M=5..8 large N={N} K={K}")
+    g = torch.Generator(device=DEV).manual_seed(N + K)
+    w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    qw, absmax, code = ta.quantize_nf4(w)
+    deq = ta.dequantize_nf4(qw, absmax, code, 64, torch.bfloat16, (N, K))
+    rows = torch.cat([torch.randint(0, N, (61,), generator=g, device=DEV), torch.tensor([0, N - 2, N - 1], device=DEV)])
+    bias = torch.randn(N, generator=g, device=DEV).to(torch.bfloat16)
+    for M in (5, 6, 7, 8):
+        x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+        assert ta.functional.fused_route(x, bias, 64, torch.bfloat16, (N, K)) == "gemv"
+        y = ta.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))
+        ref = x.double() @ deq[rows].double().t() + bias[rows].double()
+        torch.testing.assert_close(y[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("M", [1, 3, 8, 16])

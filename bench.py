@@ -110,14 +110,14 @@ def main() -> int:
     group_bytes = [sum(algorithmic_bytes(*c) for c in calls) for _, _, calls in groups]
     bytes_step = sum(group_bytes)
 
-    def step(it, ev=None):
+    # one chain of events over the timed region: event s * G + g opens group g of step s and closes
+    # the group before it (a record between two launches costs a few microseconds of the stream)
+    def step(it, ev=None, s=0):
         for gi, (_, _, calls) in enumerate(groups):
             if ev:
-                ev[gi].record(stream)
+                ev[s * len(groups) + gi].record(stream)
             for c in calls:
                 launch(*c, it)
-        if ev:
-            ev[len(groups)].record(stream)
 
     # A plain device copy of known size (256 MiB read + 256 MiB written), outside the timed region:
     # hardware-counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) are scaled by what the same
@@ -129,11 +129,12 @@ def main() -> int:
 
     for it in range(args.warmup):
         step(it)
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(len(groups) + 1)] for _ in range(args.steps)]
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(len(groups) * args.steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for it in range(args.steps):
-        step(args.warmup + it, events[it])
+        step(args.warmup + it, events, it)
+    events[-1].record(stream)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
@@ -142,7 +143,8 @@ def main() -> int:
     value = bytes_step * args.steps / wall / 1e9
     kernels = []
     for gi, (name, what, calls) in enumerate(groups):
-        ms = sum(ev[gi].elapsed_time(ev[gi + 1]) for ev in events) / args.steps
+        G = len(groups)
+        ms = sum(events[st * G + gi].elapsed_time(events[st * G + gi + 1]) for st in range(args.steps)) / args.steps
         kernels.append({
             "kernel": name, "calls": what, "launches_per_step": len(calls),
             "algorithmic_bytes_per_launch": group_bytes[gi] // len(calls),

@@ -52,7 +52,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU baseline sample (0 disables)")
-    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-regime section (BASELINE config 3)")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-regime section (BASELINE config 3) and the quantize/dequantize bandwidth section")
     ap.add_argument("--decode-tokens", type=int, default=128,
                     help="tokens of the Llama-3-8B greedy decode that follows the GEMV pass (0 disables)")
     args = ap.parse_args()
@@ -198,6 +198,7 @@ def main() -> int:
     torch.cuda.empty_cache()
     if not args.no_prefill:
         result["config"]["prefill"] = prefill_section(torch, ta)
+        result["config"]["codec"] = codec_section(torch, ta)
     if args.decode_tokens > 1:
         result["config"]["decode"] = llama_decode(torch, ta, args.decode_tokens)
     if args.cpu_seconds > 0:
@@ -255,6 +256,60 @@ def prefill_section(torch, ta) -> dict:
                              "tflops": round(2.0 * M * N * K / t / 1e12, 1),
                              "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
     return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows}
+
+
+def codec_section(torch, ta) -> dict:
+    """The two HBM-bound conversion kernels, outside the timed region of the GEMV metric: quantize
+    (bf16 -> NF4) and dequantize (NF4 -> bf16) of one Llama-3-8B FFN weight and of the lm_head, cold
+    (a ring of distinct buffers larger than the 256 MB Infinity Cache).  GB/s over the algorithmic
+    bytes: 2n read + n/2 + n/16 written, and n/2 + n/16 + 64 read + 2n written."""
+    dev = torch.device("cuda:0")
+    code = ta.nf4_code(dev)
+    out = {}
+    for N, K in [(14336, 4096), (128256, 4096)]:
+        n = N * K
+        ncopy = max(2, (640 << 20) // (2 * n) + 1)
+        g = torch.Generator(device=dev).manual_seed(N)
+        ws = [(torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16) for _ in range(ncopy)]
+        packed = [ta.quantize_nf4(w, BLOCKSIZE) for w in ws]
+        torch.cuda.synchronize()
+
+        def timed(fn, reps=2 * ncopy):
+            for i in range(ncopy):
+                fn(i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(reps):
+                fn(i % ncopy)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / reps
+
+        # through the C ABI with preallocated outputs: the kernels, not the allocator
+        lib = ta._lib.load()
+        sptr = torch.cuda.current_stream().cuda_stream
+        qout = torch.empty(n // 2, dtype=torch.uint8, device=dev)
+        aout = torch.empty(n // BLOCKSIZE, dtype=torch.float32, device=dev)
+        wout = torch.empty(N, K, dtype=torch.bfloat16, device=dev)
+
+        def quant(i):
+            ta._lib.check(lib.nf4hip_quantize(ws[i].data_ptr(), ta._lib.BF16, n, BLOCKSIZE, qout.data_ptr(), aout.data_ptr(), sptr))
+
+        def dequant(i):
+            ta._lib.check(lib.nf4hip_dequantize(packed[i][0].data_ptr(), packed[i][1].data_ptr(), code.data_ptr(), n, BLOCKSIZE,
+                                                wout.data_ptr(), ta._lib.BF16, sptr))
+
+        tq = timed(quant)
+        td = timed(dequant)
+        bq = 2 * n + n // 2 + 4 * (n // BLOCKSIZE)
+        bd = n // 2 + 4 * (n // BLOCKSIZE) + 64 + 2 * n
+        out[f"{N}x{K}"] = {
+            "quantize_us": round(tq * 1e6, 1), "quantize_GBs": round(bq / tq / 1e9, 1), "quantize_frac_of_hbm_peak": round(bq / tq / 1e9 / HBM_PEAK_GBS, 3),
+            "dequantize_us": round(td * 1e6, 1), "dequantize_GBs": round(bd / td / 1e9, 1), "dequantize_frac_of_hbm_peak": round(bd / td / 1e9 / HBM_PEAK_GBS, 3),
+        }
+        del ws, packed
+    return out
 
 
 def llama_decode(torch, ta, n_new: int) -> dict:

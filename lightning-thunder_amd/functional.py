@@ -44,9 +44,22 @@ NF4_CODE = (
 )  # fmt: skip
 
 
+_code_masters: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+
+
 def nf4_code(device=None, dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """The 16-entry code book as a tensor (``quant_map`` / ``QuantState.code``)."""
-    return torch.tensor(NF4_CODE, dtype=torch.float32, device=device).to(dtype)
+    """The 16-entry code book as a new tensor (``quant_map`` / ``QuantState.code``).  One master copy
+    per device is kept and cloned, so that only the first call on a device pays a host-to-device
+    copy (which synchronises the stream)."""
+    dev = torch.device(device) if device is not None else torch.device("cpu")
+    if dev.type == "cuda" and dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    key = (str(dev), dtype)
+    master = _code_masters.get(key)
+    if master is None:
+        master = torch.tensor(NF4_CODE, dtype=torch.float32, device=dev).to(dtype)
+        _code_masters[key] = master
+    return master.clone()
 
 
 def dynamic_map(device=None) -> torch.Tensor:

@@ -214,7 +214,7 @@ def prefill_section(torch, ta) -> dict:
     """BASELINE config 3, outside the timed region of the GEMV metric: the Llama-3-8B projection
     shapes with M in {512, 2048, 8192} rows of x through ``matmul_nf4`` (which routes them to
     nf4hip_dequantize + the dense library GEMM), and the fused NF4 GEMM kernel (nf4hip_gemm) at
-    M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events around 10 calls (3 for the fused kernel) after 3 warm-up calls."""
+    M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events bracket 10 calls (3 for the fused kernel) after 3 warm-up calls."""
     dev = torch.device("cuda:0")
     F = ta.functional
     code = ta.nf4_code(dev)

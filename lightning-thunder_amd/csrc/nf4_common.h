@@ -66,6 +66,16 @@ __device__ __forceinline__ uint4 load16(const void* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// 16-byte store, ordinary or streaming (non-temporal: the data is not meant to stay in the caches).
+template <bool STREAM>
+__device__ __forceinline__ void store16(void* p, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    const u32x4_t v = {a, b, c, d};
+    if (STREAM)
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(p));
+    else
+        *reinterpret_cast<u32x4_t*>(p) = v;
+}
+
 // fp32 -> bf16 bits, round to nearest even (finite inputs; NaN is quieted).
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);

@@ -389,19 +389,19 @@ def test_llama70b_shapes_double_quant(ta, N, K):
 
 
 @pytest.mark.parametrize("N,K", [(28672, 4096), (128256, 4096), (16384 + 16, 4096)])
-def test_gemv_five_to_eight_rows_on_large_weights(ta, N, K):
-    """M = 5..8 is served by the quad kernel up to 2^26 weights and by the MFMA tile kernel beyond
-    (fused gate/up projection, lm_head, and a shape just past the switch with a ragged last tile):
-    at full size against a float64-accumulated matmul over sampled rows of the HIP-dequantized weight,
-    which is itself pinned bit-exact against the oracle at small sizes."""
-    _sync_print(f"gemv M=5..8 large N={N} K={K}")
+def test_gemv_every_m_on_large_weights(ta, N, K):
+    """Every decode kernel at full size (fused gate/up projection, lm_head, and a shape just past
+    2^26 weights with a ragged last tile -- M = 5..8 is served by the quad kernel up to that size and
+    by the MFMA tile kernel beyond): against a float64-accumulated matmul over sampled rows of the
+    HIP-dequantized weight, which is itself pinned bit-exact against the oracle at small sizes."""
+    _sync_print(f"gemv every M, large N={N} K={K}")
     g = torch.Generator(device=DEV).manual_seed(N + K)
     w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
     qw, absmax, code = ta.quantize_nf4(w)
     deq = ta.dequantize_nf4(qw, absmax, code, 64, torch.bfloat16, (N, K))
     rows = torch.cat([torch.randint(0, N, (61,), generator=g, device=DEV), torch.tensor([0, N - 2, N - 1], device=DEV)])
     bias = torch.randn(N, generator=g, device=DEV).to(torch.bfloat16)
-    for M in (5, 6, 7, 8):
+    for M in (1, 2, 3, 4, 5, 6, 7, 8, 12, 16):
         x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
         assert ta.functional.fused_route(x, bias, 64, torch.bfloat16, (N, K)) == "gemv"
         y = ta.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))

@@ -94,12 +94,12 @@ hipError_t gemv_allow_lds(K kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-// row-streaming kernel, M = 1 (nf4_gemv_rows.hip)
+// row-streaming kernel, M = 1, 2 (nf4_gemv_rows.hip)
 size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_rows_setup();
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream);
 
-// four-weight-rows-per-quad kernel, 2 <= M <= 8 (nf4_gemv_quad.hip)
+// four-weight-rows-per-quad kernel, 3 <= M <= 8 (nf4_gemv_quad.hip)
 size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_quad_setup();
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream);

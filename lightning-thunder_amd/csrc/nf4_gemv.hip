@@ -1,7 +1,7 @@
 // Dispatch of the decode-shape fused NF4 dequant-matmul (M <= 16) between its three kernels:
-// row-streaming (M = 1, nf4_gemv_rows.hip), four weight rows per lane quad (M = 2..4, and M = 5..8
-// on weights of at most 2^26 elements, nf4_gemv_quad.hip) and MFMA tiles (the rest up to M = 16,
-// nf4_gemv_tiles.hip).
+// row-streaming (M = 1, 2, nf4_gemv_rows.hip), four weight rows per lane quad (M = 3, 4, and
+// M = 5..8 on weights of at most 2^26 elements, nf4_gemv_quad.hip) and MFMA tiles (the rest up to
+// M = 16, nf4_gemv_tiles.hip).
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -42,7 +42,7 @@ bool quad_serves(int64_t M, int64_t N, int64_t K) { return M <= 4 || (M <= 8 && 
 // ---- dispatch -------------------------------------------------------------------------------
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (M == 1) return gemv_rows_workspace_bytes(M, N, K);
+    if (M <= 2) return gemv_rows_workspace_bytes(M, N, K);
     return quad_serves(M, N, K) ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
 }
 
@@ -50,7 +50,7 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     int cus = 0;
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;
-    if (a.M == 1) return launch_gemv_rows(a, cus, stream);
+    if (a.M <= 2) return launch_gemv_rows(a, cus, stream);
     return quad_serves(a.M, a.N, a.K) ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
 }
 

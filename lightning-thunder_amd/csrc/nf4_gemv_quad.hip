@@ -1,4 +1,4 @@
-// Decode-shape fused NF4 dequant-matmul for gfx950, 2 <= M <= 8 rows of x.
+// Decode-shape fused NF4 dequant-matmul for gfx950, 3 <= M <= 8 rows of x (any M from 1 works).
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -170,9 +170,6 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
         // per request instead of 16, and with 16 waves per CU the address unit would then pace the
         // whole kernel.)  These requests go out ahead of the weights: they are served by the L2 while
         // the first weights are on their way from HBM.
-        // With two rows of x the transpose costs more than it saves: every lane then reads its own 64
-        // bytes (piece q of row `ri` lands in xraw[0][c][q]).
-        const bool direct_x = XS == 1 && M <= 2;
         uint4 xraw[XS][CPW][4];
         float lut = lut_mine;
         if constexpr (FIRST) {
@@ -183,15 +180,13 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
 #pragma unroll
             for (int c = 0; c < CPW; ++c) {
                 // a lane beyond K (or an idle wave) reads the end of the row; the value is dropped below
-                const int64_t kc = kw0 + c * LOAD_K + (direct_x ? (int64_t)kseg : (int64_t)(8 * lane));
-                const uint16_t* xb = a.x + min(kc, K - (direct_x ? 32 : 8));
-                if (direct_x) xb += (int64_t)min(ri, M - 1) * K;
+                const int64_t kc = kw0 + c * LOAD_K + 8 * lane;
+                const uint16_t* xb = a.x + min(kc, K - 8);
 #pragma unroll
                 for (int h = 0; h < XS; ++h)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)  // transposed path, rows >= M: every lane reads x[0]
-                        xraw[h][c][r] =
-                            load16(direct_x ? xb + 8 * r : (4 * h + r < M ? xb + (int64_t)(4 * h + r) * K : a.x));
+                    for (int r = 0; r < 4; ++r)  // rows >= M: every lane reads x[0] (one cache line)
+                        xraw[h][c][r] = load16(4 * h + r < M ? xb + (int64_t)(4 * h + r) * K : a.x);
             }
         }
         // get the weight stream going before anything else happens
@@ -215,20 +210,16 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
             for (int h = 0; h < XS; ++h)
 #pragma unroll
                 for (int c = 0; c < CPW; ++c) {
-                    const bool in =
-                        rg < p.row_groups && kw0 + c * LOAD_K + (direct_x ? (int64_t)kseg : (int64_t)(8 * lane)) < K;
+                    const bool in = rg < p.row_groups && kw0 + c * LOAD_K + 8 * lane < K;
                     uint32_t v[4][4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const bool keep = in && (direct_x ? ri < M : 4 * h + r < M);
+                        const bool keep = in && 4 * h + r < M;
                         v[r][0] = keep ? xraw[h][c][r].x : 0u; v[r][1] = keep ? xraw[h][c][r].y : 0u;
                         v[r][2] = keep ? xraw[h][c][r].z : 0u; v[r][3] = keep ? xraw[h][c][r].w : 0u;
                     }
-                    if (!direct_x) {
 #pragma unroll
-                        for (int d = 0; d < 4; ++d)
-                            transpose_quad(v[0][d], v[1][d], v[2][d], v[3][d], lane & 1, lane & 2);
-                    }
+                    for (int d = 0; d < 4; ++d) transpose_quad(v[0][d], v[1][d], v[2][d], v[3][d], lane & 1, lane & 2);
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
 #pragma unroll

@@ -1,4 +1,4 @@
-// Decode-shape fused NF4 dequant-matmul for gfx950, M = 1 (any M <= 4 works): the GEMV proper.
+// Decode-shape fused NF4 dequant-matmul for gfx950, M = 1 and 2 (any M <= 4 works): the GEMV proper.
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -358,7 +358,8 @@ hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_
 
 template <bool NESTED>
 hipError_t launch_n(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
-    return launch_m<1, NESTED>(a, p, grid, stream);  // M = 2..4 is served by the four-rows-per-quad kernel
+    // M = 3 and 4 are served by the four-rows-per-quad kernel
+    return a.M == 2 ? launch_m<2, NESTED>(a, p, grid, stream) : launch_m<1, NESTED>(a, p, grid, stream);
 }
 
 template <int M, int U>
@@ -387,8 +388,10 @@ size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 hipError_t gemv_rows_setup() {
-    const hipError_t e = allow_lds_mu<1, 8>();
-    return e != hipSuccess ? e : allow_lds_m<1>();
+    hipError_t e;
+    if ((e = allow_lds_mu<1, 8>()) != hipSuccess) return e;
+    if ((e = allow_lds_m<1>()) != hipSuccess) return e;
+    return allow_lds_m<2>();
 }
 
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {

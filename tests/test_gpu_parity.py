@@ -224,7 +224,7 @@ def test_gemv_blocksizes(ta, oracle, blocksize, M):
 
 
 @pytest.mark.parametrize("N,K", [(64, 1376), (2, 32), (33, 96), (5, 2048 + 32)])
-@pytest.mark.parametrize("M", [1, 4])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
 def test_gemv_rows_odd_k(ta, oracle, N, K, M):
     """The row-streaming kernel needs only K % 32 == 0: quantisation blocks may straddle rows
     (K = 1376 is the intermediate size of the reference's own llama2-like test model)."""

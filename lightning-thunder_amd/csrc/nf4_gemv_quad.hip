@@ -455,6 +455,8 @@ hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {
     int slots = 2 * cus;
     if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
     const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
+    // one arrival counter per band when K is split across workgroups
+    if (p.splits > 1 && p.nbands > GEMV_COUNTER_BYTES / 4) return hipErrorInvalidValue;
     int grid = p.ntasks < slots ? p.ntasks : slots;
     grid -= grid % p.splits;  // every workgroup keeps one K split (ntasks is a multiple of splits)
     if (grid < p.splits) grid = p.splits;

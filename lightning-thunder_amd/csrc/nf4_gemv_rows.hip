@@ -398,6 +398,8 @@ hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {
     int slots = 2 * cus;
     if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
     const RowsPlan p = make_rows_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
+    // one arrival counter per band when K is split across workgroups
+    if (p.splits > 1 && p.nbands > GEMV_COUNTER_BYTES / 4) return hipErrorInvalidValue;
     const int grid = p.ntasks < slots ? p.ntasks : slots;
     return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
 }

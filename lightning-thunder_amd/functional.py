@@ -232,8 +232,22 @@ def _gemv_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+def _chunked_gemv_wins(M: int, n_weights: int) -> bool:
+    """For a few more than 16 rows of x: is ceil(M / 16) passes of the decode kernel over the NF4
+    weight cheaper than dequantize + dense GEMM?  Both sides modelled from measurements on MI355X
+    (microseconds, W = weights in millions): a 16-row pass takes 12 + 0.105 W, the dense route
+    20 + 0.62 W before its GEMM; the passes must win by 20 %.  [28672, 4096]: up to M = 48
+    (73 vs 111 us), lm_head [128256, 4096]: up to M = 64 (259 vs 431 us); below 40 M weights never."""
+    if M <= 16 or n_weights < 40_000_000:
+        return False
+    w = n_weights / 1e6
+    passes = (M + 15) // 16
+    return passes * (12.0 + 0.105 * w) < 0.8 * (20.0 + 0.62 * w)
+
+
 def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape) -> str:
-    """Which kernel serves this call: ``"gemv"``, ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP
+    """Which kernel serves this call: ``"gemv"``, ``"gemv-chunks"`` (the decode kernel once per 16
+    rows of x), ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP
     dequantize, then the dense library GEMM, because that is the faster of the two for many rows
     of x) or ``"dequant+linear"`` (the same two steps, for dtypes and shapes no fused kernel takes).
 
@@ -259,6 +273,8 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "dequant+linear"
     if M <= 16 and K % 512 == 0:
         return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
+    if K % 512 == 0 and _chunked_gemv_wins(M, N * K):
+        return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
     # the fused GEMM kernel streams K sequentially per tile: beyond EXACT_K even a few rows of x are
     # served faster by dequantize + dense GEMM
     return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M or K > EXACT_K else "gemm"
@@ -289,8 +305,8 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
     nblocks = N * K // blocksize
     with torch.cuda.device(x.device):
         out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-        if route == "gemv":
-            need = lib.nf4hip_gemv_workspace_bytes(M, N, K)
+        if route in ("gemv", "gemv-chunks"):
+            need = lib.nf4hip_gemv_workspace_bytes(min(M, 16), N, K)
             ws = _gemv_workspace(x.device, need)
             ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
             fn, fn_dq = lib.nf4hip_gemv, lib.nf4hip_gemv_dq
@@ -298,15 +314,22 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
             ws_ptr, ws_bytes = None, 0
             fn, fn_dq = lib.nf4hip_gemm, lib.nf4hip_gemm_dq
         bptr = None if b is None else b.data_ptr()
+        # row chunks of x and out: one call, or 16 rows at a time (rows are contiguous, K and N even,
+        # so every chunk starts 16-byte aligned when the whole does and K, N are multiples of 8)
+        step = 16 if route == "gemv-chunks" else M
         if isinstance(absmax, NestedAbsmax):
             q, a2, m256, off, nbs = _nested_args(absmax, nblocks)
-            _lib.check(fn_dq(x2.data_ptr(), _lib.BF16, M, qweight.data_ptr(), q.data_ptr(), a2.data_ptr(), m256.data_ptr(), off, nbs,
-                             quant_map.data_ptr(), bptr, N, K, blocksize, out.data_ptr(), ws_ptr, ws_bytes, _stream()))  # fmt: skip
+            for m0 in range(0, M, step):
+                mc = min(step, M - m0)
+                _lib.check(fn_dq(x2.data_ptr() + 2 * m0 * K, _lib.BF16, mc, qweight.data_ptr(), q.data_ptr(), a2.data_ptr(), m256.data_ptr(), off, nbs,
+                                 quant_map.data_ptr(), bptr, N, K, blocksize, out.data_ptr() + 2 * m0 * N, ws_ptr, ws_bytes, _stream()))  # fmt: skip
         else:
             _require_gpu(absmax)
             absmax = _aligned(absmax.to(torch.float32))
             if absmax.numel() < nblocks:
                 raise ValueError(f"absmax holds {absmax.numel()} entries, need {nblocks}")
-            _lib.check(fn(x2.data_ptr(), _lib.BF16, M, qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(), bptr,
-                          N, K, blocksize, out.data_ptr(), ws_ptr, ws_bytes, _stream()))  # fmt: skip
+            for m0 in range(0, M, step):
+                mc = min(step, M - m0)
+                _lib.check(fn(x2.data_ptr() + 2 * m0 * K, _lib.BF16, mc, qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(), bptr,
+                              N, K, blocksize, out.data_ptr() + 2 * m0 * N, ws_ptr, ws_bytes, _stream()))  # fmt: skip
     return out.reshape(*x.shape[:-1], N)

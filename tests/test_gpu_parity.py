@@ -409,6 +409,32 @@ def test_gemv_every_m_on_large_weights(ta, N, K):
         torch.testing.assert_close(y[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nested", [False, True])
+def test_gemv_chunks_route(ta, nested):
+    """17..48 rows of x on a large weight go through the decode kernel 16 rows at a time: every
+    chunk boundary and a ragged last chunk, with bias, against a float64-accumulated matmul over sampled
+    rows of the HIP-dequantized weight."""
+    N, K = 28672, 4096
+    _sync_print(f"gemv-chunks nested={nested}")
+    g = torch.Generator(device=DEV).manual_seed(99)
+    w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    qw, absmax, code = ta.quantize_nf4(w)
+    state = ta.compress_absmax(absmax) if nested else absmax
+    deq = ta.dequantize_nf4(qw, state, code, 64, torch.bfloat16, (N, K))
+    rows = torch.cat([torch.randint(0, N, (61,), generator=g, device=DEV), torch.tensor([0, N - 2, N - 1], device=DEV)])
+    bias = torch.randn(N, generator=g, device=DEV).to(torch.bfloat16)
+    for M in (17, 32, 33, 48):
+        x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+        assert ta.functional.fused_route(x, bias, 64, torch.bfloat16, (N, K)) == "gemv-chunks"
+        y = ta.matmul_nf4(x.reshape(1, M, K), qw, bias, state, code, 64, torch.bfloat16, (N, K))
+        assert y.shape == (1, M, N)
+        ref = x.double() @ deq[rows].double().t() + bias[rows].double()
+        torch.testing.assert_close(y[0][:, rows].double(), ref, rtol=2e-2, atol=2e-2)
+        # a chunk computes what a 16-row call computes
+        y16 = ta.matmul_nf4(x[16:32] if M >= 32 else x[:16], qw, bias, state, code, 64, torch.bfloat16, (N, K))
+        assert torch.equal(y16, y[0][16:32] if M >= 32 else y[0][:16])
+
+
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
 def test_gemv_exact_variants_recover_dequantized_weights(ta, oracle, M):
     """K > 16384 selects the decode kernels' exact-weights variants: with one-hot rows of x every

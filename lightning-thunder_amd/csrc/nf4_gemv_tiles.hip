@@ -201,23 +201,28 @@ __device__ __forceinline__ void transpose_g(uint32_t d[4]) {
     }
 }
 
+// `on` (wave-uniform, all ones or zero) switches a request off without a branch: with on = 0 every
+// lane reads the first bytes of the phase (one cache line per instruction) and the slot's contents
+// are never used.
 template <bool B64, bool NESTED>
-__device__ __forceinline__ void load_phase(const MatmulArgs& a, PhaseRegs& r, const LaneLoad& ll, int n0c, int kabs) {
+__device__ __forceinline__ void load_phase(const MatmulArgs& a, PhaseRegs& r, const LaneLoad& ll, int n0c, int kabs,
+                                           uint32_t on = 0xffffffffu) {
     // n0c = first row actually read for the tile, kabs = first k of the phase (both wave-uniform)
     const int64_t e0 = (int64_t)n0c * a.K + kabs;
     const uint8_t* wp = a.packed + (e0 >> 1);
+    const uint32_t s_off = ll.s_off & on;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) r.w[i] = load16_stream(wp + ll.woff[i]);
+    for (int i = 0; i < 4; ++i) r.w[i] = load16_stream(wp + (ll.woff[i] & on));
     if (NESTED) {
         if (B64) {
-            const int64_t b = (e0 >> 6) + ll.s_off;
+            const int64_t b = (e0 >> 6) + s_off;
             const uint2 q = *reinterpret_cast<const uint2*>(a.nested.q + b);
             r.s[0].x = __uint_as_float(q.x);
             r.s[0].y = __uint_as_float(q.y);
             // 8 consecutive blocks starting at a multiple of 8 share one nested block (>= 64 blocks)
             r.s[0].z = a.nested.absmax2[b >> a.nested.nested_log2];
         } else {
-            const int64_t b = ((int64_t)n0c * a.K >> a.block_log2) + ll.s_off;
+            const int64_t b = ((int64_t)n0c * a.K >> a.block_log2) + s_off;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 r.s[j].x = nested_absmax(a.nested, b + ((kabs + j * 256) >> a.block_log2));
@@ -227,11 +232,11 @@ __device__ __forceinline__ void load_phase(const MatmulArgs& a, PhaseRegs& r, co
             }
         }
     } else if (B64) {
-        const float* sp = a.absmax + (e0 >> 6) + ll.s_off;
+        const float* sp = a.absmax + (e0 >> 6) + s_off;
         r.s[0] = *reinterpret_cast<const float4*>(sp);
         r.s[1] = *reinterpret_cast<const float4*>(sp + 4);
     } else {
-        const float* sp = a.absmax + ((int64_t)n0c * a.K >> a.block_log2) + ll.s_off;
+        const float* sp = a.absmax + ((int64_t)n0c * a.K >> a.block_log2) + s_off;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             r.s[j].x = sp[(kabs + j * 256) >> a.block_log2];
@@ -262,7 +267,7 @@ struct PhaseOperands {
     float sc[8];
 };
 
-template <bool B64, bool NESTED>
+template <bool B64, bool NESTED, bool STEADY>
 __device__ __forceinline__ void prepare_phase(const MatmulArgs& a, PhaseRegs& r, int lane, PhaseOperands& o) {
     const bool b0 = lane & 1, b1 = lane & 2;
     float* sc = o.sc;
@@ -274,8 +279,17 @@ __device__ __forceinline__ void prepare_phase(const MatmulArgs& a, PhaseRegs& r,
             sc[j] = __fadd_rn(__fmul_rn(a.nested.map256[code], r.s[0].z), a.nested.offset);
         }
     } else {
-        sc[0] = r.s[0].x; sc[1] = r.s[0].y; sc[2] = r.s[0].z; sc[3] = r.s[0].w;
-        sc[4] = r.s[1].x; sc[5] = r.s[1].y; sc[6] = r.s[1].z; sc[7] = r.s[1].w;
+        const float in[8] = {r.s[0].x, r.s[0].y, r.s[0].z, r.s[0].w, r.s[1].x, r.s[1].y, r.s[1].z, r.s[1].w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // STEADY: real moves.  The compiler would rename registers instead and then rotate the
+            // slot's registers at the back edge of the steady loop, which needs the data of the
+            // load just issued and so waits for it.
+            if (STEADY)
+                asm volatile("v_mov_b32 %0, %1" : "=v"(sc[j]) : "v"(in[j]));
+            else
+                sc[j] = in[j];
+        }
     }
 
     // in-quad transpose, one dword column at a time: load index <-> lane & 3
@@ -394,7 +408,13 @@ __device__ __forceinline__ void store_x_slice(const MatmulArgs& a, const uint4 (
     }
 }
 
-template <bool B64, bool NESTED, int R, bool EXACT>
+// STEADY (long work lists): the slots are refilled without branches and groups of four entries that
+// follow each other without a restage or a batch end run in an inner loop that holds nothing else.
+// The compiler can then count the loads in flight and waits for ONE slot where it otherwise waits for
+// everything in flight at the top of every group (loads under branches, and the stores of a batch
+// end, which complete out of order with loads).  The price is a drain when that loop is entered and
+// switched-off requests at the end of the list, which short lists cannot afford.
+template <bool B64, bool NESTED, int R, bool EXACT, bool STEADY>
 __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Plan p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int CAP = XBYTES_MAX / (R * 1024);  // phases of x that fit
@@ -458,7 +478,12 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j) {
-            if (j < cn) {
+            if constexpr (STEADY) {
+                const Item it = read_item(j);
+                const bool on = j < cn && !(it.info & ITEM_GAP);
+                load_phase<B64, NESTED>(a, ring[j], ll, first_row(on ? it.tg : ls.tg0),
+                                        on ? it.kabs : ls.r0 * PHASE_K, on ? 0xffffffffu : 0u);
+            } else if (j < cn) {
                 const Item it = read_item(j);
                 if (!(it.info & ITEM_GAP)) load_phase<B64, NESTED>(a, ring[j], ll, first_row(it.tg), it.kabs);
             }
@@ -493,6 +518,34 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                     __syncthreads();
                 }
             }
+            if constexpr (STEADY) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the steady loop is entered with nothing in flight
+                for (;;) {
+#pragma unroll
+                    for (int j = 0; j < SLOTS; ++j) {
+                        const Item it = read_item(base + j);
+                        const Item nx = read_item(min(base + j + SLOTS, cn - 1));
+                        const bool refill = base + j + SLOTS < cn && !(nx.info & ITEM_GAP);
+                        // codes out of the slot, the slot refilled at once, both without a branch (a
+                        // gap's operands are not used)
+                        PhaseOperands o;
+                        prepare_phase<B64, NESTED, true>(a, ring[j], lane, o);
+                        load_phase<B64, NESTED>(a, ring[j], ll, first_row(refill ? nx.tg : ls.tg0),
+                                                refill ? nx.kabs : ls.r0 * PHASE_K, refill ? 0xffffffffu : 0u);
+                        if (!(it.info & ITEM_GAP)) {
+                            contract_phase<R, EXACT>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane,
+                                                     acc[j]);
+                            if (it.info & ITEM_END) {
+                                end_info = it.info;
+                                end_tg = it.tg;
+                            }
+                        }
+                    }
+                    if ((end_info & ITEM_END) || base + SLOTS >= cn) break;
+                    if (read_item(base + SLOTS).info & ITEM_RESTAGE) break;
+                    base += SLOTS;
+                }
+            } else {
 #pragma unroll
             for (int j = 0; j < SLOTS; ++j) {
                 const Item it = read_item(base + j);
@@ -501,7 +554,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                 if (base + j + SLOTS < cn) nx = read_item(base + j + SLOTS);
                 if (!(it.info & ITEM_GAP)) {
                     PhaseOperands o;
-                    prepare_phase<B64, NESTED>(a, ring[j], lane, o);
+                    prepare_phase<B64, NESTED, false>(a, ring[j], lane, o);
                     // the slot's registers are free again: refill before the long part of the work
                     if (!(nx.info & ITEM_GAP)) load_phase<B64, NESTED>(a, ring[j], ll, first_row(nx.tg), nx.kabs);
                     contract_phase<R, EXACT>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane, acc[j]);
@@ -512,6 +565,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                 } else if (!(nx.info & ITEM_GAP)) {
                     load_phase<B64, NESTED>(a, ring[j], ll, first_row(nx.tg), nx.kabs);
                 }
+            }
             }
             if (!(end_info & ITEM_END)) continue;
             const int fin_nb = (end_info >> ITEM_NB_SHIFT) & 7;
@@ -619,6 +673,10 @@ constexpr int rows_held(int64_t M) {
 // alone; the grid does (correctness never depends on how many workgroups are resident).
 constexpr int NOMINAL_SLOTS = 256;
 
+// Work lists at least this long run the STEADY variant of the kernel (measured: it gains 3-8 % from 16
+// entries on and costs up to 2 us on lists of four).
+constexpr int STEADY_MIN_ITEMS = 16;
+
 int grid_for(int64_t ntasks, int splits, int slots) {
     int grid = (int)(ntasks < slots ? ntasks : slots);
     grid -= grid % splits;
@@ -658,13 +716,19 @@ size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return (size_t)COUNTER_BYTES + (p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)N * sizeof(float) : 0);
 }
 
+template <bool B64, bool NESTED, bool STEADY>
+hipError_t allow_rx() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, false, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, false, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, true, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, true, STEADY>, SMEM_BYTES);
+}
+
 template <bool B64, bool NESTED>
 hipError_t allow_both() {
-    hipError_t e;
-    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, true>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, true>, SMEM_BYTES);
+    const hipError_t e = allow_rx<B64, NESTED, false>();
+    return e != hipSuccess ? e : allow_rx<B64, NESTED, true>();
 }
 
 hipError_t gemv_tiles_setup() {
@@ -675,14 +739,20 @@ hipError_t gemv_tiles_setup() {
     return allow_both<true, true>();
 }
 
-template <int R, bool EXACT>
-hipError_t launch_r(const MatmulArgs& a, const Plan& p, int grid, hipStream_t stream) {
+template <int R, bool EXACT, bool STEADY>
+hipError_t launch_rs(const MatmulArgs& a, const Plan& p, int grid, hipStream_t stream) {
     const bool b64 = a.block_log2 == 6;
     const bool nested = a.nested.q != nullptr;
-    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R, EXACT> : gemv_tiles_kernel<true, false, R, EXACT>)
-                    : (nested ? gemv_tiles_kernel<false, true, R, EXACT> : gemv_tiles_kernel<false, false, R, EXACT>);
+    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R, EXACT, STEADY> : gemv_tiles_kernel<true, false, R, EXACT, STEADY>)
+                    : (nested ? gemv_tiles_kernel<false, true, R, EXACT, STEADY>
+                              : gemv_tiles_kernel<false, false, R, EXACT, STEADY>);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
+}
+
+template <int R, bool EXACT>
+hipError_t launch_r(const MatmulArgs& a, const Plan& p, int grid, bool steady, hipStream_t stream) {
+    return steady ? launch_rs<R, EXACT, true>(a, p, grid, stream) : launch_rs<R, EXACT, false>(a, p, grid, stream);
 }
 
 hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
@@ -691,17 +761,18 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
     p.tg_step = grid / p.splits;
     // the longest work list of a workgroup (the one that owns the most tile groups and a full K range)
     // must fit in LDS
-    {
-        const int cap = XBYTES_MAX / (rows_held(a.M) * 1024);
-        const int G = (p.tile_groups + p.tg_step - 1) / p.tg_step;
-        const int nsl = (p.range_phases + cap - 1) / cap;
-        const int last = p.range_phases - (nsl - 1) * cap;
-        const int n = rows_held(a.M) == 8 ? list_length<10>(G, nsl, last) : list_length<5>(G, nsl, last);
-        if (n > ITEMS_MAX) return hipErrorInvalidValue;
-    }
+    const int cap = XBYTES_MAX / (rows_held(a.M) * 1024);
+    const int G = (p.tile_groups + p.tg_step - 1) / p.tg_step;
+    const int nsl = (p.range_phases + cap - 1) / cap;
+    const int last = p.range_phases - (nsl - 1) * cap;
+    const int n = rows_held(a.M) == 8 ? list_length<10>(G, nsl, last) : list_length<5>(G, nsl, last);
+    if (n > ITEMS_MAX) return hipErrorInvalidValue;
+    const bool steady = n >= STEADY_MIN_ITEMS;
     if (gemv_wants_exact(a.K))
-        return rows_held(a.M) == 8 ? launch_r<8, true>(a, p, grid, stream) : launch_r<16, true>(a, p, grid, stream);
-    return rows_held(a.M) == 8 ? launch_r<8, false>(a, p, grid, stream) : launch_r<16, false>(a, p, grid, stream);
+        return rows_held(a.M) == 8 ? launch_r<8, true>(a, p, grid, steady, stream)
+                                   : launch_r<16, true>(a, p, grid, steady, stream);
+    return rows_held(a.M) == 8 ? launch_r<8, false>(a, p, grid, steady, stream)
+                               : launch_r<16, false>(a, p, grid, steady, stream);
 }
 
 }  // namespace nf4

@@ -337,6 +337,47 @@ def test_fallback_route(ta, oracle, case):
     torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
 
 
+def test_matmul_randomized_sweep_large(ta):
+    """Seeded sweep over every route of matmul_nf4 at sizes the CPU oracle would take too long for
+    (N up to 40000, K up to 28672, M up to 48: row / quad / tile kernels with their exact and
+    long-list variants, the 16-row chunk route, the dense route), each against a float64-accumulated
+    matmul over sampled rows of the HIP-dequantized weight (pinned bit-exact against the oracle by the
+    tests above)."""
+    rng = torch.Generator().manual_seed(4321)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rng))]
+
+    code = ta.nf4_code(DEV)
+    seen = set()
+    for case in range(120):
+        M = pick([1, 2, 3, 4, 5, 6, 7, 8, 9, 11, 13, 16, 17, 24, 33, 48])
+        K = pick([512, 1024, 2048, 3072, 4096, 6144, 8192, 14336, 16384 + 512, 28672])
+        N = pick([1, 5, 16, 31, 64, 100, 128, 257, 1000, 2049, 4096, 6000, 14336, 20000, 40000])
+        if N * K > 600_000_000:
+            N = 4096
+        blocksize = pick([64, 64, 64, 128, 256, 512])
+        bias = pick([False, True])
+        nested = pick([False, False, True])
+        _sync_print(f"large sweep {case}: M={M} N={N} K={K} bs={blocksize} bias={bias} nested={nested}")
+        g = torch.Generator(device=DEV).manual_seed(case)
+        w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+        x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+        b = torch.randn(N, generator=g, device=DEV).to(torch.bfloat16) if bias else None
+        qw, absmax, _ = ta.quantize_nf4(w, blocksize)
+        state = ta.compress_absmax(absmax) if nested else absmax
+        deq = ta.dequantize_nf4(qw, state, code, blocksize, torch.bfloat16, (N, K))
+        seen.add(ta.functional.fused_route(x, b, blocksize, torch.bfloat16, (N, K)))
+        y = ta.matmul_nf4(x, qw, b, state, code, blocksize, torch.bfloat16, (N, K))
+        rows = torch.randint(0, N, (min(N, 256),), generator=g, device=DEV)
+        ref = x.double() @ deq[rows].double().t()
+        if bias:
+            ref = ref + b[rows].double()
+        torch.testing.assert_close(y[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
+        del w, x, qw, absmax, deq, y
+    assert {"gemv", "gemv-chunks", "dequant+gemm"} <= seen
+
+
 def test_full_size_properties(ta):
     """Llama-3-8B FFN shape at full size through size-independent properties: quantize is
     idempotent on its own dequantisation, and gemv is linear in x."""

@@ -26,11 +26,11 @@ SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
 # (the cheaper "scale the partial sum" arithmetic drifts from it like sqrt(K)); the 5..16-row tile
 # kernel has no such variant, so those calls go to the prefill kernel, which is exact by construction.
 EXACT_K = 16384
-# From this many rows of x on, HIP dequantize followed by the dense library GEMM is faster than
-# the fused GEMM kernel (measured on MI355X at every Llama-3-8B projection shape: the fused kernel
-# re-expands the weight tile once per 128 rows of x and reaches ~0.5 PFLOP/s, the library GEMM
-# 1.1-1.5 PFLOP/s and the dequantize kernel runs at HBM speed).  Raise it to force the fused,
-# allocation-free kernel.
+# From this many rows of x on, HIP dequantize followed by the dense library GEMM is the default
+# (the fused GEMM kernel re-expands the weight tile once per 256 rows of x and reaches 0.9-1.0
+# PFLOP/s, the library GEMM 1.1-1.5 PFLOP/s and the dequantize kernel runs at HBM speed); see
+# _fused_gemm_wins for where the fused kernel is faster all the same.  Raise it to force the
+# fused, allocation-free kernel everywhere.
 DENSE_ROUTE_MIN_M = 17
 
 _DTYPE_CODE = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32}
@@ -232,17 +232,40 @@ def _gemv_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
-def _chunked_gemv_wins(M: int, n_weights: int) -> bool:
-    """For a few more than 16 rows of x: is ceil(M / 16) passes of the decode kernel over the NF4
-    weight cheaper than dequantize + dense GEMM?  Both sides modelled from measurements on MI355X
-    (microseconds, W = weights in millions): a 16-row pass takes 12 + 0.105 W, the dense route
-    20 + 0.62 W before its GEMM; the passes must win by 20 %.  [28672, 4096]: up to M = 48
-    (73 vs 111 us), lm_head [128256, 4096]: up to M = 64 (259 vs 431 us); below 40 M weights never."""
+# The fused GEMM kernel works on tiles of 256 weight rows; from this many rows on a weight has enough
+# tiles to fill the chip's 256 CUs with one tile of x rows.
+FUSED_GEMM_MIN_N = 28672
+
+
+def _fused_gemm_wins(M: int, N: int) -> bool:
+    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Measured on MI355X: for tall
+    weights and up to 512 rows of x it saves more by not writing the bf16 weight than it loses to the
+    library GEMM -- [28672, 4096]: 85 vs 111 us (M = 96), 133 vs 153 (512), 252 vs 209 (768);
+    [28672, 8192] M = 512: 252 vs 295; lm_head [128256, 4096]: 214 vs 453 (128), 289 vs 519 (256),
+    560 vs 733 (512), 844 vs 896 (768), 1151 vs 1085 (1024).  Shorter weights leave most CUs without a
+    tile ([14336, 4096]: 107 vs 74 us at M = 256)."""
+    if N < FUSED_GEMM_MIN_N:
+        return False
+    return M <= 512 or (M <= 768 and N >= 4 * FUSED_GEMM_MIN_N)
+
+
+def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
+    """For a few more than 16 rows of x: are ceil(M / 16) passes of the decode kernel over the NF4
+    weight cheaper than the alternatives?  All sides modelled from measurements on MI355X
+    (microseconds, W = weights in millions): a 16-row pass takes 12 + 0.105 W; the dense route
+    20 + 0.62 W before its GEMM, and the passes must beat that by 20 %; the fused GEMM kernel, where
+    it applies, 52 + 0.28 W for up to 128 rows.  [28672, 4096]: up to M = 48 (73 us vs 85 fused, 111
+    dense), lm_head [128256, 4096]: up to M = 32 (134 vs 200 fused); [14336, 4096]: up to M = 32
+    (36 vs 55 dense); below 40 M weights never."""
+    n_weights = N * K
     if M <= 16 or n_weights < 40_000_000:
         return False
     w = n_weights / 1e6
     passes = (M + 15) // 16
-    return passes * (12.0 + 0.105 * w) < 0.8 * (20.0 + 0.62 * w)
+    t = passes * (12.0 + 0.105 * w)
+    if _fused_gemm_wins(M, N) and t >= 52.0 + 0.28 * w:
+        return False
+    return t < 0.8 * (20.0 + 0.62 * w)
 
 
 def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape) -> str:
@@ -273,8 +296,10 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "dequant+linear"
     if M <= 16 and K % 512 == 0:
         return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
-    if K % 512 == 0 and _chunked_gemv_wins(M, N * K):
+    if K % 512 == 0 and _chunked_gemv_wins(M, N, K):
         return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
+    if _fused_gemm_wins(M, N):
+        return "gemm"  # tall weight, few hundred rows of x: expand the weight tiles in LDS
     # the fused GEMM kernel streams K sequentially per tile: beyond EXACT_K even a few rows of x are
     # served faster by dequantize + dense GEMM
     return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M or K > EXACT_K else "gemm"

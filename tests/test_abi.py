@@ -127,11 +127,15 @@ def test_fused_route_rules(ta):
     assert route(17, 64, 4096) == "dequant+gemm" and route(2048, 4096, 4096) == "dequant+gemm"
     # a few more than 16 rows on a large weight: the decode kernel once per 16 rows
     assert route(17, 28672, 4096) == "gemv-chunks" and route(48, 28672, 4096) == "gemv-chunks"
-    assert route(49, 28672, 4096) == "dequant+gemm"
-    assert route(64, 128256, 4096) == "gemv-chunks" and route(65, 128256, 4096) == "dequant+gemm"
+    assert route(49, 28672, 4096) == "gemm" and route(512, 28672, 4096) == "gemm"  # tall weight: fused GEMM
+    assert route(513, 28672, 4096) == "dequant+gemm"
+    assert route(32, 128256, 4096) == "gemv-chunks" and route(33, 128256, 4096) == "gemm"
+    assert route(768, 128256, 4096) == "gemm" and route(769, 128256, 4096) == "dequant+gemm"
+    assert route(256, 28672, 8192) == "gemm" and route(256, 14336, 4096) == "dequant+gemm"
     assert route(32, 14336, 4096) == "gemv-chunks" and route(33, 14336, 4096) == "dequant+gemm"
     assert route(32, 4096, 4096) == "dequant+gemm"        # small weight: dequantize is cheap
-    assert route(17, 28672, 4096 + 64) == "dequant+gemm"  # the tile kernel needs K % 512
+    assert route(17, 28672, 4096 + 64) == "gemm"          # the tile kernel needs K % 512, the fused GEMM K % 64
+    assert route(17, 14336, 4096 + 64) == "dequant+gemm"
     assert route(16, 8192, 28672) == "gemv"              # K > 16384: the tile kernel's exact-weights variant
     assert route(17, 8192, 28672) == "gemv-chunks" and route(512, 8192, 28672) == "dequant+gemm"
     assert route(1, 8192, 28672) == "gemv"               # row-streaming kernel has an exact variant

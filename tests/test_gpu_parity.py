@@ -300,6 +300,18 @@ def test_gemm_shapes(ta, oracle, M, N, K, fused_gemm):
     _matmul_case(ta, oracle, M, N, K, seed=M + N + K)
 
 
+@pytest.mark.parametrize("M,N,K,kw", [
+    (49, 28672, 512, {}), (128, 28700, 576, {"bias": True}), (129, 28672, 640, {"nested": True}),
+    (300, 28930, 512, {"blocksize": 256}), (512, 28672, 1024, {}), (700, 4 * 28672, 128, {"bias": True}),
+])
+def test_gemm_route_tall_weights(ta, oracle, M, N, K, kw):
+    """The default router sends tall weights with up to a few hundred rows of x to the fused GEMM
+    kernel (both tile heights, ragged M and N, odd and even numbers of k steps)."""
+    _sync_print(f"gemm (router) M={M} N={N} K={K} {kw}")
+    assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, kw.get("blocksize", 64), torch.bfloat16, (N, K)) == "gemm"
+    _matmul_case(ta, oracle, M, N, K, seed=M + K, **kw)
+
+
 def test_gemm_recovers_dequantized_weight_bit_exact(ta, oracle, fused_gemm):
     """x = identity makes every output a single product 1.0 * w: the fused kernel's in-LDS
     dequantisation must equal nf4hip_dequantize bit for bit."""

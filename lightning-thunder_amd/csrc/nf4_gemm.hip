@@ -2,19 +2,25 @@
 //
 // Replaces the dequantize_4bit + F.linear route of bitsandbytes.matmul_4bit
 // (MatMul4Bit.forward), reached from thunder/transforms/quantization.py:39: instead of writing
-// the whole bf16 weight to HBM and reading it back, every workgroup expands the NF4 tile it needs
-// to bf16 in LDS -- bf16_rne(lut16[code] * absmax), the same value nf4hip_dequantize produces -- and
-// contracts it with bf16 MFMA, fp32 accumulation, bf16 output.
+// the whole bf16 weight to HBM and reading it back, every wave expands the NF4 codes it needs to
+// bf16 in registers -- bf16_rne(lut16[code] * absmax), the same value nf4hip_dequantize produces --
+// and contracts them with bf16 MFMA, fp32 accumulation, bf16 output.
 //
-// Tile: BM (128 or 256 rows of x) x 256 (n) x 64 (k) per workgroup of 512 threads: 8 waves as
-// 2 (m) x 4 (n), each BM/2 x 64 outputs, v_mfma_f32_32x32x16_bf16 with A = x and B = W.  LDS holds
-// two stages of (BM + 256) rows padded to 144 bytes (128-bit fragment reads without bank
-// conflicts) and the code book.  One k step of 64 is one quantisation block per weight row at
-// blocksize 64, so a thread's 32 codes share one scale at every supported blocksize.
+// Tile: BM (128 or 256 rows of x) x 256 (n) x 64 (k) per workgroup of 512 threads.  Wave w of 8
+// owns weight rows 32 w .. + 31 of the tile against all BM rows of x: BM / 32 accumulators of
+// v_mfma_f32_32x32x16_bf16 with A = x (from LDS) and B = W (from this wave's registers).  A lane
+// loads 16 bytes = 32 codes of one weight row per k step; each of its four dwords becomes the B
+// fragment of one 16-k slice, so the weights never pass through LDS.  The k order inside a step
+// follows the codes (lane half h, slice s: k = 32 h + 8 s .. + 7) and the x fragments are read from
+// LDS in the same order.  LDS holds two stages of BM rows of x padded to 144 bytes (128-bit
+// fragment reads without bank conflicts) and the code book as a table of pairs: for every byte
+// value the two fp32 entries of its codes, in 32 copies laid out so that the 32 lanes the LDS serves
+// together never share a bank -- one ds_read_b64 per byte of codes.
 //
-// Pipeline per k step kt: the registers loaded two steps earlier (x rows, codes, absmax of step
-// kt + 1) are expanded into the other LDS stage between the MFMAs of step kt, then refilled with
-// step kt + 2; one barrier per step.
+// Pipeline per k step kt: x rows of step kt + 1 go from registers to the other LDS stage at the
+// top of the step and the registers are refilled with step kt + 2; codes and absmax run two steps
+// ahead in two register sets; the B fragment of slice s + 1 is expanded between the MFMAs of slice
+// s (pair-book reads in its first half, scaling and rounding in its second); one barrier per step.
 #include "nf4_common.h"
 
 #include <type_traits>
@@ -26,41 +32,33 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 
 constexpr int BK = 64;
 constexpr int BN = 256;
 constexpr int THREADS = 512;
 constexpr int ROW_BYTES = BK * 2 + 16;  // padded LDS row
-constexpr int LUT_BYTES = 16 * 256;     // 16 fp32 entries, one copy per lane of a wave
+constexpr int LUT_BYTES = 256 * 256;    // byte -> (fp32, fp32) of its two codes, 32 copies: 256 B per byte value
 
 template <int BM>
 struct Tile {
     static constexpr int XA = BM / 64;  // 16-byte x loads per thread and k step
-    static constexpr int A_BYTES = BM * ROW_BYTES;
-    static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+    static constexpr int STAGE_BYTES = BM * ROW_BYTES;
     static constexpr int SMEM_BYTES = LUT_BYTES + 2 * STAGE_BYTES;
-    static constexpr int TI = BM / 64;  // 32-row MFMA tiles per wave along m (wave tile BM/2 x 64)
-    static constexpr int TJ = 2;        // along n
+    static constexpr int TI = BM / 32;  // 32-row MFMA tiles per wave (every wave covers all BM rows)
     static constexpr int HI = TI / 2;   // x tiles per half slice
 };
 
-// What one thread holds of a k step on its way from global memory to LDS.
-template <int XA>
-struct Staged {
-    uint4 x[XA];  // XA x 8 bf16 of the x tile
+struct Codes {
     uint4 w;      // 32 codes of one weight row
     float scale;  // absmax of their block
 };
 
-template <bool NESTED, int XA>
-__device__ __forceinline__ void load_step(const MatmulArgs& a, Staged<XA>& st, const uint16_t* const (&xrow)[XA],
-                                          int64_t e0, int k0) {
-#pragma unroll
-    for (int u = 0; u < XA; ++u) st.x[u] = load16(xrow[u] + k0);
-    const int64_t e = e0 + k0;
-    st.w = load16(a.packed + (e >> 1));
+template <bool NESTED>
+__device__ __forceinline__ void load_codes(const MatmulArgs& a, Codes& c, int64_t e) {
+    c.w = load16(a.packed + (e >> 1));
     const int64_t blk = e >> a.block_log2;
-    st.scale = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
+    c.scale = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
 }
 
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t orv) {
@@ -69,58 +67,57 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t o
     return r;
 }
 
-// LDS addresses of the code-book entries of the 8 codes of one dword, in element order (high
-// nibble of a byte first).  The book sits at the start of the workgroup's LDS, 256 bytes per
-// code, one fp32 per lane: address = book | code << 8 | lane * 4, `book_lane` = book | lane * 4.
-__device__ __forceinline__ void lut_addresses(uint32_t d, uint32_t book_lane, uint32_t (&addr)[8]) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        addr[2 * b] = and_or(b == 0 ? d << 4 : d >> (8 * b - 4), 0xf00u, book_lane);
-        addr[2 * b + 1] = and_or(b == 0 ? d << 8 : b == 1 ? d : d >> (8 * b - 8), 0xf00u, book_lane);
-    }
+// The pair book: for every byte value (two codes) the two fp32 code-book entries, high nibble first,
+// in 32 copies: address = book | byte << 8 | copy << 3.  A lane uses copy lane % 32, so the 32 lanes
+// that the LDS serves together hit 32 different bank pairs whatever their bytes are.
+__device__ __forceinline__ void lut_addresses(uint32_t d, uint32_t book_lane, uint32_t (&addr)[4]) {
+    addr[0] = and_or(d << 8, 0xff00u, book_lane);
+    addr[1] = and_or(d, 0xff00u, book_lane);
+    addr[2] = and_or(d >> 8, 0xff00u, book_lane);
+    addr[3] = and_or(d >> 16, 0xff00u, book_lane);
 }
 
-__device__ __forceinline__ float lds_f32(uint32_t addr) {
-    return *reinterpret_cast<const __attribute__((address_space(3))) float*>(addr);
+__device__ __forceinline__ float2_t lds_f32x2(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) float2_t*>(addr);
 }
 
 __device__ __forceinline__ uint32_t dword_of(const uint4& w, int p) {
     return p == 0 ? w.x : p == 1 ? w.y : p == 2 ? w.z : w.w;
 }
 
-// 8 code-book values of one dword -> 8 bf16 = bf16_rne(value * scale), as 16 bytes
-__device__ __forceinline__ uint4 scale_round(const float (&v)[8], float scale) {
-    uint32_t o[4];
+// 8 code-book values of one dword -> 8 bf16 = bf16_rne(value * scale): one MFMA B fragment
+__device__ __forceinline__ bf16x8 scale_round(const float (&v)[8], float scale) {
+    u32x4v o;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const float2_t f = {__fmul_rn(v[2 * c], scale), __fmul_rn(v[2 * c + 1], scale)};
         o[c] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
     }
-    return make_uint4(o[0], o[1], o[2], o[3]);
+    return __builtin_bit_cast(bf16x8, o);
 }
 
+// 8 waves, wave w: all BM rows of x by weight rows n0 + 32 w .. + 31.  Lane l holds weight row l % 32,
+// codes 32 (l / 32) .. + 31 of the k step; its dword s is the B fragment of slice s, covering
+// k = 32 (l / 32) + 8 s .. + 7, and the x fragments are read from LDS in the same k order.
 template <bool NESTED, int BM>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
     using T = Tile<BM>;
-    using St = Staged<T::XA>;
-    // 4 KiB alignment: the code-book addresses are formed with OR (lut_addresses)
     extern __shared__ __attribute__((aligned(4096))) uint8_t smem[];
     uint8_t* stages = smem + LUT_BYTES;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
 
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        const int idx = tid + THREADS * it;  // 1024 dwords: entry idx / 64, lane idx % 64
-        reinterpret_cast<float*>(smem)[idx] = a.lut16[idx >> 6];
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+        const int e = tid + THREADS * it;  // 8192 entries: byte value e / 32, copy e % 32
+        const int byte = e >> 5;
+        const float2_t pair = {a.lut16[byte >> 4], a.lut16[byte & 15]};
+        *reinterpret_cast<float2_t*>(smem + (byte << 8) + ((e & 31) << 3)) = pair;
     }
     typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
-    const uint32_t book_lane = (uint32_t)(uintptr_t)(lds_ptr)smem + lane * 4;
+    const uint32_t book_lane = (uint32_t)(uintptr_t)(lds_ptr)smem + (lane & 31) * 8;
 
-    // Workgroups are handed to the 8 XCDs round-robin; give every XCD a contiguous run of tiles,
-    // m fastest, so that the m tiles sharing one n tile's weights hit that XCD's L2.
     const int total = m_tiles * n_tiles;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int chunk = total >> 3, rem = total & 7;
@@ -129,121 +126,126 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
     const int mt = id - nt * m_tiles;
     const int m0 = mt * BM, n0 = nt * BN;
 
-    f32x16 acc[T::TI][T::TJ];
+    f32x16 acc[T::TI];
 #pragma unroll
     for (int i = 0; i < T::TI; ++i)
 #pragma unroll
-        for (int j = 0; j < T::TJ; ++j)
-#pragma unroll
-            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
+        for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
 
-    // Load bases.  x: thread -> row tid / 8 (+ 64 u), 16 bytes tid % 8 of the 128-byte k step; codes:
-    // thread -> weight row tid / 2, half tid % 2 of the 64 codes.  Rows beyond M or N are clamped to
-    // the last one (their outputs are never stored).
     const uint16_t* xrow[T::XA];
 #pragma unroll
     for (int u = 0; u < T::XA; ++u)
         xrow[u] = a.x + (int64_t)min(m0 + (tid >> 3) + 64 * u, a.M - 1) * a.K + (tid & 7) * 8;
-    const int64_t e0 = (int64_t)min(n0 + (tid >> 1), a.N - 1) * a.K + (tid & 1) * 32;
-    const int a_st = (tid >> 3) * ROW_BYTES + (tid & 7) * 16;               // + 64 u rows
-    const int b_st = T::A_BYTES + (tid >> 1) * ROW_BYTES + (tid & 1) * 64;  // + 16 bytes per dword of codes
+    const int a_st = (tid >> 3) * ROW_BYTES + (tid & 7) * 16;  // + 64 u rows
+    const int64_t e0 = (int64_t)min(n0 + wave * 32 + (lane & 31), a.N - 1) * a.K + (lane >> 5) * 32;
+    const int a_off = (lane & 31) * ROW_BYTES + (lane >> 5) * 64;  // + 32 i rows, + 16 bytes per slice
 
     const int ksteps = a.K / BK;
-    St s0, s1;
-    load_step<NESTED>(a, s0, xrow, e0, 0);
-    if (ksteps > 1) load_step<NESTED>(a, s1, xrow, e0, BK);
+    uint4 xa[T::XA];
+    Codes c0, c1;
+#pragma unroll
+    for (int u = 0; u < T::XA; ++u) xa[u] = load16(xrow[u]);
+    load_codes<NESTED>(a, c0, e0);
+    if (ksteps > 1) load_codes<NESTED>(a, c1, e0 + BK);
     __syncthreads();  // code book visible
 #pragma unroll
-    for (int u = 0; u < T::XA; ++u) *reinterpret_cast<uint4*>(stages + a_st + u * 64 * ROW_BYTES) = s0.x[u];
+    for (int u = 0; u < T::XA; ++u) *reinterpret_cast<uint4*>(stages + a_st + u * 64 * ROW_BYTES) = xa[u];
+    if (ksteps > 1) {
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        uint32_t addr[8];
+        for (int u = 0; u < T::XA; ++u) xa[u] = load16(xrow[u] + BK);
+    }
+    bf16x8 fb;
+    {
+        uint32_t addr[4];
         float v[8];
-        lut_addresses(dword_of(s0.w, p), book_lane, addr);
+        lut_addresses(c0.w.x, book_lane, addr);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) v[c] = lds_f32(addr[c]);
-        *reinterpret_cast<uint4*>(stages + b_st + p * 16) = scale_round(v, s0.scale);
+        for (int c = 0; c < 4; ++c) {
+            const float2_t p = lds_f32x2(addr[c]);
+            v[2 * c] = p.x;
+            v[2 * c + 1] = p.y;
+        }
+        fb = scale_round(v, c0.scale);
     }
     __syncthreads();
 
-    const int frag_row = lane & 31;
-    const int frag_k = (lane >> 5) * 16;  // byte offset of this lane's 8 bf16 inside a 16-k slice
-    const int a_off = (wm * (BM / 2) + frag_row) * ROW_BYTES + frag_k;
-    const int b_off = T::A_BYTES + (wn * (BN / 4) + frag_row) * ROW_BYTES + frag_k;
-
-    // One k step: MFMAs on stage kt & 1 in eight half slices (half of the wave's x tiles, both W
-    // tiles, 16 k), the fragments of the next half slice read while the MFMAs of this one run.
-    // `stg` (step kt + 1) is expanded into the other stage between them: code-book reads of dword p
-    // in half slice 2p; scaling, rounding and the stores in half slice 2p + 1.  `ld` then receives
-    // step kt + 2.  The scheduling fences keep each half slice's reads, MFMAs and expansion together.
-    auto step = [&](int kt, St& ld, St& stg, auto full) {
+    // One k step.  `cur` holds the codes of step kt (dword 0 already expanded into fb), `nxt` those
+    // of step kt + 1; xa holds the x rows of step kt + 1.
+    auto step = [&](int kt, Codes& cur, Codes& nxt, auto full) {
         constexpr bool FULL = decltype(full)::value;  // steps kt + 1 and kt + 2 exist
-        const uint8_t* cur = stages + (kt & 1) * T::STAGE_BYTES;
-        uint8_t* nxt = stages + ((kt + 1) & 1) * T::STAGE_BYTES;
+        const uint8_t* st = stages + (kt & 1) * T::STAGE_BYTES;
+        uint8_t* st_next = stages + ((kt + 1) & 1) * T::STAGE_BYTES;
         const bool more = FULL || kt + 1 < ksteps;
-        bf16x8 fa[2][T::HI], fb[2][T::TJ];
-        auto read_frags = [&](int h) {
-            const int kk = h >> 1, ih = h & 1;
+        const bool more2 = FULL || kt + 2 < ksteps;
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < T::XA; ++u) *reinterpret_cast<uint4*>(st_next + a_st + u * 64 * ROW_BYTES) = xa[u];
+        }
+        if (more2) {
+#pragma unroll
+            for (int u = 0; u < T::XA; ++u) xa[u] = load16(xrow[u] + (kt + 2) * BK);
+        }
+        bf16x8 fa[2][T::HI];
+        auto read_frags = [&](int h) {  // half slice h: slice h / 2, x tiles (h % 2) * HI ..
 #pragma unroll
             for (int i = 0; i < T::HI; ++i)
-                fa[h & 1][i] =
-                    *reinterpret_cast<const bf16x8*>(cur + a_off + (ih * T::HI + i) * 32 * ROW_BYTES + kk * 32);
-#pragma unroll
-            for (int j = 0; j < T::TJ; ++j)
-                fb[h & 1][j] = *reinterpret_cast<const bf16x8*>(cur + b_off + j * 32 * ROW_BYTES + kk * 32);
+                fa[h & 1][i] = *reinterpret_cast<const bf16x8*>(st + a_off + ((h & 1) * T::HI + i) * 32 * ROW_BYTES +
+                                                                (h >> 1) * 16);
         };
         float v[8];
+        bf16x8 fbn = fb;
         read_frags(0);
 #pragma unroll
         for (int h = 0; h < 8; ++h) {
+            const int kk = h >> 1;
             if (h < 7) read_frags(h + 1);
 #pragma unroll
             for (int i = 0; i < T::HI; ++i)
-#pragma unroll
-                for (int j = 0; j < T::TJ; ++j)
-                    acc[(h & 1) * T::HI + i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        fa[h & 1][i], fb[h & 1][j], acc[(h & 1) * T::HI + i][j], 0, 0, 0);
-            if (more) {
+                acc[(h & 1) * T::HI + i] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[h & 1][i], fb, acc[(h & 1) * T::HI + i], 0, 0, 0);
+            // the B fragment of the next slice: dword kk + 1 of this step, or dword 0 of the next step
+            if (kk < 3 || more) {
+                const Codes& src = kk < 3 ? cur : nxt;
                 if ((h & 1) == 0) {
-                    uint32_t addr[8];
-                    lut_addresses(dword_of(stg.w, h >> 1), book_lane, addr);
+                    uint32_t addr[4];
+                    lut_addresses(dword_of(src.w, (kk + 1) & 3), book_lane, addr);
 #pragma unroll
-                    for (int c = 0; c < 8; ++c) v[c] = lds_f32(addr[c]);
+                    for (int c = 0; c < 4; ++c) {
+                        const float2_t p = lds_f32x2(addr[c]);
+                        v[2 * c] = p.x;
+                        v[2 * c + 1] = p.y;
+                    }
                 } else {
-                    *reinterpret_cast<uint4*>(nxt + b_st + (h >> 1) * 16) = scale_round(v, stg.scale);
-                    if ((h >> 1) < T::XA)
-                        *reinterpret_cast<uint4*>(nxt + a_st + (h >> 1) * 64 * ROW_BYTES) = stg.x[h >> 1];
+                    fbn = scale_round(v, src.scale);
                 }
             }
+            if (h == 6 && more2) load_codes<NESTED>(a, cur, e0 + (int64_t)(kt + 2) * BK);  // cur's dwords are used up
             __builtin_amdgcn_sched_barrier(0);
+            if (h & 1) fb = fbn;
         }
-        if (FULL || kt + 2 < ksteps) load_step<NESTED>(a, ld, xrow, e0, (kt + 2) * BK);
         __syncthreads();
     };
-    // step 0 is in LDS, s1 holds step 1
     int kt = 0;
     for (; kt + 3 < ksteps; kt += 2) {
-        step(kt, s0, s1, std::true_type{});      // expands s1 (step kt + 1), loads step kt + 2 into s0
-        step(kt + 1, s1, s0, std::true_type{});  // expands s0 (step kt + 2), loads step kt + 3 into s1
+        step(kt, c0, c1, std::true_type{});
+        step(kt + 1, c1, c0, std::true_type{});
     }
     for (; kt + 1 < ksteps; kt += 2) {
-        step(kt, s0, s1, std::false_type{});
-        step(kt + 1, s1, s0, std::false_type{});
+        step(kt, c0, c1, std::false_type{});
+        step(kt + 1, c1, c0, std::false_type{});
     }
-    if (kt < ksteps) step(kt, s0, s1, std::false_type{});
+    if (kt < ksteps) step(kt, c0, c1, std::false_type{});
 
-    // acc[i][j][q] = out[m][n], n = lane & 31, m = 8*(q/4) + 4*(lane/32) + q%4 inside the 32x32 tile
-#pragma unroll
-    for (int j = 0; j < T::TJ; ++j) {
-        const int n = n0 + wn * (BN / 4) + j * 32 + (lane & 31);
-        if (n >= a.N) continue;
+    // acc[i][q] = out[m][n], n = lane & 31, m = 8*(q/4) + 4*(lane/32) + q%4 inside the 32x32 tile
+    const int n = n0 + wave * 32 + (lane & 31);
+    if (n < a.N) {
         const float b = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.0f;
 #pragma unroll
         for (int i = 0; i < T::TI; ++i)
 #pragma unroll
             for (int q = 0; q < 16; ++q) {
-                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (q >> 2) + 4 * (lane >> 5) + (q & 3);
-                if (m < a.M) a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(acc[i][j][q] + b);
+                const int m = m0 + i * 32 + 8 * (q >> 2) + 4 * (lane >> 5) + (q & 3);
+                if (m < a.M) a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(acc[i][q] + b);
             }
     }
 }
@@ -277,7 +279,6 @@ hipError_t launch_tile(const MatmulArgs& a, hipStream_t stream) {
 size_t gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
 
 hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream) {
-    // 128-row tiles while one of them covers x: the weight tile is expanded once per tile of x rows
     if (a.M <= 128) return a.nested.q ? launch_tile<true, 128>(a, stream) : launch_tile<false, 128>(a, stream);
     return a.nested.q ? launch_tile<true, 256>(a, stream) : launch_tile<false, 256>(a, stream);
 }

@@ -27,7 +27,7 @@ SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
 # kernel has no such variant, so those calls go to the prefill kernel, which is exact by construction.
 EXACT_K = 16384
 # From this many rows of x on, HIP dequantize followed by the dense library GEMM is the default
-# (the fused GEMM kernel re-expands the weight tile once per 256 rows of x and reaches 0.9-1.0
+# (the fused GEMM kernel re-expands the weight tile once per 256 rows of x and reaches 0.96-1.05
 # PFLOP/s, the library GEMM 1.1-1.5 PFLOP/s and the dequantize kernel runs at HBM speed); see
 # _fused_gemm_wins for where the fused kernel is faster all the same.  Raise it to force the
 # fused, allocation-free kernel everywhere.
@@ -238,15 +238,27 @@ FUSED_GEMM_MIN_N = 28672
 
 
 def _fused_gemm_wins(M: int, N: int) -> bool:
-    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Measured on MI355X: for tall
-    weights and up to 512 rows of x it saves more by not writing the bf16 weight than it loses to the
-    library GEMM -- [28672, 4096]: 85 vs 111 us (M = 96), 133 vs 153 (512), 252 vs 209 (768);
-    [28672, 8192] M = 512: 252 vs 295; lm_head [128256, 4096]: 214 vs 453 (128), 289 vs 519 (256),
-    560 vs 733 (512), 844 vs 896 (768), 1151 vs 1085 (1024).  Shorter weights leave most CUs without a
-    tile ([14336, 4096]: 107 vs 74 us at M = 256)."""
+    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Measured on MI355X (us, fused vs
+    dense): for tall weights and a few hundred rows of x it saves more by not writing the bf16 weight
+    than it loses to the library GEMM -- [28672, 4096]: 62 vs 110 (M = 128), 125 vs 153 (512), 230
+    vs 198 (640); [28672, 8192] M = 512: 239 vs 294; [57344, 8192]: 477 vs 585 (512), 716 vs 761 (768),
+    954 vs 932 (1024); lm_head [128256, 4096]: 172 vs 456 (128), 274 vs 533 (256), 535 vs 738 (512),
+    1038 vs 1109 (1024).  Shorter weights leave most CUs without a tile ([14336, 4096]: 96 vs 77 at
+    M = 256)."""
     if N < FUSED_GEMM_MIN_N:
         return False
-    return M <= 512 or (M <= 768 and N >= 4 * FUSED_GEMM_MIN_N)
+    return M <= (512 if N < 2 * FUSED_GEMM_MIN_N else 768 if N < 4 * FUSED_GEMM_MIN_N else 1024)
+
+
+def _fused_gemm_us(N: int, K: int) -> float:
+    """Model of the fused GEMM kernel's time for up to 128 rows of x (one tile of x rows): tiles of
+    256 weight rows run in rounds of 256 (one per CU), K / 64 steps each, a step taking 0.9 us on a
+    sparsely filled chip and 1.3 us on a full one ([28672, 4096]: 60, [28672, 8192]: 125,
+    [57344, 8192]: 154, lm_head [128256, 4096]: 167 us measured)."""
+    tiles = (N + 255) // 256
+    rounds = (tiles + 255) // 256
+    fill = min(1.0, tiles / rounds / 256.0)
+    return rounds * (K // 64) * (0.9 + 0.4 * fill)
 
 
 def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
@@ -254,16 +266,16 @@ def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
     weight cheaper than the alternatives?  All sides modelled from measurements on MI355X
     (microseconds, W = weights in millions): a 16-row pass takes 12 + 0.105 W; the dense route
     20 + 0.62 W before its GEMM, and the passes must beat that by 20 %; the fused GEMM kernel, where
-    it applies, 52 + 0.28 W for up to 128 rows.  [28672, 4096]: up to M = 48 (73 us vs 85 fused, 111
-    dense), lm_head [128256, 4096]: up to M = 32 (134 vs 200 fused); [14336, 4096]: up to M = 32
-    (36 vs 55 dense); below 40 M weights never."""
+    it applies, _fused_gemm_us.  [28672, 4096] and lm_head [128256, 4096]: up to M = 32 (49 us vs 60
+    fused, 134 vs 167); [28672, 8192]: up to M = 48 (110 vs 125); [14336, 4096]: up to M = 32 (36 vs 55
+    dense); below 40 M weights never."""
     n_weights = N * K
     if M <= 16 or n_weights < 40_000_000:
         return False
     w = n_weights / 1e6
     passes = (M + 15) // 16
     t = passes * (12.0 + 0.105 * w)
-    if _fused_gemm_wins(M, N) and t >= 52.0 + 0.28 * w:
+    if _fused_gemm_wins(M, N) and t >= _fused_gemm_us(N, K):
         return False
     return t < 0.8 * (20.0 + 0.62 * w)
 

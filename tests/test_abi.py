@@ -126,11 +126,13 @@ def test_fused_route_rules(ta):
     assert route(8, 64, 1344) == "gemm"                   # fused GEMM kernel below DENSE_ROUTE_MIN_M rows
     assert route(17, 64, 4096) == "dequant+gemm" and route(2048, 4096, 4096) == "dequant+gemm"
     # a few more than 16 rows on a large weight: the decode kernel once per 16 rows
-    assert route(17, 28672, 4096) == "gemv-chunks" and route(48, 28672, 4096) == "gemv-chunks"
-    assert route(49, 28672, 4096) == "gemm" and route(512, 28672, 4096) == "gemm"  # tall weight: fused GEMM
+    assert route(17, 28672, 4096) == "gemv-chunks" and route(32, 28672, 4096) == "gemv-chunks"
+    assert route(33, 28672, 4096) == "gemm" and route(512, 28672, 4096) == "gemm"  # tall weight: fused GEMM
     assert route(513, 28672, 4096) == "dequant+gemm"
     assert route(32, 128256, 4096) == "gemv-chunks" and route(33, 128256, 4096) == "gemm"
-    assert route(768, 128256, 4096) == "gemm" and route(769, 128256, 4096) == "dequant+gemm"
+    assert route(1024, 128256, 4096) == "gemm" and route(1025, 128256, 4096) == "dequant+gemm"
+    assert route(48, 28672, 8192) == "gemv-chunks" and route(49, 28672, 8192) == "gemm"
+    assert route(768, 57344, 8192) == "gemm" and route(769, 57344, 8192) == "dequant+gemm"
     assert route(256, 28672, 8192) == "gemm" and route(256, 14336, 4096) == "dequant+gemm"
     assert route(32, 14336, 4096) == "gemv-chunks" and route(33, 14336, 4096) == "dequant+gemm"
     assert route(32, 4096, 4096) == "dequant+gemm"        # small weight: dequantize is cheap

@@ -467,7 +467,7 @@ def test_gemv_chunks_route(ta, nested):
     """17..48 rows of x on a large weight go through the decode kernel 16 rows at a time: every
     chunk boundary and a ragged last chunk, with bias, against a float64-accumulated matmul over sampled
     rows of the HIP-dequantized weight."""
-    N, K = 28672, 4096
+    N, K = 28672, 8192
     _sync_print(f"gemv-chunks nested={nested}")
     g = torch.Generator(device=DEV).manual_seed(99)
     w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)

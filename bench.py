@@ -212,9 +212,11 @@ MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CUs x 2.4 GHz x 4096 flop/clk/CU
 
 def prefill_section(torch, ta) -> dict:
     """BASELINE config 3, outside the timed region of the GEMV metric: the Llama-3-8B projection
-    shapes with M in {512, 2048, 8192} rows of x through ``matmul_nf4`` (which routes them to
-    nf4hip_dequantize + the dense library GEMM), and the fused NF4 GEMM kernel (nf4hip_gemm) at
-    M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events bracket 10 calls (3 for the fused kernel) after 3 warm-up calls."""
+    shapes (and the fused gate/up weight [28672, 4096]) with M in {512, 2048, 8192} rows of x through
+    ``matmul_nf4`` -- which routes them to nf4hip_dequantize + the dense library GEMM, or to the fused
+    NF4 GEMM kernel (nf4hip_gemm) for the tall weight at M = 512 -- and the fused kernel forced at
+    M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events bracket 10 calls (3 for the forced
+    fused kernel) after 3 warm-up calls."""
     dev = torch.device("cuda:0")
     F = ta.functional
     code = ta.nf4_code(dev)
@@ -232,16 +234,17 @@ def prefill_section(torch, ta) -> dict:
         return e0.elapsed_time(e1) * 1e-3 / reps
 
     rows = []
-    for si, (N, K) in enumerate([(4096, 4096), (14336, 4096), (4096, 14336)]):
+    routes = {"dequant+gemm": "nf4hip_dequantize + dense GEMM", "gemm": "nf4hip_gemm (fused)"}
+    for si, (N, K) in enumerate([(4096, 4096), (14336, 4096), (4096, 14336), (28672, 4096)]):
         g = torch.Generator(device=dev).manual_seed(3000 + si)
         w = (torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
         qw, absmax, _ = ta.quantize_nf4(w, BLOCKSIZE)
         del w
         for M in (512, 2048, 8192):
             x = torch.randn(M, K, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-            assert F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K)) == "dequant+gemm"
+            route = routes[F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))]
             t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 10)
-            row = {"N": N, "K": K, "M": M, "route": "nf4hip_dequantize + dense GEMM", "us": round(t * 1e6, 1),
+            row = {"N": N, "K": K, "M": M, "route": route, "us": round(t * 1e6, 1),
                    "tflops": round(2.0 * M * N * K / t / 1e12, 1),
                    "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
             rows.append(row)
@@ -252,7 +255,7 @@ def prefill_section(torch, ta) -> dict:
                     t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 3)
                 finally:
                     F.DENSE_ROUTE_MIN_M = saved
-                rows.append({"N": N, "K": K, "M": M, "route": "nf4hip_gemm (fused)", "us": round(t * 1e6, 1),
+                rows.append({"N": N, "K": K, "M": M, "route": "nf4hip_gemm (fused, forced)", "us": round(t * 1e6, 1),
                              "tflops": round(2.0 * M * N * K / t / 1e12, 1),
                              "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
     return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows}

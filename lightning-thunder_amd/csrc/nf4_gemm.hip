@@ -52,6 +52,7 @@ struct Tile {
 struct Codes {
     uint4 w;      // 32 codes of one weight row
     float scale;  // absmax of their block
+    uint32_t q;   // nested absmax only: the 8-bit absmax code of the step this set is loaded with next
 };
 
 template <bool NESTED>
@@ -59,6 +60,19 @@ __device__ __forceinline__ void load_codes(const MatmulArgs& a, Codes& c, int64_
     c.w = load16(a.packed + (e >> 1));
     const int64_t blk = e >> a.block_log2;
     c.scale = NESTED ? nested_absmax(a.nested, blk) : a.absmax[blk];
+}
+
+// Nested absmax inside the k loop: the 8-bit code is fetched one step before the two look-ups that
+// depend on it, so that no load in the loop waits for another (same arithmetic as nested_absmax).
+__device__ __forceinline__ void load_absmax_code(const MatmulArgs& a, Codes& c, int64_t e) {
+    c.q = a.nested.q[e >> a.block_log2];
+}
+__device__ __forceinline__ void load_codes_staged(const MatmulArgs& a, Codes& c, int64_t e) {
+    c.w = load16(a.packed + (e >> 1));
+    const int64_t blk = e >> a.block_log2;
+    const float m = a.nested.map256[c.q];
+    const float s = a.nested.absmax2[blk >> a.nested.nested_log2];
+    c.scale = __fadd_rn(__fmul_rn(m, s), a.nested.offset);
 }
 
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t orv) {
@@ -147,6 +161,7 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
     for (int u = 0; u < T::XA; ++u) xa[u] = load16(xrow[u]);
     load_codes<NESTED>(a, c0, e0);
     if (ksteps > 1) load_codes<NESTED>(a, c1, e0 + BK);
+    if (NESTED && ksteps > 2) load_absmax_code(a, c0, e0 + 2 * BK);
     __syncthreads();  // code book visible
 #pragma unroll
     for (int u = 0; u < T::XA; ++u) *reinterpret_cast<uint4*>(stages + a_st + u * 64 * ROW_BYTES) = xa[u];
@@ -219,7 +234,14 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
                     fbn = scale_round(v, src.scale);
                 }
             }
-            if (h == 6 && more2) load_codes<NESTED>(a, cur, e0 + (int64_t)(kt + 2) * BK);  // cur's dwords are used up
+            if (h == 6 && more2) {  // cur's dwords are used up
+                if (NESTED) {
+                    load_codes_staged(a, cur, e0 + (int64_t)(kt + 2) * BK);
+                    if (kt + 3 < ksteps) load_absmax_code(a, nxt, e0 + (int64_t)(kt + 3) * BK);
+                } else {
+                    load_codes<false>(a, cur, e0 + (int64_t)(kt + 2) * BK);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
             if (h & 1) fb = fbn;
         }

@@ -330,6 +330,9 @@ def test_gemm_bias_nested_blocksize(ta, oracle, fused_gemm):
     _matmul_case(ta, oracle, 64, 256, 1024, bias=True, seed=1)
     _matmul_case(ta, oracle, 64, 256, 1024, nested=True, seed=2)
     _matmul_case(ta, oracle, 64, 256, 1024, blocksize=256, seed=3)
+    for K in (64, 128, 192, 256, 320):  # 1..5 k steps: the nested absmax look-ups are staged across steps
+        _matmul_case(ta, oracle, 40, 300, K, nested=True, bias=True, seed=4 + K)
+        _matmul_case(ta, oracle, 200, 300, K, nested=True, seed=5 + K)
 
 
 @pytest.mark.parametrize("case", ["fp32", "fp16", "K_not_64", "n_lt_block"])

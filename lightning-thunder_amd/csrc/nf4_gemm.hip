@@ -122,12 +122,14 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
     const int lane = tid & 63;
     const int wave = tid >> 6;
 
-#pragma unroll 4
-    for (int it = 0; it < 16; ++it) {
-        const int e = tid + THREADS * it;  // 8192 entries: byte value e / 32, copy e % 32
-        const int byte = e >> 5;
-        const float2_t pair = {a.lut16[byte >> 4], a.lut16[byte & 15]};
-        *reinterpret_cast<float2_t*>(smem + (byte << 8) + ((e & 31) << 3)) = pair;
+    // pair book: thread tid writes copy tid % 32 of the 16 byte values (it << 4) | (tid / 32)
+    {
+        const float second = a.lut16[tid >> 5];
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+            const float2_t pair = {a.lut16[it], second};
+            *reinterpret_cast<float2_t*>(smem + (((it << 4) | (tid >> 5)) << 8) + ((tid & 31) << 3)) = pair;
+        }
     }
     typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
     const uint32_t book_lane = (uint32_t)(uintptr_t)(lds_ptr)smem + (lane & 31) * 8;

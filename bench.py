@@ -328,7 +328,8 @@ def llama_decode(torch, ta, n_new: int) -> dict:
     nweights = sum(m.weight.numel() for m in model.modules() if isinstance(m, torch.nn.Linear))
     out = {
         "model": "Llama-3-8B architecture (32 layers, d 4096, 32q/8kv heads, FFN 14336, vocab 128256), random init, "
-                 "all 161 linears NF4 (QKV and gate/up fused), prompt 512, greedy, HIP-graph decode step",
+                 "all 161 linears NF4 (QKV and gate/up fused), prompt 512, greedy, HIP-graph decode step; norms / rotary + attention / SiLU*up between the linears as 3 HIP kernels "
+                 "(decode_tok_per_s) or as PyTorch ops (decode_tok_per_s_torch_glue)",
         "new_tokens": n_new,
         "linear_weight_bytes_per_token": int(nweights * 0.5625),
         "hbm_bound_tok_per_s_batch1": round(HBM_PEAK_GBS * 1e9 / (nweights * 0.5625), 1),
@@ -337,12 +338,16 @@ def llama_decode(torch, ta, n_new: int) -> dict:
         g = torch.Generator(device=dev).manual_seed(4000 + B)
         prompt = torch.randint(0, cfg.vocab, (B, 512), generator=g, device=dev)
         D.greedy_decode(jm, cfg, prompt, n_new=1, use_graph=False)  # untimed: library start-up, GEMM heuristics
-        _, st = D.greedy_decode(jm, cfg, prompt, n_new=n_new, use_graph=True)
-        out[f"batch{B}"] = {
-            "decode_tok_per_s": round(st["decode_tok_per_s"], 1),
-            "ms_per_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
-            "prefill_ms": round(st["prefill_s"] * 1e3, 1),
-        }
+        res = {}
+        # the single-token step with the HIP glue kernels (norm, rotary + cache + attention, SiLU * up)
+        # around the NF4 linears, and with plain PyTorch ops in their place
+        for key, glue in (("", True), ("_torch_glue", False)):
+            cfg.hip_glue = glue
+            _, st = D.greedy_decode(jm, cfg, prompt, n_new=n_new, use_graph=True)
+            res[f"decode_tok_per_s{key}"] = round(st["decode_tok_per_s"], 1)
+            res[f"ms_per_step{key}"] = round(st["decode_s"] / st["decode_steps"] * 1e3, 3)
+            res["prefill_ms"] = round(st["prefill_s"] * 1e3, 1)
+        out[f"batch{B}"] = res
     return out
 
 

@@ -5,8 +5,10 @@ every ``nn.Linear`` is handed to ``BitsAndBytesLinearQuant4bit`` through ``jit``
 decoding loop whose single-token step is captured in a HIP graph, the way the reference's
 ``CUDAGraphTransform`` replays a forward pass (thunder/transforms/cudagraph.py:47-226) over weights
 tagged as static inputs (thunder/transforms/quantization.py:178,186).  Everything that is not a
-linear (norms, rotary embedding, attention, sampling) is plain PyTorch: it is plumbing around the
-path, not part of it.
+linear (norms, rotary embedding, attention, sampling) is plain PyTorch by default: it is plumbing
+around the path, not part of it.  With ``LlamaConfig.hip_glue`` the single-token step runs that work in
+three HIP kernels instead (``glue.py``: residual add + RMSNorm, rotary + cache update + attention,
+SiLU * up), so that the step is bound by the 4-bit linears rather than by ~18 small launches per layer.
 
 ``fused_projections=True`` builds Q/K/V and gate/up as ONE linear each ([6144, 4096] and
 [28672, 4096] for Llama-3-8B).  NF4 blocks are 64 consecutive elements of a row, so the packed
@@ -36,6 +38,7 @@ class LlamaConfig:
     norm_eps: float = 1e-5
     max_seq: int = 640
     fused_projections: bool = False
+    hip_glue: bool = False
 
     @property
     def head_dim(self) -> int:
@@ -150,7 +153,34 @@ class Llama(nn.Module):
         self.register_buffer("rope_sin", ang.sin(), persistent=False)
         self.register_buffer("key_index", torch.arange(cfg.max_seq), persistent=False)
 
+    def _decode_step_glue(self, idx, pos, kcache, vcache):
+        """The single-token forward with the HIP glue kernels: per layer four linears and four other
+        launches.  The residual stream x is updated in place by add_rmsnorm, which also returns the
+        normalised input of the next linear; `delta` is the branch output not yet added."""
+        from . import glue
+
+        cfg = self.cfg
+        H, Hkv, eps = cfg.n_head, cfg.n_kv_head, cfg.norm_eps
+        x = self.wte(idx)[:, 0, :].contiguous()
+        delta = None
+        for i, blk in enumerate(self.blocks):
+            h = glue.add_rmsnorm(x, delta, blk.norm_1.weight, eps)
+            a = blk.attn
+            if cfg.fused_projections:
+                qkv = a.qkv_proj(h)
+            else:
+                qkv = torch.cat((a.q_proj(h), a.k_proj(h), a.v_proj(h)), dim=-1)
+            y = glue.attention_decode(qkv, pos, self.rope_cos, self.rope_sin, kcache[i], vcache[i], H, Hkv)
+            delta = a.o_proj(y)
+            h = glue.add_rmsnorm(x, delta, blk.norm_2.weight, eps)
+            m = blk.mlp
+            gate_up = m.gate_up_proj(h) if cfg.fused_projections else torch.cat((m.gate_proj(h), m.up_proj(h)), dim=-1)
+            delta = m.down_proj(glue.silu_mul(gate_up))
+        return self.lm_head(glue.add_rmsnorm(x, delta, self.norm_f.weight, eps))
+
     def forward(self, idx, pos, kcache, vcache):
+        if self.cfg.hip_glue and idx.shape[1] == 1 and idx.is_cuda and self.wte.weight.dtype == torch.bfloat16:
+            return self._decode_step_glue(idx, pos, kcache, vcache)
         x = self.wte(idx)
         cos = self.rope_cos.index_select(0, pos)[:, None, :].to(x.dtype)
         sin = self.rope_sin.index_select(0, pos)[:, None, :].to(x.dtype)

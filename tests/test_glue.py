@@ -1,0 +1,171 @@
+"""Decode-step glue kernels (libnf4hip_decode.so): ABI checks without a GPU, and on the GPU each
+kernel against a plain PyTorch fp32 reference of the same operation, then the whole decode step."""
+
+import importlib
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def glue():
+    return importlib.import_module("lightning-thunder_amd.glue")
+
+
+@pytest.fixture(scope="module")
+def D():
+    return importlib.import_module("lightning-thunder_amd.decode")
+
+
+def test_library_exports_every_declared_symbol(glue):
+    text = open(os.path.join(ROOT, "include", "nf4hip_decode.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(nf4hip_decode_\w+)\s*\(", text)))
+    lib = glue.load()
+    assert len(declared) == 5
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/nf4hip_decode.h but not exported"
+    assert sorted(glue.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
+
+
+def test_argument_errors_come_before_any_hip_call(glue):
+    lib = glue.load()
+    A = 4096  # non-null, 16-byte aligned fake device address: validation never dereferences
+    err = lambda: lib.nf4hip_decode_last_error().decode()
+    assert lib.nf4hip_decode_add_rmsnorm(None, None, A, 1e-5, 1, 64, A, None) == -1 and "null" in err()
+    assert lib.nf4hip_decode_add_rmsnorm(A, None, A, 1e-5, 1, 60, A, None) == -1 and "multiple of 8" in err()
+    assert lib.nf4hip_decode_add_rmsnorm(A, None, A, 1e-5, 1, 32768, A, None) == -1
+    assert lib.nf4hip_decode_add_rmsnorm(A + 2, None, A, 1e-5, 1, 64, A, None) == -1 and "aligned" in err()
+    assert lib.nf4hip_decode_attention(A, A, A, A, A, A, 1, 8, 3, 128, 64, A, None, 0, None) == -1 and "multiple" in err()
+    assert lib.nf4hip_decode_attention(A, A, A, A, A, A, 1, 8, 2, 96, 64, A, None, 0, None) == -1 and "head_dim" in err()
+    assert lib.nf4hip_decode_attention(A, None, A, A, A, A, 1, 8, 2, 128, 64, A, None, 0, None) == -1 and "null" in err()
+    assert lib.nf4hip_decode_attention(A, A, A, A, A, A, 1, 8, 2, 128, 64, A, None, 0, None) == -1 and "workspace" in err()
+    assert lib.nf4hip_decode_attention(A, A, A, A, A, A, 1, 8, 2, 128, 64, A, A, 100, None) == -1 and "workspace" in err()
+    assert lib.nf4hip_decode_attention_workspace_bytes(1, 32, 128) == 4096 + 32 * 8 * 130 * 4
+    assert lib.nf4hip_decode_attention_workspace_bytes(8, 32, 128) == 4096 + 256 * 4 * 130 * 4
+    assert lib.nf4hip_decode_attention_workspace_bytes(64, 32, 128) == 0  # one workgroup per (sequence, head) is plenty
+    assert lib.nf4hip_decode_silu_mul(A, 1, 12, A, None) == -1 and "multiple of 8" in err()
+    assert lib.nf4hip_decode_silu_mul(A, 0, 16, A, None) == -1
+
+
+def test_missing_library_fails_loudly(glue, tmp_path):
+    with pytest.raises(RuntimeError, match="not found"):
+        glue.load(str(tmp_path / "libnf4hip_decode.so"))
+
+
+def _randn(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(torch.bfloat16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,d", [(1, 4096), (8, 4096), (3, 512), (2, 16384), (5, 72)])
+def test_add_rmsnorm(glue, rows, d):
+    print(f"add_rmsnorm rows={rows} d={d}", flush=True)
+    x, delta, w = _randn((rows, d), 1), _randn((rows, d), 2, 0.3), _randn((d,), 3) + 1
+    for use_delta in (True, False):
+        xd = x.to(DEV).clone()
+        y = glue.add_rmsnorm(xd, delta.to(DEV) if use_delta else None, w.to(DEV), 1e-5)
+        x_new = (x + delta) if use_delta else x  # bf16 add: one rounding, as the kernel does
+        assert torch.equal(xd.cpu(), x_new)
+        xf = x_new.float()
+        ref = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5) * w.float()
+        torch.testing.assert_close(y.cpu().float(), ref, rtol=8e-3, atol=1e-3)  # one bf16 rounding of the result
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,dff", [(1, 14336), (8, 14336), (3, 1024), (2, 8)])
+def test_silu_mul(glue, rows, dff):
+    print(f"silu_mul rows={rows} dff={dff}", flush=True)
+    gu = _randn((rows, 2 * dff), 4, 2.0)
+    out = glue.silu_mul(gu.to(DEV)).cpu()
+    g, u = gu[:, :dff].float(), gu[:, dff:].float()
+    ref = torch.nn.functional.silu(g) * u
+    torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1e-3)  # two bf16 roundings
+    torch_glue = (torch.nn.functional.silu(gu[:, :dff]) * gu[:, dff:]).float()
+    assert ((out.float() - torch_glue).abs() <= 8e-3 * torch_glue.abs() + 1e-6).all()  # at most one bf16 ulp apart
+
+
+def _rope_ref(x, cos, sin):  # x [..., hd] fp32, cos/sin [hd]
+    x1, x2 = x.chunk(2, dim=-1)
+    return x * cos + torch.cat((-x2, x1), dim=-1) * sin
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,Hkv,hd,max_seq,p", [
+    (1, 32, 8, 128, 640, 512), (8, 32, 8, 128, 640, 639), (3, 8, 2, 64, 64, 0), (2, 8, 8, 64, 64, 17),
+    (2, 4, 1, 128, 300, 299), (1, 32, 8, 128, 640, 1), (40, 32, 8, 128, 96, 70), (16, 32, 8, 128, 640, 300),
+])
+def test_attention_decode(glue, B, H, Hkv, hd, max_seq, p):
+    print(f"attention_decode B={B} H={H} Hkv={Hkv} hd={hd} max_seq={max_seq} p={p}", flush=True)
+    qkv = _randn((B, (H + 2 * Hkv) * hd), 5)
+    kc0, vc0 = _randn((B, Hkv, max_seq, hd), 6), _randn((B, Hkv, max_seq, hd), 7)
+    inv = 1.0 / (500000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    ang = torch.outer(torch.arange(max_seq, dtype=torch.float32), inv).repeat(1, 2)
+    cos, sin = ang.cos(), ang.sin()
+    kc, vc = kc0.to(DEV).clone(), vc0.to(DEV).clone()
+    pos = torch.tensor([p], device=DEV)
+    out = glue.attention_decode(qkv.to(DEV), pos, cos.to(DEV), sin.to(DEV), kc, vc, H, Hkv).cpu()
+    # again on the same workspace (its arrival counters must be back at zero): same result
+    again = glue.attention_decode(qkv.to(DEV), pos, cos.to(DEV), sin.to(DEV), kc, vc, H, Hkv).cpu()
+    assert torch.equal(out, again)
+    # reference, fp32
+    heads = qkv.float().reshape(B, H + 2 * Hkv, hd)
+    q = _rope_ref(heads[:, :H], cos[p], sin[p]).to(torch.bfloat16).float()
+    k_new = _rope_ref(heads[:, H:H + Hkv], cos[p], sin[p]).to(torch.bfloat16)
+    v_new = qkv.reshape(B, H + 2 * Hkv, hd)[:, H + Hkv:]
+    kref, vref = kc0.clone(), vc0.clone()
+    kref[:, :, p], vref[:, :, p] = k_new, v_new
+    # cache: only row p changes; v exactly, k to within one bf16 ulp of the fp32 rotation
+    assert torch.equal(vc.cpu(), vref)
+    kdiff = (kc.cpu().float() - kref.float()).abs()
+    assert (kdiff <= 8e-3 * kref.float().abs() + 1e-6).all()
+    rows = torch.arange(max_seq) != p
+    assert torch.equal(kc.cpu()[:, :, rows], kc0[:, :, rows])
+    rep = H // Hkv
+    kf = kc.cpu().float()[:, :, : p + 1].repeat_interleave(rep, dim=1)  # the kernel's own k row p
+    vf = vref.float()[:, :, : p + 1].repeat_interleave(rep, dim=1)
+    scores = torch.einsum("bhd,bhsd->bhs", q, kf) * hd ** -0.5
+    ref = torch.einsum("bhs,bhsd->bhd", torch.softmax(scores, dim=-1), vf).reshape(B, H * hd)
+    torch.testing.assert_close(out.float(), ref, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("batch", [1, 8])
+def test_decode_with_hip_glue(D, ta, fused, batch):
+    """The single-token step with the glue kernels: HIP-graph replay equals the eager loop token for
+    token, and its logits agree with the plain-PyTorch step of the same quantized model."""
+    print(f"decode hip_glue fused={fused} batch={batch}", flush=True)
+    dev = torch.device(DEV)
+    cfg = D.LlamaConfig.tiny(fused_projections=fused, hip_glue=True)
+    model = D.build_llama(cfg, device=dev, seed=5)
+    jm = ta.jit(model, transforms=[ta.BitsAndBytesLinearQuant4bit()])
+    g = torch.Generator(device=dev).manual_seed(2)
+    prompt = torch.randint(0, cfg.vocab, (batch, 16), generator=g, device=dev)
+    eager, s0 = D.greedy_decode(jm, cfg, prompt, n_new=12, use_graph=False)
+    graph, s1 = D.greedy_decode(jm, cfg, prompt, n_new=12, use_graph=True)
+    assert s1["graph"] and not s0["graph"]
+    assert torch.equal(eager, graph)
+
+    # one decode step after the same prefill, glue vs plain PyTorch around the same quantized linears
+    kc, vc = D.new_caches(cfg, batch, dev)
+    kr, vr = D.new_caches(cfg, batch, dev)
+    pos = torch.arange(16, device=dev)
+    first = jm(prompt, pos, kc, vc).argmax(-1, keepdim=True)
+    jm(prompt, pos, kr, vr)
+    p1 = torch.full((1,), 16, device=dev, dtype=torch.long)
+    a = jm(first, p1, kc, vc).float()
+    cfg.hip_glue = False
+    try:
+        b = jm(first, p1, kr, vr).float()
+    finally:
+        cfg.hip_glue = True
+    torch.testing.assert_close(a, b, rtol=3e-2, atol=3e-2)
+    torch.testing.assert_close(kc[:, :, :, :17].float(), kr[:, :, :, :17].float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(vc[:, :, :, :17].float(), vr[:, :, :, :17].float(), rtol=2e-2, atol=2e-2)

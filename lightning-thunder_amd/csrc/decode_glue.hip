@@ -395,20 +395,26 @@ __attribute__((visibility("default"))) int nf4hip_decode_attention(const void* q
     const int sg = ATTN_THREADS / (head_dim / 8);
     const size_t lds = sizeof(float) * (size_t)(3 * head_dim + 8 + sg * head_dim + max_seq);
     const dim3 grid((unsigned)n_head, (unsigned)batch, (unsigned)splits);
-    hipError_t e;
-    if (head_dim == 128) {
-        if ((e = allow_lds(attention_decode_kernel<128>, lds)) != hipSuccess) return fail("nf4hip_decode_attention: LDS size");
-        hipLaunchKernelGGL(attention_decode_kernel<128>, grid, dim3(ATTN_THREADS), lds, static_cast<hipStream_t>(stream),
-                           static_cast<const uint16_t*>(qkv), pos, cos_t, sin_t, static_cast<uint16_t*>(kcache),
-                           static_cast<uint16_t*>(vcache), n_head, n_kv_head, (int)max_seq, static_cast<uint16_t*>(out),
-                           splits, counters, partials);
-    } else {
-        if ((e = allow_lds(attention_decode_kernel<64>, lds)) != hipSuccess) return fail("nf4hip_decode_attention: LDS size");
-        hipLaunchKernelGGL(attention_decode_kernel<64>, grid, dim3(ATTN_THREADS), lds, static_cast<hipStream_t>(stream),
-                           static_cast<const uint16_t*>(qkv), pos, cos_t, sin_t, static_cast<uint16_t*>(kcache),
-                           static_cast<uint16_t*>(vcache), n_head, n_kv_head, (int)max_seq, static_cast<uint16_t*>(out),
-                           splits, counters, partials);
+    // allow the whole 160 KB of LDS once per device (what a launch takes is its own `lds`)
+    static bool ready[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail("nf4hip_decode_attention: no current device");
+    if (!ready[dev]) {
+        if (allow_lds(attention_decode_kernel<128>, 160 * 1024) != hipSuccess ||
+            allow_lds(attention_decode_kernel<64>, 160 * 1024) != hipSuccess)
+            return fail("nf4hip_decode_attention: LDS size");
+        ready[dev] = true;
     }
+    auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, grid, dim3(ATTN_THREADS), lds, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(qkv), pos, cos_t, sin_t, static_cast<uint16_t*>(kcache),
+                           static_cast<uint16_t*>(vcache), n_head, n_kv_head, (int)max_seq, static_cast<uint16_t*>(out),
+                           splits, counters, partials);
+    };
+    if (head_dim == 128)
+        launch(attention_decode_kernel<128>);
+    else
+        launch(attention_decode_kernel<64>);
     return hipGetLastError() == hipSuccess ? 0 : fail("nf4hip_decode_attention: launch failed");
 }
 

@@ -393,6 +393,39 @@ def test_matmul_randomized_sweep_large(ta):
     assert {"gemv", "gemv-chunks", "dequant+gemm"} <= seen
 
 
+def test_gemm_randomized_sweep(ta, fused_gemm):
+    """Seeded sweep over the fused GEMM kernel alone (forced for every shape): both tile heights, ragged
+    M and N, 1..33 k steps, every blocksize, bias, nested absmax; against a float64-accumulated
+    matmul over the HIP-dequantized weight."""
+    rng = torch.Generator().manual_seed(8765)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rng))]
+
+    code = ta.nf4_code(DEV)
+    for case in range(60):
+        M = pick([17, 31, 100, 128, 129, 200, 255, 256, 257, 400, 511, 513, 600])
+        K = pick([64, 128, 192, 256, 320, 512, 1024, 2048 + 64])
+        N = pick([2, 31, 64, 255, 256, 257, 1000, 4096 + 18, 9000])
+        blocksize = pick([b for b in (64, 64, 128, 256, 512, 1024, 2048) if K % b == 0])
+        bias = pick([False, True])
+        nested = pick([False, False, True])
+        _sync_print(f"gemm sweep {case}: M={M} N={N} K={K} bs={blocksize} bias={bias} nested={nested}")
+        g = torch.Generator(device=DEV).manual_seed(1000 + case)
+        w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+        x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+        b = torch.randn(N, generator=g, device=DEV).to(torch.bfloat16) if bias else None
+        qw, absmax, _ = ta.quantize_nf4(w, blocksize)
+        state = ta.compress_absmax(absmax) if nested else absmax
+        deq = ta.dequantize_nf4(qw, state, code, blocksize, torch.bfloat16, (N, K))
+        assert ta.functional.fused_route(x, b, blocksize, torch.bfloat16, (N, K)) == "gemm"
+        y = ta.matmul_nf4(x, qw, b, state, code, blocksize, torch.bfloat16, (N, K))
+        ref = x.double() @ deq.double().t()
+        if bias:
+            ref = ref + b.double()
+        torch.testing.assert_close(y.double(), ref, rtol=2e-2, atol=2e-2)
+
+
 def test_full_size_properties(ta):
     """Llama-3-8B FFN shape at full size through size-independent properties: quantize is
     idempotent on its own dequantisation, and gemv is linear in x."""

@@ -6,7 +6,7 @@
 // bf16 in registers -- bf16_rne(lut16[code] * absmax), the same value nf4hip_dequantize produces --
 // and contracts them with bf16 MFMA, fp32 accumulation, bf16 output.
 //
-// Tile: BM (128 or 256 rows of x) x 256 (n) x 64 (k) per workgroup of 512 threads.  Wave w of 8
+// Tile: BM (64, 128 or 256 rows of x) x 256 (n) x 64 (k) per workgroup of 512 threads.  Wave w of 8
 // owns weight rows 32 w .. + 31 of the tile against all BM rows of x: BM / 32 accumulators of
 // v_mfma_f32_32x32x16_bf16 with A = x (from LDS) and B = W (from this wave's registers).  A lane
 // loads 16 bytes = 32 codes of one weight row per k step; each of its four dwords becomes the B
@@ -303,6 +303,7 @@ hipError_t launch_tile(const MatmulArgs& a, hipStream_t stream) {
 size_t gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
 
 hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream) {
+    if (a.M <= 64) return a.nested.q ? launch_tile<true, 64>(a, stream) : launch_tile<false, 64>(a, stream);
     if (a.M <= 128) return a.nested.q ? launch_tile<true, 128>(a, stream) : launch_tile<false, 128>(a, stream);
     return a.nested.q ? launch_tile<true, 256>(a, stream) : launch_tile<false, 256>(a, stream);
 }

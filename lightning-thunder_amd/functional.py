@@ -250,15 +250,17 @@ def _fused_gemm_wins(M: int, N: int) -> bool:
     return M <= (512 if N < 2 * FUSED_GEMM_MIN_N else 768 if N < 4 * FUSED_GEMM_MIN_N else 1024)
 
 
-def _fused_gemm_us(N: int, K: int) -> float:
+def _fused_gemm_us(M: int, N: int, K: int) -> float:
     """Model of the fused GEMM kernel's time for up to 128 rows of x (one tile of x rows): tiles of
-    256 weight rows run in rounds of 256 (one per CU), K / 64 steps each, a step taking 0.9 us on a
-    sparsely filled chip and 1.3 us on a full one ([28672, 4096]: 60, [28672, 8192]: 125,
-    [57344, 8192]: 154, lm_head [128256, 4096]: 167 us measured)."""
+    256 weight rows run in rounds of 256 (one per CU), K / 64 steps each; a step takes 0.65 us (64-row
+    tile, M <= 64) or 0.9 us (128-row tile) on a sparsely filled chip and 0.3 / 0.4 us more on a full
+    one (measured, M = 64 / 128: [28672, 4096] 45 / 60, [28672, 8192] 90 / 125, [57344, 8192] 113 / 154,
+    lm_head [128256, 4096] 121 / 167 us)."""
     tiles = (N + 255) // 256
     rounds = (tiles + 255) // 256
     fill = min(1.0, tiles / rounds / 256.0)
-    return rounds * (K // 64) * (0.9 + 0.4 * fill)
+    step = 0.65 + 0.3 * fill if M <= 64 else 0.9 + 0.4 * fill
+    return rounds * (K // 64) * step
 
 
 def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
@@ -266,16 +268,16 @@ def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
     weight cheaper than the alternatives?  All sides modelled from measurements on MI355X
     (microseconds, W = weights in millions): a 16-row pass takes 12 + 0.105 W; the dense route
     20 + 0.62 W before its GEMM, and the passes must beat that by 20 %; the fused GEMM kernel, where
-    it applies, _fused_gemm_us.  [28672, 4096] and lm_head [128256, 4096]: up to M = 32 (49 us vs 60
-    fused, 134 vs 167); [28672, 8192]: up to M = 48 (110 vs 125); [14336, 4096]: up to M = 32 (36 vs 55
-    dense); below 40 M weights never."""
+    it applies, _fused_gemm_us.  [28672, 8192]: up to M = 32 (73 us vs 90 fused); [28672, 4096]: up to
+    M = 32 (a tie: 49 vs 45-50); lm_head [128256, 4096]: never (134 vs 121 at M = 32); [14336, 4096]: up to
+    M = 32 (36 vs 55 dense); [16384, 8192]: up to M = 48; below 40 M weights never."""
     n_weights = N * K
     if M <= 16 or n_weights < 40_000_000:
         return False
     w = n_weights / 1e6
     passes = (M + 15) // 16
     t = passes * (12.0 + 0.105 * w)
-    if _fused_gemm_wins(M, N) and t >= _fused_gemm_us(N, K):
+    if _fused_gemm_wins(M, N) and t >= _fused_gemm_us(M, N, K):
         return False
     return t < 0.8 * (20.0 + 0.62 * w)
 

@@ -129,9 +129,10 @@ def test_fused_route_rules(ta):
     assert route(17, 28672, 4096) == "gemv-chunks" and route(32, 28672, 4096) == "gemv-chunks"
     assert route(33, 28672, 4096) == "gemm" and route(512, 28672, 4096) == "gemm"  # tall weight: fused GEMM
     assert route(513, 28672, 4096) == "dequant+gemm"
-    assert route(32, 128256, 4096) == "gemv-chunks" and route(33, 128256, 4096) == "gemm"
+    assert route(17, 128256, 4096) == "gemm" and route(64, 128256, 4096) == "gemm"  # 64-row tiles beat two passes
     assert route(1024, 128256, 4096) == "gemm" and route(1025, 128256, 4096) == "dequant+gemm"
-    assert route(48, 28672, 8192) == "gemv-chunks" and route(49, 28672, 8192) == "gemm"
+    assert route(32, 28672, 8192) == "gemv-chunks" and route(33, 28672, 8192) == "gemm"
+    assert route(48, 16384, 8192) == "gemv-chunks" and route(49, 16384, 8192) == "dequant+gemm"
     assert route(768, 57344, 8192) == "gemm" and route(769, 57344, 8192) == "dequant+gemm"
     assert route(256, 28672, 8192) == "gemm" and route(256, 14336, 4096) == "dequant+gemm"
     assert route(32, 14336, 4096) == "gemv-chunks" and route(33, 14336, 4096) == "dequant+gemm"

@@ -301,7 +301,7 @@ def test_gemm_shapes(ta, oracle, M, N, K, fused_gemm):
 
 
 @pytest.mark.parametrize("M,N,K,kw", [
-    (49, 28672, 512, {}), (128, 28700, 576, {"bias": True}), (129, 28672, 640, {"nested": True}),
+    (20, 28672, 512, {}), (49, 28672, 512, {}), (64, 28700, 576, {"nested": True}), (128, 28700, 576, {"bias": True}), (129, 28672, 640, {"nested": True}),
     (300, 28930, 512, {"blocksize": 256}), (512, 28672, 1024, {}), (700, 4 * 28672, 128, {"bias": True}),
 ])
 def test_gemm_route_tall_weights(ta, oracle, M, N, K, kw):
@@ -503,7 +503,7 @@ def test_gemv_chunks_route(ta, nested):
     """17..48 rows of x on a large weight go through the decode kernel 16 rows at a time: every
     chunk boundary and a ragged last chunk, with bias, against a float64-accumulated matmul over sampled
     rows of the HIP-dequantized weight."""
-    N, K = 28672, 8192
+    N, K = 16384, 8192
     _sync_print(f"gemv-chunks nested={nested}")
     g = torch.Generator(device=DEV).manual_seed(99)
     w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)

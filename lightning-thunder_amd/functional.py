@@ -233,34 +233,45 @@ def _gemv_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 
 # The fused GEMM kernel works on tiles of 256 weight rows; from this many rows on a weight has enough
-# tiles to fill the chip's 256 CUs with one tile of x rows.
+# tiles for more than 128 rows of x (tiles of 256 rows of x) to be worth it.
 FUSED_GEMM_MIN_N = 28672
-
-
-def _fused_gemm_wins(M: int, N: int) -> bool:
-    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Measured on MI355X (us, fused vs
-    dense): for tall weights and a few hundred rows of x it saves more by not writing the bf16 weight
-    than it loses to the library GEMM -- [28672, 4096]: 62 vs 110 (M = 128), 125 vs 153 (512), 230
-    vs 198 (640); [28672, 8192] M = 512: 239 vs 294; [57344, 8192]: 477 vs 585 (512), 716 vs 761 (768),
-    954 vs 932 (1024); lm_head [128256, 4096]: 172 vs 456 (128), 274 vs 533 (256), 535 vs 738 (512),
-    1038 vs 1109 (1024).  Shorter weights leave most CUs without a tile ([14336, 4096]: 96 vs 77 at
-    M = 256)."""
-    if N < FUSED_GEMM_MIN_N:
-        return False
-    return M <= (512 if N < 2 * FUSED_GEMM_MIN_N else 768 if N < 4 * FUSED_GEMM_MIN_N else 1024)
 
 
 def _fused_gemm_us(M: int, N: int, K: int) -> float:
     """Model of the fused GEMM kernel's time for up to 128 rows of x (one tile of x rows): tiles of
-    256 weight rows run in rounds of 256 (one per CU), K / 64 steps each; a step takes 0.65 us (64-row
-    tile, M <= 64) or 0.9 us (128-row tile) on a sparsely filled chip and 0.3 / 0.4 us more on a full
-    one (measured, M = 64 / 128: [28672, 4096] 45 / 60, [28672, 8192] 90 / 125, [57344, 8192] 113 / 154,
-    lm_head [128256, 4096] 121 / 167 us)."""
+    256 weight rows run in rounds of 256 (one per CU), K / 64 steps each; a step takes 0.6 us (64-row
+    tile, M <= 64) or 0.8 us (128-row tile) on a sparsely filled chip and 0.35 / 0.5 us more on a full
+    one (measured, M = 64 / 128: [14336, 4096] 44 / 58, [16384, 8192] 79 / 106, [28672, 4096] 45 / 60,
+    [57344, 8192] 113 / 154, lm_head [128256, 4096] 121 / 167 us)."""
     tiles = (N + 255) // 256
     rounds = (tiles + 255) // 256
     fill = min(1.0, tiles / rounds / 256.0)
-    step = 0.65 + 0.3 * fill if M <= 64 else 0.9 + 0.4 * fill
+    step = 0.6 + 0.35 * fill if M <= 64 else 0.8 + 0.5 * fill
     return rounds * (K // 64) * step
+
+
+def _dense_route_us(N: int, K: int) -> float:
+    """Model of the dense route before its GEMM: the dequantize kernel writes 2 bytes per weight at HBM
+    speed, 20 + 0.62 W us for W million weights (measured with the GEMM of 64 rows of x: [14336, 4096]
+    56, [28672, 4096] 108, [16384, 8192] 115, lm_head [128256, 4096] 428 us)."""
+    return 20.0 + 0.62 * N * K / 1e6
+
+
+def _fused_gemm_wins(M: int, N: int, K: int) -> bool:
+    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Up to 128 rows of x the two
+    models above decide (the fused kernel's time hardly depends on N while the chip is not full, the
+    dense route's grows with the weight: [14336, 4096] M = 64 44 vs 56 us, [6144, 4096] 41 vs 41,
+    [4096, 14336] 140 vs 66).  Beyond that, measured on MI355X (us, fused vs dense): for tall weights
+    and a few hundred rows of x the fused kernel saves more by not writing the bf16 weight than it
+    loses to the library GEMM -- [28672, 4096]: 125 vs 153 (512), 230 vs 198 (640); [28672, 8192] M = 512:
+    239 vs 294; [57344, 8192]: 477 vs 585 (512), 716 vs 761 (768), 954 vs 932 (1024); lm_head
+    [128256, 4096]: 274 vs 533 (256), 535 vs 738 (512), 1038 vs 1109 (1024).  Shorter weights leave
+    most CUs without a tile ([14336, 4096]: 96 vs 77 at M = 256)."""
+    if M <= 128:
+        return _fused_gemm_us(M, N, K) < _dense_route_us(N, K)
+    if N < FUSED_GEMM_MIN_N:
+        return False
+    return M <= (512 if N < 2 * FUSED_GEMM_MIN_N else 768 if N < 4 * FUSED_GEMM_MIN_N else 1024)
 
 
 def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
@@ -277,9 +288,9 @@ def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
     w = n_weights / 1e6
     passes = (M + 15) // 16
     t = passes * (12.0 + 0.105 * w)
-    if _fused_gemm_wins(M, N) and t >= _fused_gemm_us(M, N, K):
+    if _fused_gemm_wins(M, N, K) and t >= _fused_gemm_us(M, N, K):
         return False
-    return t < 0.8 * (20.0 + 0.62 * w)
+    return t < 0.8 * _dense_route_us(N, K)
 
 
 def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape) -> str:
@@ -312,8 +323,8 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
     if K % 512 == 0 and _chunked_gemv_wins(M, N, K):
         return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
-    if _fused_gemm_wins(M, N):
-        return "gemm"  # tall weight, few hundred rows of x: expand the weight tiles in LDS
+    if _fused_gemm_wins(M, N, K):
+        return "gemm"  # expanding the weight tiles in registers beats writing the bf16 weight out
     # the fused GEMM kernel streams K sequentially per tile: beyond EXACT_K even a few rows of x are
     # served faster by dequantize + dense GEMM
     return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M or K > EXACT_K else "gemm"

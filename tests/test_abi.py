@@ -125,20 +125,22 @@ def test_fused_route_rules(ta):
     assert route(5, 64, 1376) == "dequant+linear"        # tile kernel needs K % 512, gemm K % 64
     assert route(8, 64, 1344) == "gemm"                   # fused GEMM kernel below DENSE_ROUTE_MIN_M rows
     assert route(17, 64, 4096) == "dequant+gemm" and route(2048, 4096, 4096) == "dequant+gemm"
-    # a few more than 16 rows on a large weight: the decode kernel once per 16 rows
-    assert route(17, 28672, 4096) == "gemv-chunks" and route(32, 28672, 4096) == "gemv-chunks"
-    assert route(33, 28672, 4096) == "gemm" and route(512, 28672, 4096) == "gemm"  # tall weight: fused GEMM
+    # a few more than 16 rows on a large weight: the decode kernel once per 16 rows, unless one launch of the
+    # fused GEMM (64- or 128-row tile) is modelled faster
+    assert route(17, 28672, 8192) == "gemv-chunks" and route(32, 28672, 8192) == "gemv-chunks"
+    assert route(33, 28672, 8192) == "gemm" and route(512, 28672, 8192) == "gemm" and route(513, 28672, 8192) == "dequant+gemm"
+    assert route(17, 28672, 4096) == "gemm" and route(512, 28672, 4096) == "gemm"  # tall weight: fused GEMM
     assert route(513, 28672, 4096) == "dequant+gemm"
     assert route(17, 128256, 4096) == "gemm" and route(64, 128256, 4096) == "gemm"  # 64-row tiles beat two passes
     assert route(1024, 128256, 4096) == "gemm" and route(1025, 128256, 4096) == "dequant+gemm"
-    assert route(32, 28672, 8192) == "gemv-chunks" and route(33, 28672, 8192) == "gemm"
-    assert route(48, 16384, 8192) == "gemv-chunks" and route(49, 16384, 8192) == "dequant+gemm"
+    assert route(48, 16384, 8192) == "gemv-chunks" and route(64, 16384, 8192) == "gemm" and route(65, 16384, 8192) == "dequant+gemm"
     assert route(768, 57344, 8192) == "gemm" and route(769, 57344, 8192) == "dequant+gemm"
-    assert route(256, 28672, 8192) == "gemm" and route(256, 14336, 4096) == "dequant+gemm"
-    assert route(32, 14336, 4096) == "gemv-chunks" and route(33, 14336, 4096) == "dequant+gemm"
+    assert route(32, 14336, 4096) == "gemv-chunks" and route(33, 14336, 4096) == "gemm" and route(64, 14336, 4096) == "gemm"
+    assert route(65, 14336, 4096) == "dequant+gemm" and route(256, 14336, 4096) == "dequant+gemm"
     assert route(32, 4096, 4096) == "dequant+gemm"        # small weight: dequantize is cheap
     assert route(17, 28672, 4096 + 64) == "gemm"          # the tile kernel needs K % 512, the fused GEMM K % 64
-    assert route(17, 14336, 4096 + 64) == "dequant+gemm"
+    assert route(17, 4096, 14336 + 64) == "dequant+gemm"
+    assert route(17, 128, 64) == "gemm"                   # tiny: one launch instead of two
     assert route(16, 8192, 28672) == "gemv"              # K > 16384: the tile kernel's exact-weights variant
     assert route(17, 8192, 28672) == "gemv-chunks" and route(512, 8192, 28672) == "dequant+gemm"
     assert route(1, 8192, 28672) == "gemv"               # row-streaming kernel has an exact variant

@@ -282,7 +282,7 @@ def fused_gemm(ta, monkeypatch):
     monkeypatch.setattr(ta.functional, "DENSE_ROUTE_MIN_M", 1 << 30)
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 128, 64), (512, 1024, 4096), (2048, 4096, 4096)])
+@pytest.mark.parametrize("M,N,K", [(17, 128, 4096), (512, 1024, 4096), (2048, 4096, 4096)])
 def test_dense_route(ta, oracle, M, N, K):
     """Default route for many rows of x: nf4hip_dequantize + dense GEMM."""
     _sync_print(f"dequant+gemm M={M} N={N} K={K}")

@@ -116,10 +116,12 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
 /*
  * Prefill-shape fused dequant-matmul, M > 16.  Replaces the dequantize_4bit + F.linear route of
  * bitsandbytes.matmul_4bit (MatMul4Bit.forward), reached from thunder/transforms/quantization.py:39.
- * NF4 tiles are expanded to bf16 ( bf16(lut16[c] * absmax) ) in LDS and contracted with bf16 MFMA,
+ * NF4 codes are expanded to bf16 ( bf16(lut16[c] * absmax) ) on chip and contracted with bf16 MFMA,
  * fp32 accumulation, bf16 output.  Same operand layout and fast-path rules as nf4hip_gemv, except
- * K % 64 == 0 and blocksize == 64 ... 4096 dividing K.  The workspace is reserved for split-K
- * variants; nf4hip_gemm_workspace_bytes may return 0, in which case NULL is accepted.
+ * K % 64 == 0 and blocksize == 64 ... 4096 dividing K.  Up to 128 rows of x, K may be split over
+ * workgroups that meet in `workspace`: nf4hip_gemm_workspace_bytes(M,N,K) bytes (0 = none needed,
+ * NULL accepted), under the rules of nf4hip_gemv's workspace -- zeroed once, left zeroed where that
+ * matters, one stream at a time; the two kernels may share one workspace.
  */
 size_t nf4hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int nf4hip_gemm(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,

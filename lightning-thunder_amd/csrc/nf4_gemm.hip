@@ -17,11 +17,15 @@
 // value the two fp32 entries of its codes, in 32 copies laid out so that the 32 lanes the LDS serves
 // together never share a bank -- one ds_read_b64 per byte of codes.
 //
+// Up to 128 rows of x (one tile of x rows) K is split over up to 8 workgroups per weight tile when the
+// weight has too few tiles for the chip; their fp32 partial tiles meet in the workspace and the last
+// one to arrive adds them in split order.
+//
 // Pipeline per k step kt: x rows of step kt + 1 go from registers to the other LDS stage at the
 // top of the step and the registers are refilled with step kt + 2; codes and absmax run two steps
 // ahead in two register sets; the B fragment of slice s + 1 is expanded between the MFMAs of slice
 // s (pair-book reads in its first half, scaling and rounding in its second); one barrier per step.
-#include "nf4_common.h"
+#include "nf4_gemv.h"
 
 #include <type_traits>
 
@@ -114,7 +118,8 @@ __device__ __forceinline__ bf16x8 scale_round(const float (&v)[8], float scale) 
 // codes 32 (l / 32) .. + 31 of the k step; its dword s is the B fragment of slice s, covering
 // k = 32 (l / 32) + 8 s .. + 7, and the x fragments are read from LDS in the same k order.
 template <bool NESTED, int BM>
-__global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
+__global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles, int n_tiles, int splits,
+                                                           uint32_t* counters, float* partials) {
     using T = Tile<BM>;
     extern __shared__ __attribute__((aligned(4096))) uint8_t smem[];
     uint8_t* stages = smem + LUT_BYTES;
@@ -141,6 +146,9 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
     const int nt = id / m_tiles;
     const int mt = id - nt * m_tiles;
     const int m0 = mt * BM, n0 = nt * BN;
+    // K split over blockIdx.y: this workgroup's steps start at k_base
+    const int ksteps = a.K / BK / splits;
+    const int k_base = blockIdx.y * ksteps * BK;
 
     f32x16 acc[T::TI];
 #pragma unroll
@@ -151,12 +159,11 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
     const uint16_t* xrow[T::XA];
 #pragma unroll
     for (int u = 0; u < T::XA; ++u)
-        xrow[u] = a.x + (int64_t)min(m0 + (tid >> 3) + 64 * u, a.M - 1) * a.K + (tid & 7) * 8;
+        xrow[u] = a.x + (int64_t)min(m0 + (tid >> 3) + 64 * u, a.M - 1) * a.K + k_base + (tid & 7) * 8;
     const int a_st = (tid >> 3) * ROW_BYTES + (tid & 7) * 16;  // + 64 u rows
-    const int64_t e0 = (int64_t)min(n0 + wave * 32 + (lane & 31), a.N - 1) * a.K + (lane >> 5) * 32;
+    const int64_t e0 = (int64_t)min(n0 + wave * 32 + (lane & 31), a.N - 1) * a.K + k_base + (lane >> 5) * 32;
     const int a_off = (lane & 31) * ROW_BYTES + (lane >> 5) * 64;  // + 32 i rows, + 16 bytes per slice
 
-    const int ksteps = a.K / BK;
     uint4 xa[T::XA];
     Codes c0, c1;
 #pragma unroll
@@ -260,6 +267,44 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
     }
     if (kt < ksteps) step(kt, c0, c1, std::false_type{});
 
+    if (splits > 1) {
+        // Partial sums of this K split go to the workspace in register order ([i][q][thread]: coalesced);
+        // the last split to arrive for the tile adds all of them in split order (deterministic) and
+        // writes the result.  Ordering without L2-wide fences: agent-scope stores go through to L2, every
+        // store of the workgroup has completed (s_waitcnt, barrier) before its arrival is counted, and the
+        // last workgroup reads with agent-scope loads, which bypass its CU's L1.
+        float* tile_part = partials + (int64_t)id * splits * (T::TI * 16 * THREADS);
+        float* mine = tile_part + (int64_t)blockIdx.y * (T::TI * 16 * THREADS);
+#pragma unroll
+        for (int i = 0; i < T::TI; ++i)
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+                __hip_atomic_store(mine + (i * 16 + q) * THREADS + tid, acc[i][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        uint32_t* flag = reinterpret_cast<uint32_t*>(smem);
+        if (tid == 0) *flag = __hip_atomic_fetch_add(&counters[id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*flag != (uint32_t)(splits - 1)) return;
+#pragma unroll
+        for (int i = 0; i < T::TI; ++i) {
+            float sum[16];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) sum[q] = 0.0f;
+            for (int sp = 0; sp < splits; ++sp) {
+                const float* src = tile_part + (int64_t)sp * (T::TI * 16 * THREADS) + i * 16 * THREADS + tid;
+                float v[16];
+#pragma unroll
+                for (int q = 0; q < 16; ++q) v[q] = __hip_atomic_load(src + q * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int q = 0; q < 16; ++q) sum[q] += v[q];
+            }
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][q] = sum[q];
+        }
+        if (tid == 0) __hip_atomic_store(&counters[id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
     // acc[i][q] = out[m][n], n = lane & 31, m = 8*(q/4) + 4*(lane/32) + q%4 inside the 32x32 tile
     const int n = n0 + wave * 32 + (lane & 31);
     if (n < a.N) {
@@ -275,6 +320,21 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
 }
 
 constexpr int MAX_DEVICES = 64;
+// arrival counters at the head of the workspace: the same region as the decode kernels', so that one
+// zero-initialised workspace serves both (partial sums never land where the other expects zeroed counters)
+constexpr size_t GEMM_COUNTER_BYTES = GEMV_COUNTER_BYTES;
+
+// K splits for up to 128 rows of x (one tile of x rows): enough workgroups for the chip's 256 CUs when
+// the weight has few 256-row tiles; the k steps divide evenly and every split keeps at least 4.
+int gemm_splits(int64_t M, int64_t N, int64_t K) {
+    if (M > 128) return 1;
+    const int64_t tiles = (N + BN - 1) / BN;
+    const int64_t ksteps = K / BK;
+    int best = 1;
+    for (int s = 2; s <= 8; ++s)
+        if (tiles * s <= 512 && ksteps % s == 0 && ksteps / s >= 4) best = s;
+    return tiles * best > 1024 ? 1 : best;
+}
 
 template <bool NESTED, int BM>
 hipError_t launch_tile(const MatmulArgs& a, hipStream_t stream) {
@@ -293,16 +353,25 @@ hipError_t launch_tile(const MatmulArgs& a, hipStream_t stream) {
     }
     const int m_tiles = (a.M + BM - 1) / BM;
     const int n_tiles = (a.N + BN - 1) / BN;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(m_tiles * n_tiles)), dim3(THREADS), T::SMEM_BYTES, stream, a, m_tiles,
-                       n_tiles);
+    const int splits = gemm_splits(a.M, a.N, a.K);
+    uint32_t* counters = static_cast<uint32_t*>(a.workspace);
+    float* partials = splits > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(a.workspace) + GEMM_COUNTER_BYTES) : nullptr;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(m_tiles * n_tiles), (unsigned)splits), dim3(THREADS), T::SMEM_BYTES, stream, a,
+                       m_tiles, n_tiles, splits, counters, partials);
     return hipGetLastError();
 }
 
 }  // namespace
 
-size_t gemm_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int splits = gemm_splits(M, N, K);
+    if (splits == 1) return 0;
+    const int64_t bm = M <= 64 ? 64 : 128;
+    return GEMM_COUNTER_BYTES + (size_t)((N + BN - 1) / BN) * splits * bm * BN * sizeof(float);
+}
 
 hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream) {
+    // the smallest tile height that covers x with one tile: the weight tile is expanded once per tile of x rows
     if (a.M <= 64) return a.nested.q ? launch_tile<true, 64>(a, stream) : launch_tile<false, 64>(a, stream);
     if (a.M <= 128) return a.nested.q ? launch_tile<true, 128>(a, stream) : launch_tile<false, 128>(a, stream);
     return a.nested.q ? launch_tile<true, 256>(a, stream) : launch_tile<false, 256>(a, stream);

@@ -237,17 +237,34 @@ def _gemv_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 FUSED_GEMM_MIN_N = 28672
 
 
+def _gemm_splits(M: int, N: int, K: int) -> int:
+    """K splits the fused GEMM kernel uses (gemm_splits in csrc/nf4_gemm.hip): up to 128 rows of x,
+    enough workgroups for the chip's 256 CUs when the weight has few 256-row tiles; the k steps divide
+    evenly and every split keeps at least 4."""
+    if M > 128:
+        return 1
+    tiles, ksteps = (N + 255) // 256, K // 64
+    best = 1
+    for s in range(2, 9):
+        if tiles * s <= 512 and ksteps % s == 0 and ksteps // s >= 4:
+            best = s
+    return best
+
+
 def _fused_gemm_us(M: int, N: int, K: int) -> float:
     """Model of the fused GEMM kernel's time for up to 128 rows of x (one tile of x rows): tiles of
-    256 weight rows run in rounds of 256 (one per CU), K / 64 steps each; a step takes 0.6 us (64-row
-    tile, M <= 64) or 0.8 us (128-row tile) on a sparsely filled chip and 0.35 / 0.5 us more on a full
-    one (measured, M = 64 / 128: [14336, 4096] 44 / 58, [16384, 8192] 79 / 106, [28672, 4096] 45 / 60,
-    [57344, 8192] 113 / 154, lm_head [128256, 4096] 121 / 167 us)."""
-    tiles = (N + 255) // 256
-    rounds = (tiles + 255) // 256
-    fill = min(1.0, tiles / rounds / 256.0)
+    256 weight rows x K splits run in rounds of 256 workgroups (one per CU), K / 64 / splits steps
+    each; a step takes 0.6 us (64-row tile, M <= 64) or 0.8 us (128-row tile) on a sparsely filled chip
+    and 0.35 / 0.5 us more on a full one; merging the splits adds 13 / 25 us, a launch 3 (measured,
+    M = 64 / 128: [4096, 4096] 21 / 34, [6144, 4096] 22 / 36, [4096, 14336] 35 / 52, [8192, 8192] 30 / 47,
+    [14336, 4096] 34 / 51, [28672, 4096] 42 / 60, lm_head [128256, 4096] 121 / 167 us)."""
+    splits = _gemm_splits(M, N, K)
+    wgs = (N + 255) // 256 * splits
+    rounds = (wgs + 255) // 256
+    fill = min(1.0, wgs / rounds / 256.0)
     step = 0.6 + 0.35 * fill if M <= 64 else 0.8 + 0.5 * fill
-    return rounds * (K // 64) * step
+    merge = 0.0 if splits == 1 else 13.0 if M <= 64 else 25.0
+    return 3.0 + rounds * (K // 64 // splits) * step + merge
 
 
 def _dense_route_us(N: int, K: int) -> float:
@@ -361,7 +378,9 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
             ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
             fn, fn_dq = lib.nf4hip_gemv, lib.nf4hip_gemv_dq
         else:
-            ws_ptr, ws_bytes = None, 0
+            need = lib.nf4hip_gemm_workspace_bytes(M, N, K)  # K split over workgroups: partial tiles and counters
+            ws = _gemv_workspace(x.device, need) if need else None
+            ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
             fn, fn_dq = lib.nf4hip_gemm, lib.nf4hip_gemm_dq
         bptr = None if b is None else b.data_ptr()
         # row chunks of x and out: one call, or 16 rows at a time (rows are contiguous, K and N even,

@@ -133,16 +133,18 @@ def test_fused_route_rules(ta):
     assert route(513, 28672, 4096) == "dequant+gemm"
     assert route(17, 128256, 4096) == "gemm" and route(64, 128256, 4096) == "gemm"  # 64-row tiles beat two passes
     assert route(1024, 128256, 4096) == "gemm" and route(1025, 128256, 4096) == "dequant+gemm"
-    assert route(48, 16384, 8192) == "gemv-chunks" and route(64, 16384, 8192) == "gemm" and route(65, 16384, 8192) == "dequant+gemm"
+    assert route(17, 16384, 8192) == "gemm" and route(128, 16384, 8192) == "gemm" and route(129, 16384, 8192) == "dequant+gemm"
     assert route(768, 57344, 8192) == "gemm" and route(769, 57344, 8192) == "dequant+gemm"
-    assert route(32, 14336, 4096) == "gemv-chunks" and route(33, 14336, 4096) == "gemm" and route(64, 14336, 4096) == "gemm"
-    assert route(65, 14336, 4096) == "dequant+gemm" and route(256, 14336, 4096) == "dequant+gemm"
-    assert route(32, 4096, 4096) == "dequant+gemm"        # small weight: dequantize is cheap
+    assert route(32, 57344, 8192) == "gemv-chunks" and route(33, 57344, 8192) == "gemm"
+    assert route(17, 14336, 4096) == "gemm" and route(128, 14336, 4096) == "gemm"  # K split over workgroups fills the chip
+    assert route(129, 14336, 4096) == "dequant+gemm" and route(256, 14336, 4096) == "dequant+gemm"
+    assert route(32, 4096, 14336) == "gemv-chunks" and route(33, 4096, 14336) == "gemm" and route(65, 4096, 14336) == "dequant+gemm"
+    assert route(32, 4096, 4096) == "gemm" and route(65, 4096, 4096) == "dequant+gemm"
+    assert route(17, 64, 4096) == "dequant+gemm"          # one tile, 64 sequential k steps: the dense route is quicker
     assert route(17, 28672, 4096 + 64) == "gemm"          # the tile kernel needs K % 512, the fused GEMM K % 64
-    assert route(17, 4096, 14336 + 64) == "dequant+gemm"
     assert route(17, 128, 64) == "gemm"                   # tiny: one launch instead of two
     assert route(16, 8192, 28672) == "gemv"              # K > 16384: the tile kernel's exact-weights variant
-    assert route(17, 8192, 28672) == "gemv-chunks" and route(512, 8192, 28672) == "dequant+gemm"
+    assert route(17, 8192, 28672) == "gemm" and route(512, 8192, 28672) == "dequant+gemm"  # the fused GEMM is exact at any K
     assert route(1, 8192, 28672) == "gemv"               # row-streaming kernel has an exact variant
     assert route(1, 64, 4096, dtype=torch.float32) == "dequant+linear"
     assert route(1, 64, 4096, xdtype=torch.float16, dtype=torch.float16) == "dequant+linear"

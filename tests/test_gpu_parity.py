@@ -280,6 +280,7 @@ def fused_gemm(ta, monkeypatch):
     """Route every M > 16 call to the fused GEMM kernel (the default router prefers HIP dequantize
     + the dense library GEMM from 17 rows on)."""
     monkeypatch.setattr(ta.functional, "DENSE_ROUTE_MIN_M", 1 << 30)
+    monkeypatch.setattr(ta.functional, "_chunked_gemv_wins", lambda M, N, K: False)
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 128, 4096), (512, 1024, 4096), (2048, 4096, 4096)])
@@ -390,7 +391,7 @@ def test_matmul_randomized_sweep_large(ta):
             ref = ref + b[rows].double()
         torch.testing.assert_close(y[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
         del w, x, qw, absmax, deq, y
-    assert {"gemv", "gemv-chunks", "dequant+gemm"} <= seen
+    assert {"gemv", "gemm", "dequant+gemm"} <= seen
 
 
 def test_gemm_randomized_sweep(ta, fused_gemm):
@@ -403,9 +404,9 @@ def test_gemm_randomized_sweep(ta, fused_gemm):
         return options[int(torch.randint(0, len(options), (1,), generator=rng))]
 
     code = ta.nf4_code(DEV)
-    for case in range(60):
-        M = pick([17, 31, 100, 128, 129, 200, 255, 256, 257, 400, 511, 513, 600])
-        K = pick([64, 128, 192, 256, 320, 512, 1024, 2048 + 64])
+    for case in range(90):
+        M = pick([17, 31, 33, 64, 65, 100, 128, 129, 200, 255, 256, 257, 400, 511, 513, 600])
+        K = pick([64, 128, 192, 256, 320, 512, 1024, 2048 + 64, 4096, 14336])  # K splits of 1, 2, 4, 8
         N = pick([2, 31, 64, 255, 256, 257, 1000, 4096 + 18, 9000])
         blocksize = pick([b for b in (64, 64, 128, 256, 512, 1024, 2048) if K % b == 0])
         bias = pick([False, True])
@@ -500,10 +501,10 @@ def test_gemv_every_m_on_large_weights(ta, N, K):
 
 @pytest.mark.parametrize("nested", [False, True])
 def test_gemv_chunks_route(ta, nested):
-    """17..48 rows of x on a large weight go through the decode kernel 16 rows at a time: every
-    chunk boundary and a ragged last chunk, with bias, against a float64-accumulated matmul over sampled
-    rows of the HIP-dequantized weight."""
-    N, K = 16384, 8192
+    """17..32 rows of x on a large weight go through the decode kernel 16 rows at a time: a full and
+    a ragged last chunk, with bias, against a float64-accumulated matmul over sampled rows of the
+    HIP-dequantized weight."""
+    N, K = 28672, 8192
     _sync_print(f"gemv-chunks nested={nested}")
     g = torch.Generator(device=DEV).manual_seed(99)
     w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
@@ -512,7 +513,7 @@ def test_gemv_chunks_route(ta, nested):
     deq = ta.dequantize_nf4(qw, state, code, 64, torch.bfloat16, (N, K))
     rows = torch.cat([torch.randint(0, N, (61,), generator=g, device=DEV), torch.tensor([0, N - 2, N - 1], device=DEV)])
     bias = torch.randn(N, generator=g, device=DEV).to(torch.bfloat16)
-    for M in (17, 32, 33, 48):
+    for M in (17, 20, 31, 32):
         x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
         assert ta.functional.fused_route(x, bias, 64, torch.bfloat16, (N, K)) == "gemv-chunks"
         y = ta.matmul_nf4(x.reshape(1, M, K), qw, bias, state, code, 64, torch.bfloat16, (N, K))

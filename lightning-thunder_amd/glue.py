@@ -35,7 +35,8 @@ _workspaces: dict = {}  # (device index, stream) -> zero-initialised scratch of 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Zero-initialised scratch, one per (device, stream); the kernel leaves its counters zeroed, so
     the buffer is reused without clearing."""
-    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    key = (idx, _raw_stream(idx) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
@@ -78,7 +79,13 @@ def _bf16_cuda(*tensors: torch.Tensor) -> None:
             raise ValueError(f"expected a contiguous bf16 tensor on the GPU, got {t.dtype} {t.device} contiguous={t.is_contiguous()}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    idx = t.device.index if t.device.index is not None else torch.cuda.current_device()
+    if _raw_stream is not None:
+        return _raw_stream(idx)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 

@@ -216,7 +216,8 @@ def prefill_section(torch, ta) -> dict:
     ``matmul_nf4`` -- which routes them to nf4hip_dequantize + the dense library GEMM, or to the fused
     NF4 GEMM kernel (nf4hip_gemm) for the tall weight at M = 512 -- and the fused kernel forced at
     M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events bracket 10 calls (3 for the forced
-    fused kernel) after 3 warm-up calls."""
+    fused kernel) after 3 warm-up calls.  ``rows64``: the same weights with 64 rows of x, the router's
+    route (the fused kernel, K split over workgroups) next to the dense route forced."""
     dev = torch.device("cuda:0")
     F = ta.functional
     code = ta.nf4_code(dev)
@@ -233,7 +234,7 @@ def prefill_section(torch, ta) -> dict:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3 / reps
 
-    rows = []
+    rows, mid = [], []
     routes = {"dequant+gemm": "nf4hip_dequantize + dense GEMM", "gemm": "nf4hip_gemm (fused)"}
     for si, (N, K) in enumerate([(4096, 4096), (14336, 4096), (4096, 14336), (28672, 4096)]):
         g = torch.Generator(device=dev).manual_seed(3000 + si)
@@ -258,7 +259,14 @@ def prefill_section(torch, ta) -> dict:
                 rows.append({"N": N, "K": K, "M": M, "route": "nf4hip_gemm (fused, forced)", "us": round(t * 1e6, 1),
                              "tflops": round(2.0 * M * N * K / t / 1e12, 1),
                              "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
-    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows}
+        # 64 rows of x (between the decode and the prefill regime): the router's choice, which is the fused
+        # kernel with K split over workgroups, next to the dense route (dequantize + library GEMM) forced
+        x = torch.randn(64, K, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        route = F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))
+        t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 20)
+        td = timed(lambda: torch.nn.functional.linear(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K))), 20)
+        mid.append({"N": N, "K": K, "M": 64, "route": route, "us": round(t * 1e6, 1), "dense_route_us": round(td * 1e6, 1)})
+    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows, "rows64": mid}
 
 
 def codec_section(torch, ta) -> dict:

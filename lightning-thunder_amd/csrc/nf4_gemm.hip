@@ -286,18 +286,30 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
         if (tid == 0) *flag = __hip_atomic_fetch_add(&counters[id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*flag != (uint32_t)(splits - 1)) return;
+        // G splits' worth of loads are issued before the first add, so the merge costs a few memory
+        // round trips instead of one per split
+        constexpr int G = BM <= 64 ? 8 : 4;
 #pragma unroll
         for (int i = 0; i < T::TI; ++i) {
             float sum[16];
 #pragma unroll
             for (int q = 0; q < 16; ++q) sum[q] = 0.0f;
-            for (int sp = 0; sp < splits; ++sp) {
-                const float* src = tile_part + (int64_t)sp * (T::TI * 16 * THREADS) + i * 16 * THREADS + tid;
-                float v[16];
+            for (int sp0 = 0; sp0 < splits; sp0 += G) {
+                float v[G][16];
 #pragma unroll
-                for (int q = 0; q < 16; ++q) v[q] = __hip_atomic_load(src + q * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int g = 0; g < G; ++g) {
+                    const int sp = min(sp0 + g, splits - 1);
+                    const float* src = tile_part + (int64_t)sp * (T::TI * 16 * THREADS) + i * 16 * THREADS + tid;
 #pragma unroll
-                for (int q = 0; q < 16; ++q) sum[q] += v[q];
+                    for (int q = 0; q < 16; ++q)
+                        v[g][q] = __hip_atomic_load(src + q * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    if (sp0 + g < splits) {
+#pragma unroll
+                        for (int q = 0; q < 16; ++q) sum[q] += v[g][q];
+                    }
             }
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][q] = sum[q];
@@ -324,16 +336,17 @@ constexpr int MAX_DEVICES = 64;
 // zero-initialised workspace serves both (partial sums never land where the other expects zeroed counters)
 constexpr size_t GEMM_COUNTER_BYTES = GEMV_COUNTER_BYTES;
 
-// K splits for up to 128 rows of x (one tile of x rows): enough workgroups for the chip's 256 CUs when
-// the weight has few 256-row tiles; the k steps divide evenly and every split keeps at least 4.
+// K splits for up to 128 rows of x (one tile of x rows): as many workgroups as fit the chip's 256 CUs in
+// one round when the weight has few 256-row tiles; the k steps divide evenly and every split keeps at
+// least 4.
 int gemm_splits(int64_t M, int64_t N, int64_t K) {
     if (M > 128) return 1;
     const int64_t tiles = (N + BN - 1) / BN;
     const int64_t ksteps = K / BK;
     int best = 1;
     for (int s = 2; s <= 8; ++s)
-        if (tiles * s <= 512 && ksteps % s == 0 && ksteps / s >= 4) best = s;
-    return tiles * best > 1024 ? 1 : best;
+        if (tiles * s <= 256 && ksteps % s == 0 && ksteps / s >= 4) best = s;
+    return best;
 }
 
 template <bool NESTED, int BM>

@@ -262,14 +262,14 @@ FUSED_GEMM_MIN_N = 28672
 
 def _gemm_splits(M: int, N: int, K: int) -> int:
     """K splits the fused GEMM kernel uses (gemm_splits in csrc/nf4_gemm.hip): up to 128 rows of x,
-    enough workgroups for the chip's 256 CUs when the weight has few 256-row tiles; the k steps divide
-    evenly and every split keeps at least 4."""
+    as many workgroups as fit the chip's 256 CUs in one round when the weight has few 256-row tiles; the
+    k steps divide evenly and every split keeps at least 4."""
     if M > 128:
         return 1
     tiles, ksteps = (N + 255) // 256, K // 64
     best = 1
     for s in range(2, 9):
-        if tiles * s <= 512 and ksteps % s == 0 and ksteps // s >= 4:
+        if tiles * s <= 256 and ksteps % s == 0 and ksteps // s >= 4:
             best = s
     return best
 
@@ -278,15 +278,15 @@ def _fused_gemm_us(M: int, N: int, K: int) -> float:
     """Model of the fused GEMM kernel's time for up to 128 rows of x (one tile of x rows): tiles of
     256 weight rows x K splits run in rounds of 256 workgroups (one per CU), K / 64 / splits steps
     each; a step takes 0.6 us (64-row tile, M <= 64) or 0.8 us (128-row tile) on a sparsely filled chip
-    and 0.35 / 0.5 us more on a full one; merging the splits adds 13 / 25 us, a launch 3 (measured,
-    M = 64 / 128: [4096, 4096] 21 / 34, [6144, 4096] 22 / 36, [4096, 14336] 35 / 52, [8192, 8192] 30 / 47,
-    [14336, 4096] 34 / 51, [28672, 4096] 42 / 60, lm_head [128256, 4096] 121 / 167 us)."""
+    and 0.35 / 0.5 us more on a full one; merging the splits adds 9 / 16 us, a launch 3 (measured,
+    M = 64 / 128: [4096, 4096] 19 / 30, [6144, 4096] 20 / 30, [4096, 14336] 31 / 45, [14336, 4096] 26 / 35,
+    [16384, 8192] 40 / 56, [28672, 4096] 37 / 52, lm_head [128256, 4096] 121 / 167 us)."""
     splits = _gemm_splits(M, N, K)
     wgs = (N + 255) // 256 * splits
     rounds = (wgs + 255) // 256
     fill = min(1.0, wgs / rounds / 256.0)
     step = 0.6 + 0.35 * fill if M <= 64 else 0.8 + 0.5 * fill
-    merge = 0.0 if splits == 1 else 13.0 if M <= 64 else 25.0
+    merge = 0.0 if splits == 1 else 9.0 if M <= 64 else 16.0
     return 3.0 + rounds * (K // 64 // splits) * step + merge
 
 
@@ -300,8 +300,8 @@ def _dense_route_us(N: int, K: int) -> float:
 def _fused_gemm_wins(M: int, N: int, K: int) -> bool:
     """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Up to 128 rows of x the two
     models above decide (the fused kernel's time hardly depends on N while the chip is not full, the
-    dense route's grows with the weight: [14336, 4096] M = 64 44 vs 56 us, [6144, 4096] 41 vs 41,
-    [4096, 14336] 140 vs 66).  Beyond that, measured on MI355X (us, fused vs dense): for tall weights
+    dense route's grows with the weight: M = 64, [4096, 4096] 19 vs 34 us, [14336, 4096] 26 vs 55,
+    [4096, 14336] 31 vs 64, [28672, 4096] 37 vs 107).  Beyond that, measured on MI355X (us, fused vs dense): for tall weights
     and a few hundred rows of x the fused kernel saves more by not writing the bf16 weight than it
     loses to the library GEMM -- [28672, 4096]: 125 vs 153 (512), 230 vs 198 (640); [28672, 8192] M = 512:
     239 vs 294; [57344, 8192]: 477 vs 585 (512), 716 vs 761 (768), 954 vs 932 (1024); lm_head

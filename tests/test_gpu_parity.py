@@ -283,7 +283,7 @@ def fused_gemm(ta, monkeypatch):
     monkeypatch.setattr(ta.functional, "_chunked_gemv_wins", lambda M, N, K: False)
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 128, 4096), (512, 1024, 4096), (2048, 4096, 4096)])
+@pytest.mark.parametrize("M,N,K", [(200, 128, 4096), (512, 1024, 4096), (2048, 4096, 4096)])
 def test_dense_route(ta, oracle, M, N, K):
     """Default route for many rows of x: nf4hip_dequantize + dense GEMM."""
     _sync_print(f"dequant+gemm M={M} N={N} K={K}")
@@ -503,8 +503,9 @@ def test_gemv_every_m_on_large_weights(ta, N, K):
 def test_gemv_chunks_route(ta, nested):
     """17..32 rows of x on a large weight go through the decode kernel 16 rows at a time: a full and
     a ragged last chunk, with bias, against a float64-accumulated matmul over sampled rows of the
-    HIP-dequantized weight."""
-    N, K = 28672, 8192
+    HIP-dequantized weight.  (A short, very wide weight: everywhere else one launch of the fused GEMM
+    is faster than two passes.)"""
+    N, K = 2048, 20480
     _sync_print(f"gemv-chunks nested={nested}")
     g = torch.Generator(device=DEV).manual_seed(99)
     w = (torch.randn(N, K, generator=g, device=DEV) * 0.02).to(torch.bfloat16)

@@ -326,7 +326,7 @@ def codec_section(torch, ta) -> dict:
 def llama_decode(torch, ta, n_new: int) -> dict:
     """BASELINE config 4, outside the timed region of the GEMV metric: the full Llama-3-8B
     architecture with random-init weights, every nn.Linear NF4-quantized through the transform,
-    greedy decode from random prompts of length 512 at batch 1 and 8, decode step replayed from a
+    greedy decode from random prompts of length 512 at batch 1 and 8 (and 32), decode step replayed from a
     HIP graph, Q/K/V and gate/up as one linear each."""
     D = importlib.import_module("lightning-thunder_amd.decode")
     dev = torch.device("cuda:0")
@@ -342,7 +342,7 @@ def llama_decode(torch, ta, n_new: int) -> dict:
         "linear_weight_bytes_per_token": int(nweights * 0.5625),
         "hbm_bound_tok_per_s_batch1": round(HBM_PEAK_GBS * 1e9 / (nweights * 0.5625), 1),
     }
-    for B in (1, 8):
+    for B in (1, 8, 32):  # 32 is not a BASELINE case: the linears of its step run through nf4hip_gemm (M = 32)
         g = torch.Generator(device=dev).manual_seed(4000 + B)
         prompt = torch.randint(0, cfg.vocab, (B, 512), generator=g, device=dev)
         D.greedy_decode(jm, cfg, prompt, n_new=1, use_graph=False)  # untimed: library start-up, GEMM heuristics
@@ -350,6 +350,8 @@ def llama_decode(torch, ta, n_new: int) -> dict:
         # the single-token step with the HIP glue kernels (norm, rotary + cache + attention, SiLU * up)
         # around the NF4 linears, and with plain PyTorch ops in their place
         for key, glue in (("", True), ("_torch_glue", False)):
+            if B > 8 and not glue:
+                continue
             cfg.hip_glue = glue
             _, st = D.greedy_decode(jm, cfg, prompt, n_new=n_new, use_graph=True)
             res[f"decode_tok_per_s{key}"] = round(st["decode_tok_per_s"], 1)

@@ -270,11 +270,15 @@ __global__ __launch_bounds__(ATTN_THREADS) void attention_decode_kernel(const ui
         __hip_atomic_store(mine, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(mine + 1, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    // compiler: no store sinks below the release fence, no load rises above the acquire fence;
+    // hardware: the s_waitcnt holds the wave until L2 has acknowledged its stores
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (tid == 0)
         red[0] = __uint_as_float(__hip_atomic_fetch_add(&counters[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (__float_as_uint(red[0]) != (uint32_t)(splits - 1)) return;
     if (tid < HD) {
         const float* all = partials + bh * splits * (HD + 2);

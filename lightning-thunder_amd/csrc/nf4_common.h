@@ -42,6 +42,9 @@ hipError_t launch_dq_compress(const float* absmax, int64_t nblocks, int nested_l
                               float offset, uint8_t* q, float* absmax2, hipStream_t stream);
 hipError_t launch_dq_reconstruct(const NestedAbsmax& nested, int64_t nblocks, float* absmax, hipStream_t stream);
 
+// Head of every matmul workspace: the split-K arrival counters (zero between calls).
+constexpr size_t GEMV_COUNTER_REGION_BYTES = 65536 * 4;
+
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
@@ -85,6 +88,26 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// Hand-off of split-K partial sums between workgroups: the producer stores its partials with
+// agent-scope relaxed atomic stores (write-through to L2, the level all CUs of the device share),
+// calls publish_partials(), then counts its arrival with an agent-scope relaxed RMW; the last arriver
+// calls acquire_partials() and reads every producer's partials with agent-scope relaxed atomic loads
+// (which bypass its CU's L1).
+//   * For the compiler the two fences are ordering points: no store may sink below the release
+//     fence, no load may be hoisted above the acquire fence, and neither may be moved across the
+//     counter RMW between them.
+//   * For the hardware the release fence at workgroup scope costs nothing on this target (a CU keeps
+//     a workgroup's vector memory operations in order), so the explicit s_waitcnt(0) behind it is
+//     what makes the wave wait until L2 has acknowledged every store before the arrival is counted.
+//   * An agent-scope fence would also be correct, but it writes back and invalidates the whole L2
+//     (measured at 45 us per launch); nothing here needs that, because every access to the shared
+//     data is itself an agent-scope atomic.
+__device__ __forceinline__ void publish_partials() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+}
+__device__ __forceinline__ void acquire_partials() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
 // Reconstruct one absmax value from its nested form: (map * absmax2) + offset, two roundings.
 __device__ __forceinline__ float nested_absmax(const NestedAbsmax& nq, int64_t block) {

@@ -280,11 +280,12 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(MatmulArgs a, int m_tiles
 #pragma unroll
             for (int q = 0; q < 16; ++q)
                 __hip_atomic_store(mine + (i * 16 + q) * THREADS + tid, acc[i][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_s_waitcnt(0);
+        publish_partials();
         __syncthreads();
         uint32_t* flag = reinterpret_cast<uint32_t*>(smem);
         if (tid == 0) *flag = __hip_atomic_fetch_add(&counters[id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
+        acquire_partials();
         if (*flag != (uint32_t)(splits - 1)) return;
         // G splits' worth of loads are issued before the first add, so the merge costs a few memory
         // round trips instead of one per split

@@ -8,7 +8,7 @@ namespace nf4 {
 constexpr int GEMV_THREADS = 512;  // 8 waves; two workgroups per CU
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_TABLE_BYTES = 256 * 256;     // 256 byte values x 64 lanes x 4 B
-constexpr int GEMV_COUNTER_BYTES = 65536 * 4;   // split-K arrival counters at the head of the workspace
+constexpr int GEMV_COUNTER_BYTES = (int)GEMV_COUNTER_REGION_BYTES;  // split-K arrival counters at the head of the workspace
 
 // Byte -> (bf16, bf16) table at the start of LDS.  Entry b holds the code values of the two
 // nibbles of b as bf16, the high nibble (even element) in the low half.  It is replicated for the

@@ -325,7 +325,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 __hip_atomic_store(&partial[((int64_t)ks * M + m) * a.N + r_begin + r], sum, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             }
-            __builtin_amdgcn_s_waitcnt(0);
+            publish_partials();
             __syncthreads();
             if (tid == 0) {
                 const unsigned prev =
@@ -333,6 +333,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 *flag = (prev == (unsigned)p.splits - 1u);
             }
             __syncthreads();
+            acquire_partials();
             if (*flag != 0) {
                 for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
                     const int r = idx / M, m = idx - r * M;

@@ -599,8 +599,9 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                     // Partial sums cross workgroups (and XCDs, whose L2s are not coherent with each
                     // other) through agent-scope relaxed atomics only: such stores write through
                     // and such loads bypass stale lines, so no L2-wide write-back/invalidate is
-                    // needed.  Ordering: every store of the wave has completed (s_waitcnt) before
-                    // the wave bumps the tile's counter; the wave that finds splits - 1 there reduces.
+                    // needed.  Ordering: a tile belongs to ONE wave per K range, so the hand-off is per
+                    // wave: every store of the wave has completed (publish_partials) before the wave bumps
+                    // the tile's counter; the wave that finds splits - 1 there reduces.
                     if (mine) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -610,11 +611,12 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         }
                     }
-                    __builtin_amdgcn_s_waitcnt(0);
+                    publish_partials();
                     unsigned prev = 0;
                     if (lane == 0)
                         prev = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     prev = __builtin_amdgcn_readfirstlane(prev);
+                    acquire_partials();
                     if (prev == (unsigned)p.splits - 1u) {
                         // the lane's R / 4 outputs of the 16 x M tile; the loads of eight slices of all
                         // of them are in flight together, the adds run in slice order

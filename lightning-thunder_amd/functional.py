@@ -19,6 +19,7 @@ from dataclasses import dataclass
 import torch
 
 from . import _lib
+from ._workspace import WorkspacePool
 
 SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
 
@@ -241,18 +242,23 @@ def reconstruct_absmax(nq: NestedAbsmax) -> torch.Tensor:
 # matmul
 # ------------------------------------------------------------------------------------------------
 
-_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+# 40 MiB covers every Llama-3-8B / 70B projection shape on both fused routes (the largest need is the fused
+# GEMM's 33 MB of partial tiles at [16384, 8192], M = 128), so a stream's buffer is normally allocated once.
+_workspace_pool = WorkspacePool(40 << 20, "NF4 matmul")
 
 
 def _gemv_workspace(device: torch.device, nbytes: int, stream: int | None = None) -> torch.Tensor:
-    """Zero-initialised scratch for the gemv kernel, one per (device, stream); the kernel leaves
-    its counters zeroed, so the buffer is reused without clearing."""
-    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream() if stream is None else stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    """Zero-initialised scratch of the split-K kernels for (device, stream); the kernels leave their
+    counters zeroed, so it is reused without clearing.  Raises instead of allocating under capture."""
+    return _workspace_pool.get(device, nbytes, stream)
+
+
+def reserve_workspace(device=None, nbytes: int | None = None) -> int:
+    """Give the current stream of ``device`` its matmul workspace now (for example before capturing a
+    graph on a stream that has not run an NF4 matmul yet).  Returns the buffer's size in bytes."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with _on_device(dev):
+        return _workspace_pool.reserve(dev, nbytes)
 
 
 # The fused GEMM kernel works on tiles of 256 weight rows; from this many rows on a weight has enough

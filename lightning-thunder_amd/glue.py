@@ -29,19 +29,14 @@ SYMBOLS = {
 
 _lib = None
 _lock = threading.Lock()
-_workspaces: dict = {}  # (device index, stream) -> zero-initialised scratch of the attention kernel
+_workspace_pool = WorkspacePool(1 << 20, "decode attention")  # split-key partials and counters
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Zero-initialised scratch, one per (device, stream); the kernel leaves its counters zeroed, so
-    the buffer is reused without clearing."""
-    idx = device.index if device.index is not None else torch.cuda.current_device()
-    key = (idx, _raw_stream(idx) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    """Zero-initialised scratch of the attention kernel for (device, current stream); the kernel leaves
+    its counters zeroed, so the buffer is reused without clearing.  Raises instead of allocating under
+    capture."""
+    return _workspace_pool.get(device, nbytes)
 
 
 def load(path: str | None = None) -> ctypes.CDLL:

@@ -36,7 +36,9 @@ class WorkspacePool:
         self._retired: list[torch.Tensor] = []
 
     def _key(self, device: torch.device, stream: int | None) -> tuple[int, int]:
-        idx = device.index if device.index is not None else torch.cuda.current_device()
+        idx = device.index
+        if idx is None:
+            idx = torch.cuda.current_device() if device.type == "cuda" else -1
         return idx, current_stream_handle(idx) if stream is None else stream
 
     def get(self, device: torch.device, nbytes: int, stream: int | None = None) -> torch.Tensor:

@@ -15,6 +15,8 @@ import threading
 
 import torch
 
+from ._workspace import WorkspacePool
+
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libnf4hip_decode.so")
 
 _vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float

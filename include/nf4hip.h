@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define NF4HIP_ABI_VERSION 1
+#define NF4HIP_ABI_VERSION 2
 
 #define NF4HIP_BF16 0
 #define NF4HIP_F16 1
@@ -112,6 +112,27 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
                    const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
                    const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/*
+ * nf4hip_gemv for callers that cannot allocate or own a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference:
+ * bitsandbytes' gemv_4bit needs no scratch, and the workspace of nf4hip_gemv is this library's own
+ * invention.  Same arguments, rules and results as nf4hip_gemv (fp32 absmax), but the split-K
+ * counters and partial sums live in an array inside the library's device image,
+ * NF4HIP_STATIC_SCRATCH_BYTES per GPU, held from the library's first use on that GPU until the
+ * process ends.  The call allocates and frees nothing, on the device or through any library.
+ *   - A shape whose nf4hip_gemv_workspace_bytes(M,N,K) exceeds NF4HIP_STATIC_SCRATCH_BYTES is refused
+ *     with NF4HIP_E_WORKSPACE (every Llama-3-8B / 70B projection shape fits).
+ *   - All calls on one GPU share that GPU's array: two calls that may overlap in time on the same GPU
+ *     (different streams, or a graph replayed beside eager calls) race.  The array keeps the last
+ *     call's partial sums; the counters at its head are back at zero whenever a call has completed.
+ *   - The first call on a GPU resolves the array's address and clears its counters with a small
+ *     kernel on `stream`; make that call outside a capture.
+ */
+#define NF4HIP_STATIC_SCRATCH_BYTES (4u << 20)
+int nf4hip_gemv_static(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
+                       const float* lut16, const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out,
+                       void* stream);
 
 /*
  * Prefill-shape fused dequant-matmul, M > 16.  Replaces the dequantize_4bit + F.linear route of

@@ -11,9 +11,11 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 BF16, F16, F32 = 0, 1, 2
+
+STATIC_SCRATCH_BYTES = 4 << 20  # NF4HIP_STATIC_SCRATCH_BYTES
 
 E_NULL, E_DTYPE, E_BLOCKSIZE, E_SHAPE, E_ALIGN, E_WORKSPACE, E_HIP = -1, -2, -3, -4, -5, -6, -7
 
@@ -44,6 +46,7 @@ SYMBOLS = {
     "nf4hip_gemv_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "nf4hip_gemv": (_i32, _MATMUL),
     "nf4hip_gemv_dq": (_i32, _MATMUL_DQ),
+    "nf4hip_gemv_static": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp]),
     "nf4hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "nf4hip_gemm": (_i32, _MATMUL),
     "nf4hip_gemm_dq": (_i32, _MATMUL_DQ),

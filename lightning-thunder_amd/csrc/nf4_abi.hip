@@ -3,10 +3,50 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "../../include/nf4hip.h"
 #include "nf4_common.h"
 
+// Scratch of nf4hip_gemv_static: split-K arrival counters and partial sums, in the image of the code
+// object instead of a caller's buffer.  Every device that loads the library holds its own copy at its
+// own address (zero-filled when the code object is loaded); in host code the name below is only a
+// handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) unsigned char scratch[NF4HIP_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each device, once resolved
+
+// zero fill as a kernel (a memset node recorded into a captured graph is not reliable on this target)
+__global__ void fill_zero_kernel(uint4* p, size_t n16) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// Device address of the current device's copy of `scratch`.  The first call on a device resolves it
+// and clears the arrival counters at its head (the kernels leave them at zero after every call, so
+// this only matters if the process wrote there by other means); later calls cost one hipGetDevice.
+hipError_t static_scratch(void** out, hipStream_t stream) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        const size_t n16 = nf4::GEMV_COUNTER_REGION_BYTES / 16;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<uint4*>(p), n16);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return hipSuccess;
+}
 
 thread_local char g_err[512] = "";
 
@@ -52,10 +92,12 @@ int check_nested(const uint8_t* absmax_q, const float* absmax2, const float* map
 
 enum MatmulKind { GEMV, GEMM };
 
+// use_static: the workspace is the library's own `scratch` array (nf4hip_gemv_static)
 int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
                   const nf4::NestedAbsmax* nested, const float* lut16, const void* bias, int64_t N, int64_t K,
-                  int blocksize, void* out, void* workspace, size_t workspace_bytes, void* stream) {
-    const char* name = kind == GEMV ? "nf4hip_gemv" : "nf4hip_gemm";
+                  int blocksize, void* out, void* workspace, size_t workspace_bytes, void* stream,
+                  bool use_static = false) {
+    const char* name = use_static ? "nf4hip_gemv_static" : kind == GEMV ? "nf4hip_gemv" : "nf4hip_gemm";
     if (!x || !packed || !lut16 || !out) return fail(NF4HIP_E_NULL, "%s: null pointer", name);
     if (!nested && !absmax) return fail(NF4HIP_E_NULL, "%s: absmax is null", name);
     if (x_dtype != NF4HIP_BF16)
@@ -81,7 +123,13 @@ int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const 
         (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
         return fail(NF4HIP_E_ALIGN, "%s: pointer not 16-byte aligned", name);
     const size_t need = kind == GEMV ? nf4::gemv_workspace_bytes(M, N, K) : nf4::gemm_workspace_bytes(M, N, K);
-    if (need) {
+    if (use_static) {
+        if (need > (size_t)NF4HIP_STATIC_SCRATCH_BYTES)
+            return fail(NF4HIP_E_WORKSPACE,
+                        "%s: this shape needs %zu bytes of scratch, the built-in array holds %zu (use nf4hip_gemv with a "
+                        "workspace)",
+                        name, need, (size_t)NF4HIP_STATIC_SCRATCH_BYTES);
+    } else if (need) {
         if (!workspace || workspace_bytes < need)
             return fail(NF4HIP_E_WORKSPACE, "%s: workspace of %zu bytes required, got %zu", name, need,
                         workspace ? workspace_bytes : (size_t)0);
@@ -102,6 +150,11 @@ int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const 
     a.block_log2 = bl;
     a.workspace = workspace;
     a.workspace_bytes = workspace_bytes;
+    if (use_static) {
+        const hipError_t es = static_scratch(&a.workspace, static_cast<hipStream_t>(stream));
+        if (es != hipSuccess) return hip_fail(name, es);
+        a.workspace_bytes = NF4HIP_STATIC_SCRATCH_BYTES;
+    }
     const hipError_t e = kind == GEMV ? nf4::launch_gemv(a, static_cast<hipStream_t>(stream))
                                       : nf4::launch_gemm(a, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(name, e);
@@ -204,6 +257,13 @@ int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, co
                 size_t workspace_bytes, void* stream) {
     return matmul_common(GEMV, x, x_dtype, M, packed, absmax, nullptr, lut16, bias_or_null, N, K, blocksize, out,
                          workspace, workspace_bytes, stream);
+}
+
+int nf4hip_gemv_static(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
+                       const float* lut16, const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out,
+                       void* stream) {
+    return matmul_common(GEMV, x, x_dtype, M, packed, absmax, nullptr, lut16, bias_or_null, N, K, blocksize, out,
+                         nullptr, 0, stream, true);
 }
 
 int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(ta):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/nf4hip.h but not exported"
     assert sorted(ta._lib.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
-    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 1
+    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 2
 
 
 def test_missing_library_fails_loudly(ta, tmp_path):
@@ -80,6 +80,14 @@ def test_matmul_argument_errors(ta):
     assert gemv(x=A + 4) == L.E_ALIGN and gemm(packed=A + 1) == L.E_ALIGN and gemv(bias=A + 1) == L.E_ALIGN
     assert gemv(w=None) == L.E_WORKSPACE and gemv(wb=16) == L.E_WORKSPACE
     assert "workspace" in _err(ta)
+    # the entry point that brings its own scratch: same checks, and a shape whose partial sums exceed the
+    # built-in array is refused before any HIP call
+    assert lib.nf4hip_gemv_static(A, L.BF16, 1, A, A, None, None, 64, 4096, 64, A, None) == L.E_NULL
+    assert lib.nf4hip_gemv_static(A, L.BF16, 17, A, A, A, None, 64, 4096, 64, A, None) == L.E_SHAPE
+    assert lib.nf4hip_gemv_static(A, L.BF16, 16, A + 4, A, A, None, 64, 4096, 64, A, None) == L.E_ALIGN
+    assert lib.nf4hip_gemv_workspace_bytes(16, 8192, 1 << 20) > L.STATIC_SCRATCH_BYTES
+    assert lib.nf4hip_gemv_static(A, L.BF16, 16, A, A, A, None, 8192, 1 << 20, 64, A, None) == L.E_WORKSPACE
+    assert "scratch" in _err(ta)
     assert lib.nf4hip_gemv_dq(A, L.BF16, 1, A, None, A, A, 0.0, 256, A, None, 64, 4096, 64, A, A, ws, None) == L.E_NULL
     assert lib.nf4hip_gemm_dq(A, L.BF16, 64, A, A, A, A, 0.0, 7, A, None, 64, 4096, 64, A, None, 0, None) == L.E_BLOCKSIZE
     # workspace sizing is pure arithmetic: split-K arrival counters (65536 x 4 bytes), then partial sums

@@ -388,6 +388,8 @@ hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream) {
     // the smallest tile height that covers x with one tile: the weight tile is expanded once per tile of x rows
     if (a.M <= 64) return a.nested.q ? launch_tile<true, 64>(a, stream) : launch_tile<false, 64>(a, stream);
     if (a.M <= 128) return a.nested.q ? launch_tile<true, 128>(a, stream) : launch_tile<false, 128>(a, stream);
+    // more rows: the kernel of nf4_gemm_wide.hip, whose x loads address x with 32-bit offsets
+    if ((int64_t)a.M * a.K * 2 < ((int64_t)1 << 32)) return launch_gemm_wide(a, stream);
     return a.nested.q ? launch_tile<true, 256>(a, stream) : launch_tile<false, 256>(a, stream);
 }
 

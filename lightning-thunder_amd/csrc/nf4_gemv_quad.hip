@@ -23,7 +23,7 @@
 //    v_perm_b32 and bank-conflict free.
 //  * Scale: a lane's 32 weights share one absmax; the 8-MFMA partial of row i is scaled by the
 //    absmax lane i of the quad loaded (a DPP quad broadcast folded into the FMA).  EXACT variant
-//    (K > 16384): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA, which is
+//    (K > 8192): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA, which is
 //    the reference's dequantisation bit for bit.
 //  * Reduction over the 16 k segments: a transposing butterfly leaves the 16 (row, m) totals of the
 //    group in lanes 0..15; per-(row, wave) sums are parked in LDS and added in a fixed order.

@@ -22,7 +22,7 @@
 //    a lane's 32 weights and leave the VALU with the table addressing only.
 //  * Scale.  The 32 weights of a lane share one quantisation block, so absmax multiplies the lane's
 //    partial sum once.  This differs from the reference's dequantise-then-multiply only in where the
-//    bf16 rounding happens; the difference grows like sqrt(K), so for K > 16384 an exact variant
+//    bf16 rounding happens; the difference grows like sqrt(K), so for K > 8192 an exact variant
 //    rounds every weight as bf16(lut * absmax) before the MFMA (fp32 table, two multiplies and one
 //    convert per byte more).
 //  * Reduction.  Per-lane partial sums of 8 (row, m) pairs are reduced together by a transposing

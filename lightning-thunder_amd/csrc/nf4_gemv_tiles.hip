@@ -306,7 +306,7 @@ __device__ __forceinline__ void prepare_phase(const MatmulArgs& a, PhaseRegs& r,
 }
 
 // MFMA j = 4p + q of the phase covers k [32j, 32j + 32) and uses d[q][p].
-// EXACT (K > 16384): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA -- the
+// EXACT (K > 8192): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA -- the
 // reference's dequantisation bit for bit -- and the MFMAs accumulate straight into acc.
 template <int R, bool EXACT>
 __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uint8_t* xph, int lane, f32x4& acc) {

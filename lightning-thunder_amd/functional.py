@@ -26,12 +26,14 @@ SUPPORTED_BLOCKSIZES = (64, 128, 256, 512, 1024, 2048, 4096)
 # Beyond this K the decode kernels round every weight exactly like the reference's dequantisation
 # (the cheaper "scale the partial sum" arithmetic drifts from it like sqrt(K)); the 5..16-row tile
 # kernel has no such variant, so those calls go to the prefill kernel, which is exact by construction.
-EXACT_K = 16384
-# From this many rows of x on, HIP dequantize followed by the dense library GEMM is the default
-# (the fused GEMM kernel re-expands the weight tile once per 256 rows of x and reaches 0.96-1.05
+EXACT_K = 8192
+# K beyond which a call that no model above claims goes to dequantize + dense GEMM even for a few rows of x
+LONG_K = 16384
+# From this many rows of x on, HIP dequantize followed by the dense library GEMM is a candidate
+# (the fused GEMM kernels re-expand the weight tile once per 256 rows of x and reach 1.0-1.15
 # PFLOP/s, the library GEMM 1.1-1.5 PFLOP/s and the dequantize kernel runs at HBM speed); see
-# _fused_gemm_wins for where the fused kernel is faster all the same.  Raise it to force the
-# fused, allocation-free kernel everywhere.
+# _fused_gemm_wins for which of the two serves a shape.  Raise it to force the fused, allocation-free
+# kernels everywhere.
 DENSE_ROUTE_MIN_M = 17
 
 _DTYPE_CODE = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32}
@@ -261,11 +263,6 @@ def reserve_workspace(device=None, nbytes: int | None = None) -> int:
         return _workspace_pool.reserve(dev, nbytes)
 
 
-# The fused GEMM kernel works on tiles of 256 weight rows; from this many rows on a weight has enough
-# tiles for more than 128 rows of x (tiles of 256 rows of x) to be worth it.
-FUSED_GEMM_MIN_N = 28672
-
-
 def _gemm_splits(M: int, N: int, K: int) -> int:
     """K splits the fused GEMM kernel uses (gemm_splits in csrc/nf4_gemm.hip): up to 128 rows of x,
     as many workgroups as fit the chip's 256 CUs in one round when the weight has few 256-row tiles; the
@@ -303,21 +300,46 @@ def _dense_route_us(N: int, K: int) -> float:
     return 20.0 + 0.62 * N * K / 1e6
 
 
+def _wide_gemm_us(M: int, N: int, K: int) -> float:
+    """Model of the fused GEMM kernel for more than 128 rows of x (csrc/nf4_gemm_wide.hip): tiles of 256 x 256
+    (128 x 256 when the larger tile would leave half the chip without a workgroup) run in rounds of 256
+    workgroups, K / 64 steps each; a step of the 256-row tile takes 1.85 us on a full chip, of the 128-row tile
+    1.0 us, 40 % less on a nearly empty one; 12 us of launch, prologue and epilogue.  Measured / modelled,
+    us: [14336, 4096] M = 256 / 1024 / 2048: 55 / 117 / 232 vs 62 / 124 / 237; [4096, 14336] M = 256 / 1024: 162 / 174 vs 158 /
+    191; [8192, 28672] M = 512: 361 vs 370; lm_head [128256, 4096] M = 1024 / 2048: 978 / 1938 vs 950 / 1890."""
+    n_tiles = (N + 255) // 256
+    bm = 128 if ((M + 255) // 256) * n_tiles <= 128 else 256
+    wgs = ((M + bm - 1) // bm) * n_tiles
+    rounds = (wgs + 255) // 256
+    fill = wgs / (rounds * 256.0)
+    step = (1.85 if bm == 256 else 1.0) * (0.6 + 0.4 * fill)
+    return 12.0 + rounds * (K // 64) * step
+
+
+def _dense_gemm_us(M: int, N: int, K: int) -> float:
+    """Model of the dense route for more than 128 rows of x: the dequantize pass (0.56 us per million
+    weights) plus the library GEMM at the rate it reaches for M rows of x on this part -- 0.8 PFLOP/s at
+    256 rows, 1.15 at 512, 1.38 at 1024, 1.45 at 2048, 1.5 beyond (measured / modelled, us: [14336, 4096] M =
+    256 / 1024 / 2048: 70 / 118 / 198 vs 76 / 125 / 204; lm_head M = 1024 / 2048: 1099 / 1831 vs 1079 / 1783; [4096, 14336]
+    M = 256: 80 vs 75)."""
+    rate = 0.8 if M <= 256 else 1.15 if M <= 512 else 1.38 if M <= 1024 else 1.45 if M <= 2048 else 1.5
+    return 5.0 + 0.56 * N * K / 1e6 + 2.0 * M * N * K / (rate * 1e9)
+
+
 def _fused_gemm_wins(M: int, N: int, K: int) -> bool:
-    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Up to 128 rows of x the two
-    models above decide (the fused kernel's time hardly depends on N while the chip is not full, the
-    dense route's grows with the weight: M = 64, [4096, 4096] 19 vs 34 us, [14336, 4096] 26 vs 55,
-    [4096, 14336] 31 vs 64, [28672, 4096] 37 vs 107).  Beyond that, measured on MI355X (us, fused vs dense): for tall weights
-    and a few hundred rows of x the fused kernel saves more by not writing the bf16 weight than it
-    loses to the library GEMM -- [28672, 4096]: 125 vs 153 (512), 230 vs 198 (640); [28672, 8192] M = 512:
-    239 vs 294; [57344, 8192]: 477 vs 585 (512), 716 vs 761 (768), 954 vs 932 (1024); lm_head
-    [128256, 4096]: 274 vs 533 (256), 535 vs 738 (512), 1038 vs 1109 (1024).  Shorter weights leave
-    most CUs without a tile ([14336, 4096]: 96 vs 77 at M = 256)."""
+    """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Both sides are modelled from
+    measurements on MI355X.  Up to 128 rows of x (one tile of x rows, K split over workgroups) the fused kernel's
+    time hardly depends on N while the chip is not full, the dense route's grows with the weight (M = 64, us:
+    [4096, 4096] 19 vs 34, [14336, 4096] 26 vs 55, [4096, 14336] 31 vs 64, [28672, 4096] 37 vs 107).  Beyond that the fused kernel
+    runs at 1.0-1.15 PFLOP/s, the library GEMM at up to 1.5, but the dense route first writes the bf16 weight: the
+    two cross near 1024 rows of x wherever the fused kernel has a workgroup for most CUs (fused vs dense, us, M =
+    512 / 1024 / 2048: [14336, 4096] 71 / 117 / 232 vs 84 / 118 / 198; [28672, 4096] 127 / 239 / 473 vs 155 / 238 / 405; [28672, 8192] 226 /
+    442 / 881 vs 291 / 466 / 789; lm_head [128256, 4096] 497 / 978 / 1938 vs 741 / 1099 / 1831; short weights leave the chip
+    empty: [4096, 14336] 164 / 174 / 255 vs 107 / 142 / 216, [4096, 4096] 54 / 58 / 79 vs 42 / 52 / 75).  A tie goes to the fused kernel,
+    which needs no transient bf16 weight."""
     if M <= 128:
         return _fused_gemm_us(M, N, K) < _dense_route_us(N, K)
-    if N < FUSED_GEMM_MIN_N:
-        return False
-    return M <= (512 if N < 2 * FUSED_GEMM_MIN_N else 768 if N < 4 * FUSED_GEMM_MIN_N else 1024)
+    return _wide_gemm_us(M, N, K) <= 1.03 * _dense_gemm_us(M, N, K)
 
 
 def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
@@ -371,9 +393,9 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
     if _fused_gemm_wins(M, N, K):
         return "gemm"  # expanding the weight tiles in registers beats writing the bf16 weight out
-    # the fused GEMM kernel streams K sequentially per tile: beyond EXACT_K even a few rows of x are
+    # the fused GEMM kernel streams K sequentially per tile: beyond LONG_K even a few rows of x are
     # served faster by dequantize + dense GEMM
-    return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M or K > EXACT_K else "gemm"
+    return "dequant+gemm" if M >= DENSE_ROUTE_MIN_M or K > LONG_K else "gemm"
 
 
 def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> torch.Tensor:

@@ -81,3 +81,70 @@ def test_quantized_decode_graph_equals_eager(D, ta, fused, batch):
     a = jm(prompt, pos, kc, vc).float()
     b = ref(prompt, pos, kr, vr).float()
     torch.testing.assert_close(a, b, rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.gpu
+def test_llama3_8b_full_size_decode(D, ta):
+    """The benchmark's model at full size: 32 layers, d = 4096, 32 / 8 heads, FFN 14336, vocab 128256, every
+    linear NF4-quantized through the transform, prompts of 512 random token ids, batch 1 and 8.  The HIP-graph
+    replay of the decode step must give the tokens of the eager loop, token for token.
+
+    Logits (prefill, then one decode step on the caches the prefill wrote) are judged against the SAME model in
+    fp32 -- dequantized weights, fp32 activations, plain PyTorch -- next to a plain PyTorch bf16 model on the same
+    weights: through 32 layers two correct bf16 evaluations differ from each other by accumulated roundings
+    (measured: 0.09 rms on logits of rms 1.3, for PyTorch's bf16 path as for this one), so the quantized path is
+    required to be as close to the fp32 result as PyTorch's own bf16 path is: rms and maximum error within 1.5 x,
+    cosine similarity of the logit rows no more than 1e-3 below PyTorch's.
+    """
+    print("llama-3-8b full size", flush=True)
+    dev = torch.device("cuda:0")
+    cfg = D.LlamaConfig.llama3_8b(fused_projections=True, hip_glue=True)
+    model = D.build_llama(cfg, device=dev, seed=4000)
+    jm = ta.jit(model, transforms=[ta.BitsAndBytesLinearQuant4bit()])
+    n_linear = sum(1 for k in jm.state_dict() if k.endswith(".absmax"))
+    assert n_linear == 32 * 4 + 1  # fused qkv, o, fused gate/up, down per layer, and the lm_head
+
+    # references: same architecture and seed, weights replaced by their NF4 round trip, plain PyTorch ops
+    ref_cfg = D.LlamaConfig.llama3_8b(fused_projections=True, hip_glue=False)
+    ref = D.build_llama(ref_cfg, device=dev, seed=4000)
+    for name, mod in ref.named_modules():
+        if isinstance(mod, torch.nn.Linear):
+            qw, absmax, code = ta.quantize_nf4(mod.weight.data)
+            mod.weight.data = ta.dequantize_nf4(qw, absmax, code, 64, torch.bfloat16, tuple(mod.weight.shape))
+    ref32 = D.build_llama(ref_cfg, device=dev, seed=4000)
+    ref32.load_state_dict(ref.state_dict())
+    ref32 = ref32.float()
+
+    def judge(a, b, c, what):
+        a, b, c = a.float(), b.float(), c.float()
+        ea, eb = a - c, b - c
+        rms_a, rms_b = float(ea.pow(2).mean().sqrt()), float(eb.pow(2).mean().sqrt())
+        max_a, max_b = float(ea.abs().max()), float(eb.abs().max())
+        cos = float(torch.nn.functional.cosine_similarity(a.flatten(0, -2), c.flatten(0, -2), dim=-1).min())
+        cos_b = float(torch.nn.functional.cosine_similarity(b.flatten(0, -2), c.flatten(0, -2), dim=-1).min())
+        print(f"  {what}: logits rms {float(c.pow(2).mean().sqrt()):.3f}; error vs fp32: HIP path rms {rms_a:.4f} max {max_a:.3f}, "
+              f"PyTorch bf16 rms {rms_b:.4f} max {max_b:.3f}; cosine {cos:.5f} / {cos_b:.5f}", flush=True)
+        assert cos >= 0.99 and cos >= cos_b - 1e-3, f"{what}: cosine similarity {cos:.5f} vs PyTorch bf16 {cos_b:.5f}"
+        assert rms_a <= 1.5 * rms_b + 1e-3, f"{what}: rms error {rms_a:.4f} vs PyTorch bf16 {rms_b:.4f}"
+        assert max_a <= 1.5 * max_b + 1e-2, f"{what}: max error {max_a:.4f} vs PyTorch bf16 {max_b:.4f}"
+
+    g = torch.Generator().manual_seed(4001)
+    for batch in (1, 8):
+        print(f"  batch {batch}", flush=True)
+        prompt = torch.randint(0, cfg.vocab, (batch, 512), generator=g).to(dev)
+        eager, s0 = D.greedy_decode(jm, cfg, prompt, n_new=8, use_graph=False)
+        graph, s1 = D.greedy_decode(jm, cfg, prompt, n_new=8, use_graph=True)
+        assert s1["graph"] and not s0["graph"]
+        assert torch.equal(eager, graph), "graph replay and eager decode disagree"
+        assert int(eager.min()) >= 0 and int(eager.max()) < cfg.vocab
+        kc, vc = D.new_caches(cfg, batch, dev)
+        kr, vr = D.new_caches(cfg, batch, dev)
+        k32, v32 = D.new_caches(cfg, batch, dev, torch.float32)
+        pos = torch.arange(512, device=dev)
+        a = jm(prompt, pos, kc, vc)
+        b = ref(prompt, pos, kr, vr)
+        c = ref32(prompt, pos, k32, v32)
+        judge(a, b, c, f"prefill, batch {batch}")
+        tok = c.argmax(-1, keepdim=True)
+        pos1 = torch.full((1,), 512, device=dev, dtype=torch.long)
+        judge(jm(tok, pos1, kc, vc), ref(tok, pos1, kr, vr), ref32(tok, pos1, k32, v32), f"decode step, batch {batch}")

@@ -305,10 +305,10 @@ def test_gemm_shapes(ta, oracle, M, N, K, fused_gemm):
     (20, 28672, 512, {}), (49, 28672, 512, {}), (64, 28700, 576, {"nested": True}), (128, 28700, 576, {"bias": True}), (129, 28672, 640, {"nested": True}),
     (300, 28930, 512, {"blocksize": 256}), (512, 28672, 1024, {}), (700, 4 * 28672, 128, {"bias": True}),
 ])
-def test_gemm_route_tall_weights(ta, oracle, M, N, K, kw):
-    """The default router sends tall weights with up to a few hundred rows of x to the fused GEMM
-    kernel (both tile heights, ragged M and N, odd and even numbers of k steps)."""
-    _sync_print(f"gemm (router) M={M} N={N} K={K} {kw}")
+def test_gemm_route_tall_weights(ta, oracle, M, N, K, kw, fused_gemm):
+    """Tall weights through the fused GEMM kernels (all tile heights, ragged M and N, odd and even numbers
+    of k steps, fewer k steps than pipeline stages); up to 128 rows of x the default router picks them itself."""
+    _sync_print(f"gemm (tall) M={M} N={N} K={K} {kw}")
     assert ta.functional.fused_route(torch.empty(M, K, dtype=torch.bfloat16), None, kw.get("blocksize", 64), torch.bfloat16, (N, K)) == "gemm"
     _matmul_case(ta, oracle, M, N, K, seed=M + K, **kw)
 

@@ -45,7 +45,7 @@ typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef const __attribute__((address_space(1))) void* global_void_ptr;
 
-constexpr int BK = 64;
+[[maybe_unused]] constexpr int BK = 64;
 constexpr int BN = 256;
 constexpr int BOOK_BYTES = 256 * 256;  // byte -> (fp32, fp32) of its two codes, 32 copies: 256 B per byte value
 constexpr int CHUNK_BYTES = 1024;      // eight 128-byte rows of x

@@ -9,8 +9,6 @@ the generated computation reaches the kernel.  There is no tracing compiler behi
 
 from __future__ import annotations
 
-import itertools
-import os
 from collections.abc import Callable, Hashable, Sequence
 from dataclasses import dataclass, field
 from typing import Any
@@ -141,197 +139,227 @@ class ImplInfo:
 
 
 class Executor:
-    """thunder/extend/__init__.py:53-198.  Executors hash and compare by name."""
+    """An executor owns operator symbols and knows which foreign symbols it can run
+    (interface of thunder/extend/__init__.py:53-198).  Two executors are the same executor when their
+    names are equal: they hash and compare by name."""
 
     def __init__(self, name: Hashable, *, version: Any = None):
-        self._name = name
-        self._version = version
+        self._name, self._version = name, version
         self._implmap: dict[Hashable, ImplInfo] = {}
         self._lookasides: dict[Callable, Symbol] = {}
         self._opmap: dict[str, Symbol] = {}
 
-    name = property(lambda self: self._name)
-    version = property(lambda self: self._version)
-    implmap = property(lambda self: self._implmap)
-    opmap = property(lambda self: self._opmap)
+    @property
+    def name(self) -> Hashable:
+        return self._name
+
+    @property
+    def version(self) -> Any:
+        return self._version
+
+    @property
+    def implmap(self) -> dict:
+        return self._implmap
+
+    @property
+    def opmap(self) -> dict:
+        return self._opmap
 
     def __repr__(self) -> str:
-        return f"{self.__class__.__module__}.{self.__class__.__name__}('{self.name}')"
+        return f"{type(self).__module__}.{type(self).__name__}('{self._name}')"
 
     def __hash__(self) -> int:
-        return hash(self.name)
+        return hash(self._name)
 
     def __eq__(self, other) -> bool:
-        return isinstance(other, Executor) and other.name == self.name
+        return isinstance(other, Executor) and self._name == other._name
+
+    # ---- which bound symbols this executor takes --------------------------------------------------
+    def _accepting_impl(self, bsym: BoundSymbol) -> ImplInfo | None:
+        """The registered implementation for the bound symbol's id whose checker accepts its arguments."""
+        info = self._implmap.get(bsym.sym.id)
+        if info is None:
+            return None
+        if info.checker is not None and not info.checker(*bsym.args, **bsym.kwargs):
+            return None
+        return info
 
     def can_execute(self, bsym: BoundSymbol) -> bool:
-        impl = self.implmap.get(bsym.sym.id)
-        if impl is None:
-            return False
-        return True if impl.checker is None else bool(impl.checker(*bsym.args, **bsym.kwargs))
+        return self._accepting_impl(bsym) is not None
 
     def can_fuse(self, bsym: BoundSymbol) -> bool:
         if self.can_execute(bsym):
             return True
-        return len(bsym.subsymbols) > 0 and all(self.can_fuse(s) for s in bsym.subsymbols)
+        subs = bsym.subsymbols
+        return bool(subs) and all(self.can_fuse(sub) for sub in subs)
 
     def can_execute_or_fuse(self, bsym: BoundSymbol) -> bool:
-        return self.can_execute(bsym) or self.can_fuse(bsym)
+        return self.can_fuse(bsym)  # can_fuse already covers direct execution
 
     def get_execution_transform(self, bsym: BoundSymbol):
-        impl = self.implmap.get(bsym.sym.id)
-        if impl is None or not (impl.checker is None or impl.checker(*bsym.args, **bsym.kwargs)):
-            return None
-        return impl.execution_transform
+        info = self._accepting_impl(bsym)
+        return info.execution_transform if info is not None else None
 
     def get_grad_transform(self, sym: Symbol):
-        impl = self.implmap.get(sym.id)
-        return None if impl is None else impl.grad_transform
+        info = self._implmap.get(sym.id)
+        return info.grad_transform if info is not None else None
 
+    # ---- operators ---------------------------------------------------------------------------------
     def register_operator(self, name: str, *, like: Symbol | None = None, meta: Callable | None = None, tags=None,
                           module=None, fn: Callable | None = None, bind_postprocess: Callable | None = None,
                           replaces=None) -> Symbol:
-        """Create a symbol owned by this executor.  Exactly one of ``like`` / ``meta``; ``fn`` becomes
-        the call context of every bound symbol; ``replaces`` registers look-asides
-        (thunder/extend/__init__.py:146-198)."""
-        ln, mn = like is None, meta is None
-        assert ln ^ mn, (
-            f"Expected one and only one of 'like' and 'meta' to be specified. {'Neither' if ln and mn else 'Both'} were specified."
-        )
-        is_prim = meta is not None
-        if tags is None and like is not None:
-            tags = getattr(like, "tags", None)
-        meta = meta if meta is not None else like
-        call_ctx = None if fn is None else {name: fn}
+        """Create the symbol ``name`` owned by this executor (thunder/extend/__init__.py:146-198).
 
-        def _bind_postprocess(bsym: BoundSymbol) -> None:
-            bsym._call_ctx = call_ctx
+        Give either ``meta`` (the symbol is a primitive with that shape/dtype inference) or ``like`` (it
+        borrows the inference, and by default the tags, of an existing symbol).  ``fn`` is the
+        implementation: every bound symbol carries ``{name: fn}`` as its call context.  ``replaces`` names
+        callables this symbol stands in for (look-asides)."""
+        given = [k for k, v in (("like", like), ("meta", meta)) if v is not None]
+        assert len(given) == 1, (
+            f"register_operator({name!r}): pass exactly one of `like` and `meta` -- "
+            f"{'neither was' if not given else 'both were'} given"
+        )
+        infer = meta if meta is not None else like
+        if like is not None and tags is None:
+            tags = getattr(like, "tags", None)
+        ctx = {name: fn} if fn is not None else None
+
+        def on_bind(bsym: BoundSymbol) -> None:
+            bsym._call_ctx = ctx
             if bind_postprocess is not None:
                 bind_postprocess(bsym)
 
-        sym = Symbol(name, meta, id=name, is_prim=is_prim, executor=self, tags=tags,
-                     _bind_postprocess=_bind_postprocess, _module=module)
-        self.opmap[name] = sym
-        if callable(replaces):
-            replaces = (replaces,)
-        self._lookasides.update({r: sym for r in replaces or ()})
+        sym = Symbol(name, infer, id=name, is_prim=meta is not None, executor=self, tags=tags, _bind_postprocess=on_bind,
+                     _module=module)
+        self._opmap[name] = sym
+        if replaces is not None:
+            for target in (replaces,) if callable(replaces) else tuple(replaces):
+                self._lookasides[target] = sym
         return sym
 
 
 class OperatorExecutor(Executor):
-    """thunder/extend/__init__.py:260-281."""
+    """An executor that runs symbols one by one (thunder/extend/__init__.py:260-281)."""
 
     def register_implementation(self, sym_or_id, op: Symbol | None = None, *, checker=None, execution_transform=None,
                                 grad_transform=None) -> None:
-        if execution_transform is None:
-            assert op is not None
-        _id = sym_or_id.id if isinstance(sym_or_id, Symbol) else sym_or_id
-        self.implmap[_id] = ImplInfo(op, checker, execution_transform, grad_transform)
+        """Claim a symbol (given as such or by id): run it with ``op``, or rewrite it with
+        ``execution_transform``; ``checker(*args)`` may decline individual calls."""
+        assert op is not None or execution_transform is not None, "register_implementation needs `op` or `execution_transform`"
+        key = sym_or_id.id if isinstance(sym_or_id, Symbol) else sym_or_id
+        self._implmap[key] = ImplInfo(op, checker, execution_transform, grad_transform)
 
 
 # ------------------------------------------------------------------------------------------------
-# registries (thunder/extend/__init__.py:518-651)
+# registries (interface of thunder/extend/__init__.py:518-651)
 # ------------------------------------------------------------------------------------------------
 
-_executor_map: dict[Hashable, Executor] = {}
-_default_executors: list[Executor] = []
-_always_executors: list[Executor] = []
+
+class _Registry:
+    """All registered executors by name, plus the two ordered preference lists.  The most recently added
+    default / always executor comes first."""
+
+    def __init__(self):
+        self.by_name: dict[Hashable, Executor] = {}
+        self.defaults: list[Executor] = []
+        self.always: list[Executor] = []
+
+    @staticmethod
+    def key(ex_or_name) -> Hashable:
+        return ex_or_name.name if isinstance(ex_or_name, Executor) else ex_or_name
+
+    def prepend(self, which: str, ex: Executor) -> list[Executor]:
+        setattr(self, which, [ex, *getattr(self, which)])
+        return getattr(self, which)
+
+    def drop(self, which: str, ex_or_name) -> list[Executor]:
+        k = self.key(ex_or_name)
+        setattr(self, which, [e for e in getattr(self, which) if e.name != k])
+        return getattr(self, which)
+
+
+_registry = _Registry()
 
 
 def register_executor(ex: Executor) -> Executor:
-    _executor_map[ex.name] = ex
+    _registry.by_name[ex.name] = ex
     return ex
 
 
 def deregister_executor(ex) -> None:
-    _id = ex.name if isinstance(ex, Executor) else ex
-    _executor_map.pop(_id, None)
-    remove_always_executor(_id)
-    remove_default_executor(_id)
+    _registry.by_name.pop(_registry.key(ex), None)
+    _registry.drop("always", ex)
+    _registry.drop("defaults", ex)
 
 
 def get_all_executors() -> tuple[Executor, ...]:
-    return tuple(_executor_map.values())
+    return tuple(_registry.by_name.values())
 
 
 def get_executor(name) -> Executor | None:
-    return _executor_map.get(name)
+    return _registry.by_name.get(name)
 
 
 def get_default_executors() -> tuple[Executor, ...]:
-    return tuple(_default_executors)
+    return tuple(_registry.defaults)
 
 
 def get_always_executors() -> tuple[Executor, ...]:
-    return tuple(_always_executors)
+    return tuple(_registry.always)
 
 
 def add_default_executor(ex: Executor) -> list[Executor]:
-    global _default_executors
-    _default_executors = [ex] + _default_executors
-    return _default_executors
+    return _registry.prepend("defaults", ex)
 
 
 def add_always_executor(ex: Executor) -> list[Executor]:
-    global _always_executors
-    _always_executors = [ex] + _always_executors
-    return _always_executors
+    return _registry.prepend("always", ex)
 
 
 def remove_default_executor(ex) -> list[Executor]:
-    global _default_executors
-    _id = ex.name if isinstance(ex, Executor) else ex
-    _default_executors = [x for x in _default_executors if x.name != _id]
-    return _default_executors
+    return _registry.drop("defaults", ex)
 
 
 def remove_always_executor(ex) -> list[Executor]:
-    global _always_executors
-    _id = ex.name if isinstance(ex, Executor) else ex
-    _always_executors = [x for x in _always_executors if x.name != _id]
-    return _always_executors
+    return _registry.drop("always", ex)
 
 
 def resolve_executors(executors: Sequence[Executor | str] | None) -> tuple[Executor, ...]:
-    """Instances pass through, names are looked up; ``None`` means the defaults.  Unknown names and
-    foreign objects raise ``ValueError`` (thunder/extend/__init__.py:622-651)."""
+    """``None`` -> the default executors; otherwise every entry is an :class:`Executor` (kept) or the name of a
+    registered one (looked up).  Anything else, and any unknown name, is a ``ValueError``
+    (thunder/extend/__init__.py:622-651)."""
     if executors is None:
         return get_default_executors()
-    failed: list[str] = []
-    resolved: list[Executor] = []
-    for e in executors:
-        if isinstance(e, str):
-            ex = get_executor(e)
-            if ex is None:
-                failed.append(e)
-            else:
-                resolved.append(ex)
-        elif not isinstance(e, Executor):
-            raise ValueError(f"An object of type {type(e)} is not a valid Executor. Executor list: {executors}")
+    out: list[Executor] = []
+    unknown: list[str] = []
+    for entry in executors:
+        if isinstance(entry, Executor):
+            out.append(entry)
+        elif isinstance(entry, str):
+            found = get_executor(entry)
+            (out if found is not None else unknown).append(found if found is not None else entry)
         else:
-            resolved.append(e)
-    if failed:
-        raise ValueError(
-            f"Expected an Executor or the name of a registered Executor, instead got: {failed[0] if len(failed) == 1 else failed}"
-            + os.linesep + f"Registered executors: {get_all_executors()}"
-        )
-    return tuple(resolved)
+            raise ValueError(f"executors={executors!r}: {entry!r} ({type(entry).__name__}) is neither an Executor nor the name of one")
+    if unknown:
+        known = ", ".join(repr(e.name) for e in get_all_executors())
+        raise ValueError(f"no executor registered under {', '.join(map(repr, unknown))}; registered: {known or 'none'}")
+    return tuple(out)
 
 
 def add_executor_lists(exc_list, other_exc_list) -> list[Executor]:
-    out: list[Executor] = []
-    for exc in itertools.chain(resolve_executors(exc_list), resolve_executors(other_exc_list)):
-        if exc not in out:
-            out.append(exc)
-    return out
+    """Concatenation of the two (resolved) lists without repeats, first occurrence wins."""
+    merged: dict[Executor, None] = {}
+    for ex in (*resolve_executors(exc_list), *resolve_executors(other_exc_list)):
+        merged.setdefault(ex, None)
+    return list(merged)
 
 
 def single_op_executor(exc_name, op_name: str, fn: Callable, meta: Callable, *, version=None, replaces=None, tags=None,
                        checker=None, execution_transform=None, grad_transform=None) -> OperatorExecutor:
-    """One executor with one operator implemented by ``fn`` (thunder/extend/__init__.py:459-514)."""
-    exc = OperatorExecutor(exc_name, version=version)
-    register_executor(exc)
-    sym = exc.register_operator(op_name, fn=fn, replaces=fn if replaces is None else replaces, meta=meta, tags=tags)
-    exc.register_implementation(sym, op=sym, checker=checker, execution_transform=execution_transform,
-                                grad_transform=grad_transform)
-    return exc
+    """A registered executor holding one operator implemented by ``fn``, which it also claims for itself
+    (thunder/extend/__init__.py:459-514)."""
+    ex = register_executor(OperatorExecutor(exc_name, version=version))
+    lookaside = fn if replaces is None else replaces
+    sym = ex.register_operator(op_name, meta=meta, fn=fn, tags=tags, replaces=lookaside)
+    ex.register_implementation(sym, op=sym, checker=checker, execution_transform=execution_transform, grad_transform=grad_transform)
+    return ex

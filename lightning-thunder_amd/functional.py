@@ -240,6 +240,56 @@ def reconstruct_absmax(nq: NestedAbsmax) -> torch.Tensor:
     return out
 
 
+# Nested state as plain tensors (what a state dict can hold): absmax_q uint8 [nblocks], nested_absmax fp32
+# [ceil(nblocks / nested_blocksize)], nested_quant_map fp32 [256], nested_offset fp32 [1].  The C ABI takes the
+# offset by value; reading it back from the device costs a synchronisation, so it is read once per tensor and
+# again only after the tensor was written to (torch bumps ``_version`` on every in-place write).
+_offset_cache: dict[int, tuple[int, int, float]] = {}
+
+
+def _offset_value(nested_offset) -> float:
+    if not isinstance(nested_offset, torch.Tensor):
+        return float(nested_offset)
+    key = id(nested_offset)
+    hit = _offset_cache.get(key)
+    if hit is not None and hit[0] == nested_offset.data_ptr() and hit[1] == nested_offset._version:
+        return hit[2]
+    if len(_offset_cache) > 4096:
+        _offset_cache.clear()
+    value = float(nested_offset.reshape(-1)[0].item())
+    _offset_cache[key] = (nested_offset.data_ptr(), nested_offset._version, value)
+    return value
+
+
+def nested_state(absmax_q, nested_absmax, nested_quant_map, nested_offset, nested_blocksize: int = 256) -> NestedAbsmax:
+    return NestedAbsmax(absmax_q, nested_absmax, nested_quant_map, _offset_value(nested_offset), int(nested_blocksize))
+
+
+def quantize_nf4_dq(w: torch.Tensor, blocksize: int = 64, nested_blocksize: int = 256):
+    """NF4 quantisation with double-quantised statistics (bitsandbytes' ``compress_statistics=True``).  Returns
+    ``(qweight, absmax_q, nested_absmax, nested_quant_map, nested_offset, code)``; ``nested_offset`` is a one-element
+    fp32 tensor so that it can live in a state dict."""
+    qw, absmax, code = quantize_nf4(w, blocksize)
+    nq = compress_absmax(absmax, nested_blocksize)
+    offset = torch.tensor([nq.offset], dtype=torch.float32, device=qw.device)
+    _offset_cache[id(offset)] = (offset.data_ptr(), offset._version, float(nq.offset))
+    return qw, nq.q, nq.absmax2, nq.map256, offset, code
+
+
+def dequantize_nf4_dq(qweight, absmax_q, nested_absmax, nested_quant_map, nested_offset, quant_map, blocksize, nested_blocksize,
+                      dtype, shape) -> torch.Tensor:
+    nq = nested_state(absmax_q, nested_absmax, nested_quant_map, nested_offset, nested_blocksize)
+    return dequantize_nf4(qweight, nq, quant_map, blocksize, dtype, shape)
+
+
+def matmul_nf4_dq(x, qweight, bias, absmax_q, nested_absmax, nested_quant_map, nested_offset, quant_map, blocksize,
+                  nested_blocksize, dtype, shape) -> torch.Tensor:
+    """:func:`matmul_nf4` on double-quantised statistics given as tensors: ``absmax`` is replaced by ``(absmax_q,
+    nested_absmax, nested_quant_map, nested_offset)`` and ``nested_blocksize`` follows ``blocksize``."""
+    nq = nested_state(absmax_q, nested_absmax, nested_quant_map, nested_offset, nested_blocksize)
+    return matmul_nf4(x, qweight, bias, nq, quant_map, blocksize, dtype, shape)
+
+
 # ------------------------------------------------------------------------------------------------
 # matmul
 # ------------------------------------------------------------------------------------------------

@@ -1,55 +1,25 @@
-"""``MaterializationTransform``: give a meta-device model real storage AFTER the other transforms
-have run, so that e.g. bf16 weights never exist on the device, only their NF4 form
-(thunder/transforms/materialization.py:15-172)."""
+"""``MaterializationTransform``: give a meta-device model real storage AFTER the other transforms have
+run, so that e.g. bf16 weights never exist on the device -- only their NF4 form does
+(interface of thunder/transforms/materialization.py:15-172).
+
+Order of events in ``transform_module``:
+
+1. every meta parameter / buffer of the wrapped module is tagged with the device it will live on
+   (``_thunder_device``, which earlier transforms and the planner read instead of ``.device``);
+2. every override that is still a meta tensor is replaced by uninitialised storage on that device -- tied
+   names keep sharing one tensor -- and its names are remembered in ``have_materialized``;
+3. the ``init`` strategy fills the storage: from a state dict of the original model, from a state dict of the
+   transformed model, or by running each submodule's own ``reset_parameters``.
+"""
 
 from __future__ import annotations
 
 import copy
 from collections.abc import Callable
-from itertools import chain
 
 import torch
 
 from ..transform_common import Transform
-
-
-def module_init_from_original_module_init(transform: "MaterializationTransform", tm, *, non_persistent_only: bool = False):
-    """Initialise materialised tensors with the wrapped module's own ``reset_parameters``, one
-    submodule at a time, and push the result through the other transforms (so a freshly
-    initialised Linear weight is quantised right away)."""
-    if non_persistent_only:
-        non_persistent = tm._non_persistent_buffers()
-
-        def skip(n):
-            return n not in non_persistent
-    else:
-
-        def skip(n):
-            return False
-
-    shared_names = tm._get_shared_names()
-    processed: set[str] = set()
-    for module_name, _ in tm._model.named_modules():
-        submodule = tm.get_submodule(module_name)
-        own = list(chain(submodule.named_parameters(recurse=False, prefix=module_name),
-                         submodule.named_buffers(recurse=False, prefix=module_name)))
-        if not any((n in transform.have_materialized) and not skip(n) for n, _ in own):
-            continue
-        module_copy = copy.copy(submodule)  # leave the user's module alone
-        module_copy._parameters = module_copy._parameters.copy()
-        module_copy._buffers = module_copy._buffers.copy()
-        module_copy._modules = module_copy._modules.__class__()
-        need_init = not all((shared_names[n] & processed) or skip(n) for n, _ in own)
-        if need_init:
-            module_copy.to_empty(device=transform.device, recurse=False)
-            if not hasattr(module_copy, "reset_parameters"):
-                raise TypeError(
-                    f"Materialization requires that the `{type(submodule).__name__}.reset_parameters` method is implemented."
-                    " This method is used to initialize any children parameters or buffers in this module."
-                )
-            module_copy.reset_parameters()
-        sd = {n: p for n, p in chain(module_copy.named_parameters(recurse=False), module_copy.named_buffers(recurse=False))}
-        tm._transform_and_load_for_submodule(module_name, sd, shared_names, processed)
 
 
 class MaterializationTransform(Transform):
@@ -60,45 +30,96 @@ class MaterializationTransform(Transform):
     def __init__(self, device, *, init: Callable) -> None:
         self.device = torch.device(device)
         self.init = init
+        self.have_materialized: set[str] = set()
+
+    # ---- step 1 and 2 -------------------------------------------------------------------------------
+    def _target_device(self, t: torch.Tensor) -> torch.device:
+        return getattr(t, "_thunder_device", self.device)
+
+    def _materialize_table(self, table, entries, groups) -> None:
+        for name, meta_tensor in entries:
+            if meta_tensor.device.type != "meta" or name in self.have_materialized:
+                continue
+            storage = torch.empty_like(meta_tensor, device=self._target_device(meta_tensor), requires_grad=meta_tensor.requires_grad)
+            if isinstance(meta_tensor, torch.nn.Parameter):
+                storage = torch.nn.Parameter(storage, requires_grad=meta_tensor.requires_grad)
+            for tied in groups[name]:
+                table[tied] = storage
+            self.have_materialized |= groups[name]
 
     def transform_module(self, model) -> None:
-        for p in chain(model._model.parameters(), model._model.buffers()):
-            if p.device.type == "meta" and not hasattr(p, "_thunder_device"):
-                p._thunder_device = self.device
-        shared_names = model._get_shared_names()
-        self.have_materialized: set[str] = set()
-        for n, p in list(model.named_parameters()):
-            if p.device.type == "meta":
-                new = torch.empty_like(p, device=getattr(p, "_thunder_device", self.device))
-                if isinstance(p, torch.nn.Parameter):
-                    new = torch.nn.Parameter(new, requires_grad=p.requires_grad)
-                for n2 in shared_names[n]:
-                    model._overrides_parameters[n2] = new
-                    self.have_materialized.add(n2)
-        for n, b in list(model.named_buffers()):
-            if b.device.type == "meta":
-                new = torch.empty_like(b, device=getattr(b, "_thunder_device", self.device), requires_grad=b.requires_grad)
-                for n2 in shared_names[n]:
-                    model._overrides_buffers[n2] = new
-                    self.have_materialized.add(n2)
+        wrapped = model._model
+        for t in (*wrapped.parameters(), *wrapped.buffers()):
+            if t.device.type == "meta" and not hasattr(t, "_thunder_device"):
+                t._thunder_device = self.device
+        groups = model._get_shared_names()
+        self.have_materialized = set()
+        self._materialize_table(model._overrides_parameters, list(model.named_parameters()), groups)
+        self._materialize_table(model._overrides_buffers, list(model.named_buffers()), groups)
         self.init(self, model)
 
+    # ---- step 3 -------------------------------------------------------------------------------------
+    def _run_module_inits(self, model, *, only_non_persistent: bool) -> None:
+        """Fill materialised tensors with what the owning submodule's ``reset_parameters`` produces, and send
+        the result through the other transforms (a freshly initialised Linear weight is quantised at once).
+        With ``only_non_persistent`` just the buffers that no state dict carries are of interest."""
+        transient = model._non_persistent_buffers() if only_non_persistent else None
+
+        def wanted(name: str) -> bool:
+            return name in self.have_materialized and (transient is None or name in transient)
+
+        groups = model._get_shared_names()
+        done: set[str] = set()
+        for module_name in [n for n, _ in model._model.named_modules()]:
+            submodule = model.get_submodule(module_name)
+            own = [n for n, _ in (*submodule.named_parameters(recurse=False, prefix=module_name),
+                                  *submodule.named_buffers(recurse=False, prefix=module_name))]
+            pending = [n for n in own if wanted(n)]
+            if not pending:
+                continue
+            # a private, childless stand-in for the submodule: the user's module keeps its meta tensors
+            stand_in = copy.copy(submodule)
+            stand_in._parameters = dict(submodule._parameters)
+            stand_in._buffers = dict(submodule._buffers)
+            stand_in._modules = type(submodule._modules)()
+            # nothing to compute if every wanted tensor is tied to one that an earlier submodule initialised
+            if any(not (groups[n] & done) for n in pending):
+                init_fn = getattr(stand_in, "reset_parameters", None)
+                if init_fn is None:
+                    raise TypeError(f"cannot materialise {module_name or 'the root module'!r}: "
+                                    f"{type(submodule).__name__} has no reset_parameters() to initialise its tensors with")
+                stand_in.to_empty(device=self.device, recurse=False)
+                init_fn()
+            fresh = dict(stand_in.named_parameters(recurse=False))
+            fresh.update(stand_in.named_buffers(recurse=False))
+            model._transform_and_load_for_submodule(module_name, fresh, groups, done)
+
     @staticmethod
-    def init_from_original_state_dict(state_dict):
-        def init(transform, model):
-            module_init_from_original_module_init(transform, model, non_persistent_only=True)
+    def init_from_original_state_dict(state_dict) -> Callable:
+        """Weights come from a state dict of the ORIGINAL model (streamed through the other transforms);
+        non-persistent buffers, which no state dict holds, from the modules' own init."""
+
+        def init(transform: "MaterializationTransform", model) -> None:
+            transform._run_module_inits(model, only_non_persistent=True)
             model.load_original_state_dict(state_dict)
 
         return init
 
     @staticmethod
-    def init_from_transformed_state_dict(state_dict):
-        def init(transform, model):
-            module_init_from_original_module_init(transform, model, non_persistent_only=True)
+    def init_from_transformed_state_dict(state_dict) -> Callable:
+        """Weights come from a state dict of the TRANSFORMED model (e.g. packed NF4 tensors), loaded as is."""
+
+        def init(transform: "MaterializationTransform", model) -> None:
+            transform._run_module_inits(model, only_non_persistent=True)
             model.load_state_dict(state_dict)
 
         return init
 
     @staticmethod
-    def init_from_original_module_init():
-        return module_init_from_original_module_init
+    def init_from_original_module_init() -> Callable:
+        """Every materialised tensor is initialised by its submodule's ``reset_parameters``."""
+
+        def init(transform: "MaterializationTransform", model) -> None:
+            transform._run_module_inits(model, only_non_persistent=False)
+
+        return init

@@ -1,9 +1,15 @@
 """``BitsAndBytesLinearQuant4bit`` with the HIP executor behind it.
 
-Mirror of thunder/transforms/quantization.py: same class name, hooks, ``quant_states`` layout,
-override keys (``<w>``, ``<w>.absmax``, ``<w>.code``) and operator signature.  The executor is
-``quant_hip_nf4`` instead of ``quant_bnb`` and its operator ``hip_matmul_nf4`` calls the gfx950
-kernels of libnf4hip.so instead of bitsandbytes.
+Same class name, hooks, ``quant_states`` layout, override keys (``<w>``, ``<w>.absmax``, ``<w>.code``) and
+operator signature as thunder/transforms/quantization.py; the executor is ``quant_hip_nf4`` instead of
+``quant_bnb`` and its operator ``hip_matmul_nf4`` runs the gfx950 kernels of libnf4hip.so instead of
+bitsandbytes.
+
+Beyond the reference (which leaves it as a TODO, thunder/transforms/quantization.py:84):
+``BitsAndBytesLinearQuant4bit(double_quant=True)`` also quantises the per-block absmax to 8 bits
+(bitsandbytes' ``compress_statistics=True``).  ``<w>.absmax`` then holds the uint8 codes and three more
+entries appear next to it -- ``<w>.nested_absmax``, ``<w>.nested_quant_map``, ``<w>.nested_offset`` -- and the
+linears run ``hip_matmul_nf4_dq``, whose arguments are those tensors in place of ``absmax``.
 """
 
 from __future__ import annotations
@@ -29,18 +35,51 @@ hip_nf4_executor: extend.OperatorExecutor | None = None
 hip_matmul_nf4: extend.Symbol | None = None
 hip_quantize_nf4: extend.Symbol | None = None
 hip_dequantize_nf4: extend.Symbol | None = None
+hip_matmul_nf4_dq: extend.Symbol | None = None
+hip_quantize_nf4_dq: extend.Symbol | None = None
+hip_dequantize_nf4_dq: extend.Symbol | None = None
+
+# Device on which weights are quantised.  The reference hard-codes "cuda" (quantization.py:53-63);
+# ROCm builds of torch use the same device name.
+WORK_DEVICE = "cuda"
+
+
+# ---- operators: meta (shape / dtype inference on proxies) and implementation --------------------------
+
+
+def _numel(shape) -> int:
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+def _check_matmul_shapes(x, shape) -> None:
+    assert isinstance(shape, Sequence) and len(shape) == 2
+    assert x.shape[-1] == shape[1], f"{x.shape=}, rhs {shape=}"
 
 
 def hip_matmul_nf4_meta(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape):
     """Shape/dtype inference of the operator (thunder/transforms/quantization.py:29-32)."""
-    assert isinstance(shape, Sequence) and len(shape) == 2
-    assert x.shape[-1] == shape[1], f"{x.shape=}, rhs {shape=}"
+    _check_matmul_shapes(x, shape)
     return TensorProxy(like=x, shape=(*x.shape[:-1], shape[0]))
 
 
 def hip_matmul_nf4_impl(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape):
     """``x @ dequantize(qweight).T + bias`` (thunder/transforms/quantization.py:34-39)."""
     return functional.matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape)
+
+
+def hip_matmul_nf4_dq_meta(x, qweight, bias, absmax_q, nested_absmax, nested_quant_map, nested_offset, quant_map, blocksize,
+                           nested_blocksize, dtype, shape):
+    _check_matmul_shapes(x, shape)
+    return TensorProxy(like=x, shape=(*x.shape[:-1], shape[0]))
+
+
+def hip_matmul_nf4_dq_impl(x, qweight, bias, absmax_q, nested_absmax, nested_quant_map, nested_offset, quant_map, blocksize,
+                           nested_blocksize, dtype, shape):
+    return functional.matmul_nf4_dq(x, qweight, bias, absmax_q, nested_absmax, nested_quant_map, nested_offset, quant_map,
+                                    blocksize, nested_blocksize, dtype, shape)
 
 
 def hip_quantize_nf4_impl(w, blocksize=64):
@@ -51,24 +90,30 @@ def hip_dequantize_nf4_impl(qweight, absmax, quant_map, blocksize, dtype, shape)
     return functional.dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape)
 
 
-# Device on which weights are quantised.  The reference hard-codes "cuda" (quantization.py:53-63);
-# ROCm builds of torch use the same device name.
-WORK_DEVICE = "cuda"
+def _plain(like, shape, dtype) -> TensorProxy:
+    return TensorProxy(like=like, shape=tuple(shape), dtype=dtype, requires_grad=False)
 
 
 def _quantize_meta(w, blocksize=64):
-    n = 1
-    for s in w.shape:
-        n *= s
-    return (
-        TensorProxy(like=w, shape=((n + 1) // 2, 1), dtype=torch.uint8, requires_grad=False),
-        TensorProxy(like=w, shape=((n + blocksize - 1) // blocksize,), dtype=torch.float32, requires_grad=False),
-        TensorProxy(like=w, shape=(16,), dtype=torch.float32, requires_grad=False),
-    )
+    n = _numel(w.shape)
+    return (_plain(w, ((n + 1) // 2, 1), torch.uint8), _plain(w, (-(-n // blocksize),), torch.float32), _plain(w, (16,), torch.float32))
 
 
 def _dequantize_meta(qweight, absmax, quant_map, blocksize, dtype, shape):
-    return TensorProxy(like=qweight, shape=tuple(shape), dtype=dtype, requires_grad=False)
+    return _plain(qweight, shape, dtype)
+
+
+def _quantize_dq_meta(w, blocksize=64, nested_blocksize=256):
+    n = _numel(w.shape)
+    nblocks = -(-n // blocksize)
+    return (_plain(w, ((n + 1) // 2, 1), torch.uint8), _plain(w, (nblocks,), torch.uint8),
+            _plain(w, (-(-nblocks // nested_blocksize),), torch.float32), _plain(w, (256,), torch.float32),
+            _plain(w, (1,), torch.float32), _plain(w, (16,), torch.float32))
+
+
+def _dequantize_dq_meta(qweight, absmax_q, nested_absmax, nested_quant_map, nested_offset, quant_map, blocksize, nested_blocksize,
+                        dtype, shape):
+    return _plain(qweight, shape, dtype)
 
 
 def get_hip_nf4_executor() -> extend.OperatorExecutor:
@@ -76,6 +121,7 @@ def get_hip_nf4_executor() -> extend.OperatorExecutor:
     (thunder/transforms/quantization.py:19-44).  Loading the HIP library is part of it: a missing
     or mismatching ``libnf4hip.so`` fails here, not at the first forward."""
     global hip_nf4_executor, hip_matmul_nf4, hip_quantize_nf4, hip_dequantize_nf4
+    global hip_matmul_nf4_dq, hip_quantize_nf4_dq, hip_dequantize_nf4_dq
     if hip_nf4_executor is None:
         from .. import _lib
 
@@ -84,6 +130,11 @@ def get_hip_nf4_executor() -> extend.OperatorExecutor:
         hip_matmul_nf4 = ex.register_operator("hip_matmul_nf4", meta=hip_matmul_nf4_meta, fn=hip_matmul_nf4_impl)
         hip_quantize_nf4 = ex.register_operator("hip_quantize_nf4", meta=_quantize_meta, fn=hip_quantize_nf4_impl)
         hip_dequantize_nf4 = ex.register_operator("hip_dequantize_nf4", meta=_dequantize_meta, fn=hip_dequantize_nf4_impl)
+        hip_matmul_nf4_dq = ex.register_operator("hip_matmul_nf4_dq", meta=hip_matmul_nf4_dq_meta, fn=hip_matmul_nf4_dq_impl)
+        hip_quantize_nf4_dq = ex.register_operator("hip_quantize_nf4_dq", meta=_quantize_dq_meta,
+                                                   fn=lambda w, blocksize=64, nested_blocksize=256: functional.quantize_nf4_dq(w, blocksize, nested_blocksize))
+        hip_dequantize_nf4_dq = ex.register_operator("hip_dequantize_nf4_dq", meta=_dequantize_dq_meta,
+                                                     fn=lambda *a: functional.dequantize_nf4_dq(*a))
         extend.register_executor(ex)
         hip_nf4_executor = ex
     return hip_nf4_executor
@@ -93,170 +144,222 @@ def get_hip_nf4_executor() -> extend.OperatorExecutor:
 get_bitsandbytes_executor = get_hip_nf4_executor
 
 
+# ---- the transform -------------------------------------------------------------------------------------
+
+# What a quantised weight brings along besides the packed tensor, as suffixes of the weight's name, in the order
+# in which the entries are installed, appear in state dicts and are appended to the computation's inputs.
+_PLAIN_EXTRAS = ("absmax", "code")
+_NESTED_EXTRAS = ("absmax", "code", "nested_absmax", "nested_quant_map", "nested_offset")
+
+
 class BitsAndBytesLinearQuant4bit(Transform):
     """Quantise the weight of every ``nn.Linear`` to NF4 and route its matmul to the HIP operator.
 
     ``BitsAndBytesLinearQuant4bit()`` behaves like the reference (blocksize 64, fp32 absmax).
     ``lut_rounding="dtype"`` stores the code book pre-rounded to the weight dtype, which reproduces
-    bitsandbytes' eager (non-CUDA) dequantisation instead of its CUDA kernel's.
+    bitsandbytes' eager (non-CUDA) dequantisation instead of its CUDA kernel's.  ``double_quant=True`` stores the
+    absmax statistics in 8 bits (nested blocks of ``nested_blocksize``) next to an fp32 offset.
     """
 
-    def __init__(self, *, blocksize: int = 64, lut_rounding: str = "none"):
+    def __init__(self, *, blocksize: int = 64, lut_rounding: str = "none", double_quant: bool = False, nested_blocksize: int = 256):
         assert lut_rounding in ("none", "dtype")
         self.quant_states: dict[str, dict] = {}
         self.quantized_submodule_names: set[str] = set()
         self.blocksize = blocksize
         self.lut_rounding = lut_rounding
+        self.double_quant = bool(double_quant)
+        self.nested_blocksize = nested_blocksize
         get_hip_nf4_executor()
 
-    def quantize_weight(self, w: torch.Tensor):
-        """Device policy of the reference (quantization.py:53-63): meta -> zeros on the GPU, anything
-        not on the GPU is moved there; then the quantise kernel.  Returns (qweight, absmax, code)."""
+    @property
+    def _extras(self) -> tuple[str, ...]:
+        return _NESTED_EXTRAS if self.double_quant else _PLAIN_EXTRAS
+
+    # ---- quantising one weight ---------------------------------------------------------------------
+    @staticmethod
+    def _on_work_device(w: torch.Tensor) -> torch.Tensor:
+        """Device policy of the reference (quantization.py:53-63): a meta weight stands for zeros on the GPU,
+        a weight anywhere else is copied to the GPU, a GPU weight is used where it is."""
         work = torch.device(WORK_DEVICE)
         if w.device.type == "meta":
-            w_work = torch.zeros_like(w, device=work)
-        elif w.device.type != work.type:
-            with torch.no_grad():
-                w_work = w.to(work)
+            return torch.zeros_like(w, device=work)
+        if w.device.type == work.type:
+            return w.detach()
+        with torch.no_grad():
+            return w.to(work).detach()
+
+    def _quantized_tensors(self, w: torch.Tensor) -> dict[str, torch.Tensor]:
+        """suffix -> tensor for one weight: ``""`` is the packed weight, the others are this transform's extras."""
+        src = self._on_work_device(w)
+        if self.double_quant:
+            qw, absmax_q, nested_absmax, nested_map, nested_offset, code = hip_quantize_nf4_dq(src, self.blocksize, self.nested_blocksize)
+            out = {"": qw, "absmax": absmax_q, "code": code, "nested_absmax": nested_absmax, "nested_quant_map": nested_map,
+                   "nested_offset": nested_offset}
         else:
-            w_work = w
-        qw, absmax, code = hip_quantize_nf4(w_work.detach(), self.blocksize)
+            qw, absmax, code = hip_quantize_nf4(src, self.blocksize)
+            out = {"": qw, "absmax": absmax, "code": code}
         if self.lut_rounding == "dtype":
-            code = code.to(w.dtype).to(torch.float32)
-        return qw, absmax, code
+            out["code"] = out["code"].to(w.dtype).to(torch.float32)
+        return out
 
+    def quantize_weight(self, w: torch.Tensor):
+        """``(qweight, absmax, code)`` of ``w`` like the reference's method of the same name; with ``double_quant``
+        ``absmax`` is a :class:`functional.NestedAbsmax`."""
+        t = self._quantized_tensors(w)
+        if not self.double_quant:
+            return t[""], t["absmax"], t["code"]
+        nested = functional.nested_state(t["absmax"], t["nested_absmax"], t["nested_quant_map"], t["nested_offset"], self.nested_blocksize)
+        return t[""], nested, t["code"]
+
+    def _state_record(self, w: torch.Tensor, tensors: dict[str, torch.Tensor]) -> dict:
+        qw = tensors[""]
+        record = {"dtype": w.dtype, "shape": tuple(w.shape), "blocksize": self.blocksize,
+                  "qweight.dtype": qw.dtype, "qweight.shape": tuple(qw.shape)}
+        for suffix in self._extras:
+            record[f"{suffix}.dtype"] = tensors[suffix].dtype
+            record[f"{suffix}.shape"] = tuple(tensors[suffix].shape)
+        record["device"] = getattr(w, "_thunder_device", w.device)
+        if self.double_quant:
+            record["nested_blocksize"] = self.nested_blocksize
+        return record
+
+    # ---- hooks --------------------------------------------------------------------------------------
     def transform_module(self, model) -> None:
+        """Quantise every ``nn.Linear`` weight of the wrapped module, in ``named_modules()`` order, into the
+        wrapper's parameter overrides.  Tied weights are quantised once and keep sharing their tensors."""
         self.thunder_module = model
-        shared_names = model._get_shared_names()
-        processed: set[str] = set()
-
-        def convert_linear_submodule(tm, name: str) -> None:
-            self.quantized_submodule_names.add(name)
-            weight_name = f"{name}.weight" if name else "weight"
-            done_copies = shared_names[weight_name] & processed
-            if done_copies:  # tied weight: share the already quantised tensors
-                copy_name = next(iter(done_copies))
-                self.quant_states[weight_name] = self.quant_states[copy_name]
-                for suffix in ("", ".absmax", ".code"):
-                    tm._overrides_parameters[weight_name + suffix] = tm._overrides_parameters[copy_name + suffix]
-                processed.add(weight_name)
-                return
-            w = tm.get_parameter(weight_name)
-            qw, absmax, code = self.quantize_weight(w)
-            tm._overrides_parameters[weight_name] = qw.to(w.device)
-            tm._overrides_parameters[f"{weight_name}.absmax"] = absmax.to(w.device)
-            tm._overrides_parameters[f"{weight_name}.code"] = code.to(w.device)
-            self.quant_states[weight_name] = {
-                "dtype": w.dtype,
-                "shape": tuple(w.shape),
-                "blocksize": self.blocksize,
-                "qweight.dtype": qw.dtype,
-                "qweight.shape": tuple(qw.shape),
-                "absmax.dtype": absmax.dtype,
-                "absmax.shape": tuple(absmax.shape),
-                "code.dtype": code.dtype,
-                "code.shape": tuple(code.shape),
-                "device": getattr(w, "_thunder_device", w.device),
-            }
-            processed.add(weight_name)
-
-        for n, submodule in model._model.named_modules():
-            if isinstance(submodule, torch.nn.Linear):
-                convert_linear_submodule(model, n)
+        table = model._overrides_parameters
+        tied = model._get_shared_names()
+        for module_name, submodule in model._model.named_modules():
+            if not isinstance(submodule, torch.nn.Linear):
+                continue
+            self.quantized_submodule_names.add(module_name)
+            weight_name = f"{module_name}.weight" if module_name else "weight"
+            twin = next((other for other in sorted(tied[weight_name]) if other != weight_name and other in self.quant_states), None)
+            if twin is not None:
+                self.quant_states[weight_name] = self.quant_states[twin]
+                for suffix in ("", *self._extras):
+                    dot = "." if suffix else ""
+                    table[f"{weight_name}{dot}{suffix}"] = table[f"{twin}{dot}{suffix}"]
+                continue
+            w = model.get_parameter(weight_name)
+            tensors = self._quantized_tensors(w)
+            table[weight_name] = tensors[""].to(w.device)
+            for suffix in self._extras:
+                table[f"{weight_name}.{suffix}"] = tensors[suffix].to(w.device)
+            self.quant_states[weight_name] = self._state_record(w, tensors)
 
     def transform_state_dict_for_submodule(self, model, submodule_name: str, state_dict: dict) -> dict:
-        """Quantise an incoming original weight; keys carry no submodule prefix (quantization.py:108-126)."""
+        """An incoming ORIGINAL weight of a quantised submodule is replaced by its packed form plus extras; keys
+        carry no submodule prefix (quantization.py:108-126)."""
         if submodule_name not in self.quantized_submodule_names:
             return state_dict
-        weight_name_full = f"{submodule_name}.weight" if submodule_name else "weight"
-        qs = self.quant_states[weight_name_full]
+        record = self.quant_states[f"{submodule_name}.weight" if submodule_name else "weight"]
         w = state_dict["weight"]
-        assert w.dtype == qs["dtype"]
-        assert tuple(w.shape) == tuple(qs["shape"])
-        qw, absmax, code = self.quantize_weight(w)
-        state_dict = state_dict.copy()
-        state_dict["weight"] = qw.to(w.device)
-        state_dict["weight.absmax"] = absmax.to(w.device)
-        state_dict["weight.code"] = code.to(w.device)
-        return state_dict
+        assert w.dtype == record["dtype"], f"{submodule_name}.weight: dtype {w.dtype}, quantised as {record['dtype']}"
+        assert tuple(w.shape) == tuple(record["shape"]), f"{submodule_name}.weight: shape {tuple(w.shape)}, quantised as {record['shape']}"
+        tensors = self._quantized_tensors(w)
+        out = dict(state_dict)
+        out["weight"] = tensors[""].to(w.device)
+        for suffix in self._extras:
+            out[f"weight.{suffix}"] = tensors[suffix].to(w.device)
+        return out
 
     def reverse_transform_state_dict_for_submodule(self, model, submodule_name: str, state_dict: dict) -> dict:
         """Dequantise back to the original dtype and shape.  (The reference has no reverse; its
         ``original_state_dict()`` of a quantised module returns the packed tensors.)"""
         if submodule_name not in self.quantized_submodule_names or "weight.absmax" not in state_dict:
             return state_dict
-        qs = self.quant_states[f"{submodule_name}.weight" if submodule_name else "weight"]
-        sd = {k: v for k, v in state_dict.items() if k not in ("weight.absmax", "weight.code")}
-        qw, absmax, code = state_dict["weight"], state_dict["weight.absmax"], state_dict["weight.code"]
-        dev = qw.device
-        w = hip_dequantize_nf4(qw.to(WORK_DEVICE), absmax.to(WORK_DEVICE), code.to(WORK_DEVICE), qs["blocksize"], qs["dtype"], qs["shape"])
-        sd["weight"] = w.to(dev)
-        return sd
+        record = self.quant_states[f"{submodule_name}.weight" if submodule_name else "weight"]
+        extra_keys = {f"weight.{suffix}" for suffix in self._extras}
+        out = {k: v for k, v in state_dict.items() if k not in extra_keys}
+        home = state_dict["weight"].device
+        on_gpu = {k: state_dict[k].to(WORK_DEVICE) for k in ("weight", *sorted(extra_keys))}
+        if self.double_quant:
+            w = hip_dequantize_nf4_dq(on_gpu["weight"], on_gpu["weight.absmax"], on_gpu["weight.nested_absmax"],
+                                      on_gpu["weight.nested_quant_map"], on_gpu["weight.nested_offset"], on_gpu["weight.code"],
+                                      record["blocksize"], record["nested_blocksize"], record["dtype"], record["shape"])
+        else:
+            w = hip_dequantize_nf4(on_gpu["weight"], on_gpu["weight.absmax"], on_gpu["weight.code"], record["blocksize"],
+                                   record["dtype"], record["shape"])
+        out["weight"] = w.to(home)
+        return out
+
+    # ---- the plan of a call -------------------------------------------------------------------------
+    def _operator_call(self, bsym, record: dict, extras: dict[str, TensorProxy]):
+        """``linear(x, w, b)`` on a quantised weight as a call of this executor's operator."""
+        x, w, b = bsym.args
+        if self.double_quant:
+            args = (x, w, b, extras["absmax"], extras["nested_absmax"], extras["nested_quant_map"], extras["nested_offset"],
+                    extras["code"], record["blocksize"], record["nested_blocksize"], record["dtype"], record["shape"])
+            return bsym.from_bsym(sym=hip_matmul_nf4_dq, subsymbols=(), args=args)
+        args = (x, w, b, extras["absmax"], extras["code"], record["blocksize"], record["dtype"], record["shape"])
+        return bsym.from_bsym(sym=hip_matmul_nf4, subsymbols=(), args=args)
 
     def transform_traces_pre_prologue(self, prologue_trace, computation_trace, epilogue_trace, **kwargs):
-        """Rewrite the plan of a call (quantization.py:128-293): the checks of quantised weights expect
-        the packed tensor; absmax and code become extra prologue outputs / computation inputs; every
-        ``linear`` on a quantised weight becomes ``hip_matmul_nf4(x, qweight, bias, absmax, code,
-        blocksize, dtype, shape)``; nothing else changes."""
-        tm = self.thunder_module
+        """Rewrite the plan of a call (what quantization.py:128-293 does to Thunder's traces):
+
+        * the prologue's check of every quantised weight expects the packed tensor (uint8, ``[n/2, 1]``, no grad);
+        * the weight's extras are fetched and checked in the prologue too, become prologue outputs and -- tagged as
+          static memory -- inputs of the computation, after the existing ones;
+        * every ``linear`` on a quantised weight becomes ``hip_matmul_nf4(x, qweight, bias, absmax, code, blocksize,
+          dtype, shape)`` (or its ``_dq`` form); nothing else in the computation changes."""
+        model = self.thunder_module
+        packed_meta = {}
+        for name, (check, unpack) in get_checks(prologue_trace).items():
+            if name in self.quant_states:
+                record = self.quant_states[name]
+                packed_meta[unpack.output.name] = {"shape": record["qweight.shape"], "dtype": record["qweight.dtype"]}
+        prologue_trace = trace_with_replaced_proxy_metadata(prologue_trace, packed_meta)
         checks = get_checks(prologue_trace)
-        prologue_proxy_map = {
-            get_param.output.name: dict(shape=self.quant_states[n]["qweight.shape"], dtype=self.quant_states[n]["qweight.dtype"])
-            for n, (check, get_param) in checks.items()
-            if n in self.quant_states
-        }
-        prologue_trace = trace_with_replaced_proxy_metadata(prologue_trace, prologue_proxy_map)
-        checks = get_checks(prologue_trace)
-        output_idxes = {o.name: i for i, o in enumerate(prologue_trace.output[0])}
+        returned = {proxy.name for proxy in prologue_trace.output[0]}
 
-        quantized_proxies: dict[str, str] = {}  # proxy name -> parameter name
-        additional_proxies: dict[str, TensorProxy] = {}  # parameter name.(absmax|code) -> proxy
-        new_bsyms, new_compute_inputs = [], []
-        for n, qs in self.quant_states.items():
-            for key in (n, f"{n}.absmax", f"{n}.code"):
-                tm.get_parameter(key)  # must exist
-            check, get_param = checks[n]
-            quantized_proxies[get_param.output.name] = n
-            proxy, _, device, _, _ = check.args
-            check.args = (proxy, qs["qweight.shape"], device, qs["qweight.dtype"], False)
-            proxy.requires_grad = False
-            if get_param.output.name not in output_idxes:
-                continue
-            for suffix in ("absmax", "code"):
-                p = TensorProxy(f"{get_param.output.name}_{suffix}", shape=qs[f"{suffix}.shape"], dtype=qs[f"{suffix}.dtype"],
-                                device=device, requires_grad=False, tags={STATIC_MEMORY_LOCATION})
-                new_bsyms.append(get_param.sym.bind(get_param.args[0], f"{n}.{suffix}", output=p))
-                add_trace_output(prologue_trace, p, subindex=0)
-                new_compute_inputs.append(p)
-                new_bsyms.append(check_tensor_shape_and_metadata.bind(p, qs[f"{suffix}.shape"], device, qs[f"{suffix}.dtype"], False, output=None))
-                additional_proxies[f"{n}.{suffix}"] = p
-        prologue_trace.bound_symbols[-1:-1] = new_bsyms
+        weight_of_proxy: dict[str, str] = {}           # proxy of a packed weight -> parameter name
+        extras_of: dict[str, dict[str, TensorProxy]] = {}  # parameter name -> suffix -> proxy
+        fetches, new_inputs = [], []
+        for name, record in self.quant_states.items():
+            for suffix in ("", *self._extras):
+                model.get_parameter(f"{name}.{suffix}" if suffix else name)  # the overrides must be in place
+            check, unpack = checks[name]
+            weight_proxy, _, device, _, _ = check.args
+            check.args = (weight_proxy, record["qweight.shape"], device, record["qweight.dtype"], False)
+            weight_proxy.requires_grad = False
+            weight_of_proxy[unpack.output.name] = name
+            if unpack.output.name not in returned:
+                continue  # the computation never sees this weight
+            owner = unpack.args[0]
+            extras_of[name] = {}
+            for suffix in self._extras:
+                shape, dtype = record[f"{suffix}.shape"], record[f"{suffix}.dtype"]
+                proxy = TensorProxy(f"{unpack.output.name}_{suffix}", shape=shape, dtype=dtype, device=device, requires_grad=False,
+                                    tags={STATIC_MEMORY_LOCATION})
+                fetches.append(unpack.sym.bind(owner, f"{name}.{suffix}", output=proxy))
+                fetches.append(check_tensor_shape_and_metadata.bind(proxy, shape, device, dtype, False, output=None))
+                add_trace_output(prologue_trace, proxy, subindex=0)
+                extras_of[name][suffix] = proxy
+                new_inputs.append(proxy)
+        at_return = len(prologue_trace.bound_symbols) - 1
+        prologue_trace.bound_symbols[at_return:at_return] = fetches
 
-        computation_trace.args = (*computation_trace.args, *new_compute_inputs)
-        computation_trace.names.update(i.name for i in new_compute_inputs)
-        insert_idx = 0
-        for i, bsym in enumerate(computation_trace.bound_symbols):
-            if bsym.sym is unpack_trivial:
-                insert_idx = i + 1
-        computation_trace.bound_symbols[insert_idx:insert_idx] = [
-            unpack_trivial.bind(i, output=i, name=i.name) for i in new_compute_inputs
-        ]
+        computation_trace.args = (*computation_trace.args, *new_inputs)
+        computation_trace.names |= {p.name for p in new_inputs}
+        body = computation_trace.bound_symbols
+        after_unpacks = max((i + 1 for i, b in enumerate(body) if b.sym is unpack_trivial), default=0)
+        body[after_unpacks:after_unpacks] = [unpack_trivial.bind(p, output=p, name=p.name) for p in new_inputs]
 
-        new_bound_symbols = []
-        for bsym in computation_trace.bound_symbols:
-            if bsym.sym is extend.linear and isinstance(bsym.args[1], TensorProxy) and bsym.args[1].name in quantized_proxies:
-                assert len(bsym.args) == 3  # linear(input, weight, bias)
-                n = quantized_proxies[bsym.args[1].name]
-                qs = self.quant_states[n]
-                new_args = (*bsym.args[:3], additional_proxies[f"{n}.absmax"], additional_proxies[f"{n}.code"],
-                            qs["blocksize"], qs["dtype"], qs["shape"])
-                new_bound_symbols.append(bsym.from_bsym(sym=hip_matmul_nf4, subsymbols=(), args=new_args))
+        rewritten = []
+        for bsym in body:
+            weight = bsym.args[1] if bsym.sym is extend.linear and len(bsym.args) > 1 else None
+            if isinstance(weight, TensorProxy) and weight.name in weight_of_proxy:
+                assert len(bsym.args) == 3, "linear(input, weight, bias)"
+                name = weight_of_proxy[weight.name]
+                rewritten.append(self._operator_call(bsym, self.quant_states[name], extras_of[name]))
             elif bsym.sym is python_return:
-                ret = dict(bsym.args[0])
-                ret["flat_args"] = list(computation_trace.args)
-                new_bound_symbols.append(bsym.from_bsym(args=(ret,)))
+                returned_dict = dict(bsym.args[0])
+                returned_dict["flat_args"] = list(computation_trace.args)
+                rewritten.append(bsym.from_bsym(args=(returned_dict,)))
             else:
-                new_bound_symbols.append(bsym)
-        computation_trace.bound_symbols = new_bound_symbols
+                rewritten.append(bsym)
+        computation_trace.bound_symbols = rewritten
         computation_trace.set_provenance("quant pass")
         return prologue_trace, computation_trace, epilogue_trace

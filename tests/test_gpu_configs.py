@@ -283,3 +283,40 @@ def test_quantize_guard_bands(ta, oracle, n, blocksize):
     qw_o, absmax_o = oracle.C().quantize(w, blocksize)
     assert torch.equal(packed_g.view(torch.uint8, ((n + 1) // 2, 1)).cpu(), qw_o)
     assert torch.equal(absmax_g.view(torch.float32, (nblocks,)).cpu(), absmax_o)
+
+
+# ------------------------------------------------------------------------------------------------
+# double quantisation through the product API: jit(model, transforms=[BitsAndBytesLinearQuant4bit(double_quant=True)])
+# ------------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("N,K", [(1024, 8192), (8192, 8192)])
+def test_double_quant_linear_through_jit(ta, oracle, N, K):
+    print(f"double_quant through jit [{N},{K}]", flush=True)
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(_cpu_weight(N, K, 5100 + N // 1024))
+    w_cpu = lin.weight.detach().clone()
+    lin = lin.to(DEV).eval().requires_grad_(False)
+    jm = ta.jit(lin, transforms=[ta.BitsAndBytesLinearQuant4bit(double_quant=True)], executors=(ta.get_hip_nf4_executor(),))
+    sd = {k: v.cpu() for k, v in jm.state_dict().items()}
+    assert set(sd) == {"weight", "weight.absmax", "weight.code", "weight.nested_absmax", "weight.nested_quant_map", "weight.nested_offset"}
+    # every stored tensor is what the CPU oracle computes from the same weight
+    qw_o, absmax_o = oracle.C().quantize(w_cpu, 64)
+    D = oracle.create_dynamic_map()
+    off = oracle.C().dq_offset(absmax_o)
+    q_o, a2_o = oracle.C().dq_compress(absmax_o, D, off)
+    assert torch.equal(sd["weight"], qw_o) and torch.equal(sd["weight.absmax"], q_o) and torch.equal(sd["weight.nested_absmax"], a2_o)
+    assert torch.equal(sd["weight.nested_quant_map"], D) and sd["weight.nested_offset"].tolist() == [off]
+    absmax_ref = oracle.C().dq_reconstruct(q_o, a2_o, D, off)
+    g = torch.Generator().manual_seed(N + K)
+    rows = torch.unique(torch.cat([torch.arange(0, 256), torch.arange(N - 256, N), torch.randint(0, N, (64,), generator=g)]))
+    deq = oracle.C().dequantize(qw_o.view(N, K // 2)[rows].reshape(-1, 1), absmax_ref.view(N, K // 64)[rows].reshape(-1), oracle.nf4_lut(),
+                                64, torch.bfloat16, (len(rows), K)).to(DEV).double()
+    for M in (1, 16, 2048):
+        x = _cpu_acts(M, K, 510000 + M).to(DEV)
+        y = jm(x)
+        assert y.shape == (M, N) and y.dtype == torch.bfloat16
+        torch.testing.assert_close(y[:, rows.to(DEV)].double(), x.double() @ deq.T, rtol=2e-2, atol=2e-2)
+    calls = [b.sym.name for b in ta.last_traces(jm)[-1].bound_symbols if b.sym.executor is not None]
+    assert calls == ["hip_matmul_nf4_dq"]

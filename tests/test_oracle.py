@@ -260,6 +260,188 @@ def test_nested_absmax_invariants(oracle):
     assert (qz == 127).all() and (az == 0).all() and (oracle.C().dq_reconstruct(qz, az, D, 0.0) == 0).all()
 
 
+# ---- nested absmax, pinned by mathematics -----------------------------------------------------------
+#
+# No file of the reference uses compress_statistics, so there is no call site, test or fixture to pin these
+# against; what follows checks the oracle's nested functions against exact rational arithmetic
+# (fractions.Fraction), math.fsum and closed forms -- none of them a restatement of the oracle's own fp32
+# formulas -- with inputs chosen so that a dropped offset, a fused multiply-add, fp32 accumulation of the
+# mean, a wrong nested block index or a wrong tie rule each fail at least one check.
+
+from fractions import Fraction
+import math
+
+
+def _f32(x: float) -> float:
+    return float(np.float32(x))
+
+
+def _round_fraction_to_f32(v: Fraction) -> float:
+    """Round-to-nearest-even of an exact rational to binary32 (normal range), by integer arithmetic."""
+    if v == 0:
+        return 0.0
+    sign = -1 if v < 0 else 1
+    a = abs(v)
+    e = a.numerator.bit_length() - a.denominator.bit_length()  # 2^(e-1) <= a < 2^(e+1)
+    if a < Fraction(2) ** e:
+        e -= 1
+    assert Fraction(2) ** e <= a < Fraction(2) ** (e + 1)
+    assert -126 <= e <= 127
+    scaled = a / Fraction(2) ** (e - 23)  # in [2^23, 2^24)
+    m = scaled.numerator // scaled.denominator
+    rem = scaled - m
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and m % 2 == 1):
+        m += 1
+    return sign * float(m) * 2.0 ** (e - 23)  # m <= 2^24 and the power of two are exact in double
+
+
+def test_round_fraction_helper_agrees_with_numpy_casts():
+    g = np.random.default_rng(5)
+    for x in np.concatenate([g.standard_normal(2000) * 0.05, g.standard_normal(2000) * 1e-4, [1.0, 0.1, 1 / 3, 2**-20 * (2**24 + 1)]]):
+        assert _round_fraction_to_f32(Fraction(float(x))) == _f32(float(x))
+    # an exact tie goes to the even significand: 2^24 + 1 is halfway between 2^24 and 2^24 + 2
+    assert _round_fraction_to_f32(Fraction(2**24 + 1)) == float(2**24)
+    assert _round_fraction_to_f32(Fraction(2**24 + 3)) == float(2**24 + 4)
+
+
+def test_dynamic_map_closed_form_by_rationals(oracle):
+    """256 distinct values; 0 and 1; for decade i = 0..6, 2^i positive values, equally spaced by 0.9 * 10^(i-6) / 2^i,
+    the first at (0.1 + 0.45 / 2^i) * 10^(i-6) -- all inside (0.1 * 10^(i-6), 10^(i-6)) -- and their mirror images."""
+    D = oracle.create_dynamic_map()
+    vals = [float(v) for v in D]
+    assert len(set(vals)) == 256 and vals == sorted(vals)
+    # the minimum is -(0.1 + 0.9 * 127 / 128) = -0.99296875 up to the fp32 linspace's last bit (-0.99296874 as published)
+    assert vals[127] == 0.0 and vals[255] == 1.0 and abs(vals[0] + 0.99296875) <= 2.0**-23
+    pos = vals[128:255]
+    assert [-v for v in reversed(vals[:127])] == pos, "the map is symmetric except for the lone 1.0"
+    k = 0
+    for i in range(7):
+        cnt = 2**i
+        scale = Fraction(10) ** (i - 6)
+        lo, hi = Fraction(1, 10) * scale, scale
+        seg = pos[k:k + cnt]
+        assert all(lo < Fraction(v) < hi for v in seg), f"decade {i} out of its edges"
+        for j, v in enumerate(seg):
+            exact = (Fraction(1, 10) + Fraction(9, 10) * Fraction(2 * j + 1, 2 * cnt)) * scale
+            # the published construction goes through fp32 linspace and a double product: allow 2 ulp of fp32
+            assert abs(Fraction(v) - exact) <= exact * Fraction(2, 2**23), (i, j, v, float(exact))
+        k += cnt
+    assert k == 127
+
+
+def test_offset_is_the_correctly_rounded_mean(oracle):
+    g = torch.Generator().manual_seed(99)
+    cases = [
+        (torch.rand(100000, generator=g) * 0.08 + 0.01).float(),
+        torch.cat([torch.full((1,), 1000.0), torch.rand(70000, generator=g) * 1e-4]).float(),  # fp32 accumulation loses the tail
+        torch.tensor([0.1, 0.2, 0.30000001, 1e-8], dtype=torch.float32),
+        torch.full((3,), 0.1, dtype=torch.float32),
+    ]
+    for a in cases:
+        exact = Fraction(0)
+        for v in a.tolist():
+            exact += Fraction(v)
+        want = _round_fraction_to_f32(exact / len(a))
+        assert oracle.C().dq_offset(a) == want
+        assert want == _f32(math.fsum(a.tolist()) / len(a))
+    # the case with one large value must tell a float32 running sum from the exact mean
+    a = cases[1]
+    running = np.float32(0)
+    for v in a.numpy():
+        running = np.float32(running + v)
+    assert _f32(float(running) / len(a)) != oracle.C().dq_offset(a)
+
+
+def test_nested_codes_are_exact_nearest_neighbours(oracle):
+    """absmax2 = max |absmax - offset| (each difference rounded to fp32, as the format stores fp32 statistics), code =
+    the map entry nearest to r / absmax2 in EXACT arithmetic.  The oracle works in fp32 (r * (1 / absmax2)), so it may
+    differ from the exact rule only where r / absmax2 lies within fp32 rounding distance of the midpoint of two map
+    entries; every such case found by the sweep is counted and its distance from the midpoint checked."""
+    D = oracle.create_dynamic_map()
+    Dq = [Fraction(float(v)) for v in D]
+    mids = [(Dq[j] + Dq[j + 1]) / 2 for j in range(255)]
+    g = torch.Generator().manual_seed(7)
+    # two nested blocks of ordinary statistics, plus a block built to land near every midpoint
+    ordinary = (torch.rand(512, generator=g) * 0.08 + 0.01).float()
+    probe = torch.tensor([float(m) for m in mids] + [1.0], dtype=torch.float32)  # absmax2 = 1, offset = 0 below
+    near_ties = {}
+    for name, absmax, offset in (("ordinary", ordinary, oracle.C().dq_offset(ordinary)), ("probe", probe, 0.0)):
+        near_ties[name] = 0
+        q, a2 = oracle.C().dq_compress(absmax, D, offset)
+        nb = absmax.numel()
+        for c in range((nb + 255) // 256):
+            blk = absmax[c * 256:(c + 1) * 256].tolist()
+            r = [Fraction(float(np.float32(v) - np.float32(offset))) for v in blk]  # fp32 subtraction, exact afterwards
+            m = max(abs(x) for x in r)
+            assert Fraction(float(a2[c])) == m, "absmax2 is the exact maximum of the fp32 differences"
+            for i, x in enumerate(r):
+                s = x / m
+                dist = [abs(s - d) for d in Dq]
+                best = min(dist)
+                winners = [j for j, d in enumerate(dist) if d == best]
+                got = int(q[c * 256 + i])
+                if got in winners:
+                    if len(winners) > 1:
+                        assert got == winners[0], "exact tie: the lowest index wins"
+                    continue
+                # not the exact nearest neighbour: only legitimate within fp32 rounding of a midpoint
+                near_ties[name] += 1
+                j = min(got, winners[0])
+                assert abs(got - winners[0]) == 1 and abs(s - mids[j]) <= abs(mids[j]) * Fraction(4, 2**24) + Fraction(1, 2**40), (i, got, winners)
+    # ordinary statistics never land that close; the probe block may, for some of its 255 midpoints
+    assert near_ties["ordinary"] == 0 and near_ties["probe"] <= 255, near_ties
+    print("nested codes: near-midpoint cases where fp32 and exact arithmetic pick neighbouring entries:", near_ties)
+    q, _ = oracle.C().dq_compress(ordinary, D, oracle.C().dq_offset(ordinary))
+    assert len(set(q.tolist())) > 100  # the sweep really exercises the map, not a handful of codes
+
+
+def test_nested_block_indexing_and_partial_last_block(oracle):
+    """Statistics of different magnitude per nested block: a wrong block index or a maximum taken over the wrong range
+    changes absmax2; 600 entries = two full nested blocks and one of 88."""
+    D = oracle.create_dynamic_map()
+    a = torch.cat([torch.linspace(0.01, 0.02, 256), torch.linspace(1.0, 3.0, 256), torch.linspace(10.0, 10.5, 88)]).float()
+    off = oracle.C().dq_offset(a)
+    q, a2 = oracle.C().dq_compress(a, D, off)
+    assert a2.numel() == 3 and q.numel() == 600
+    for c, (lo, hi) in enumerate(((0, 256), (256, 512), (512, 600))):
+        want = max(abs(float(np.float32(v) - np.float32(off))) for v in a[lo:hi].tolist())
+        assert float(a2[c]) == want
+    # the element that attains the maximum gets code 255 (+1.0) or 0 (the most negative entry's neighbour -1 is absent:
+    # the map's minimum is -0.99296875, so a value of exactly -absmax2 maps to index 0)
+    r = a.numpy() - np.float32(off)
+    for c, (lo, hi) in enumerate(((0, 256), (256, 512), (512, 600))):
+        i = lo + int(np.abs(r[lo:hi]).argmax())
+        assert int(q[i]) == (255 if r[i] > 0 else 0)
+
+
+def test_reconstruction_is_multiply_then_add_rounded_twice(oracle):
+    D = oracle.create_dynamic_map()
+    g = torch.Generator().manual_seed(21)
+    q = torch.randint(0, 256, (4000,), generator=g, dtype=torch.int64).to(torch.uint8)
+    a2 = (torch.rand(16, generator=g) * 0.05 + 1e-3).float()
+    off = _f32(0.0423)
+    rec = oracle.C().dq_reconstruct(q, a2, D, off)
+    fused_differs = 0
+    for i in range(q.numel()):
+        d, s = Fraction(float(D[int(q[i])])), Fraction(float(a2[i // 256]))
+        p = _round_fraction_to_f32(d * s)
+        want = _round_fraction_to_f32(Fraction(p) + Fraction(off))
+        assert float(rec[i]) == want, i
+        fused_differs += want != _round_fraction_to_f32(d * s + Fraction(off))
+    # the sample tells two roundings from one (a fused multiply-add) ...
+    assert fused_differs > 50
+    # ... a dropped offset, and swapped nested blocks
+    assert not torch.equal(rec, oracle.C().dq_reconstruct(q, a2, D, 0.0))
+    assert not torch.equal(rec, oracle.C().dq_reconstruct(q, a2.flip(0), D, off))
+    # round trip: compress then reconstruct stays within half the widest map gap of each nested block's scale
+    absmax = (torch.rand(1000, generator=g) * 0.08 + 0.01).float()
+    o = oracle.C().dq_offset(absmax)
+    qq, aa = oracle.C().dq_compress(absmax, D, o)
+    back = oracle.C().dq_reconstruct(qq, aa, D, o)
+    gap = float(D.diff().max())
+    assert ((back - absmax).abs() <= aa.repeat_interleave(256)[:1000] * (gap / 2) + 1e-7).all()
+
+
 # ---- golden vectors ---------------------------------------------------------------------------------
 
 

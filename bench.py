@@ -13,8 +13,9 @@ Prints ONE JSON line:
               timed group by group): algorithmic bytes per launch / average launch duration, from
               HIP events recorded inside the timed region on the launch stream, against the
               8 TB/s HBM peak; config.kernels lists all three
-  config.prefill = BASELINE config 3 (M in {512, 2048, 8192}) run after the timed region: TFLOP/s of the
-              default route (HIP dequantize + dense GEMM) and of the fused GEMM kernel, vs the bf16 MFMA peak
+  config.prefill = BASELINE config 3 (M in {512, 2048, 8192}) run after the timed region: TFLOP/s of the fused GEMM
+              kernel and of HIP dequantize + dense GEMM, vs the bf16 MFMA peak; which of the two the router picks
+  config.llama70b_double_quant = BASELINE config 5 (nested absmax, M in {1, 16, 2048}) run after the timed region
   config.decode = BASELINE config 4 (full Llama-3-8B architecture, greedy decode, batch 1 and 8)
               run after the timed region: decode tokens/s, the second half of the metric
   cpu_baseline = the reference's CPU-side route (torch-eager dequantize + linear, restated in
@@ -70,6 +71,16 @@ def main() -> int:
     code = ta.nf4_code(dev)
 
     # ---- synthetic weights: seeded bf16 N(0, 0.02), quantized by the HIP kernel, `ncopy` copies ----
+    # Copy 0 of every ring is the canonical tensor of the configuration, drawn on the CPU (weight seed 2000 + index
+    # of the shape, activation seed 200000 + 100 * shape + index of M) and fingerprinted with SHA-256 so that runs on
+    # different boxes can be compared; the other copies only exist to defeat the Infinity Cache and are drawn on the
+    # GPU.
+    import hashlib
+
+    def sha(t):
+        return hashlib.sha256(t.contiguous().view(torch.int16).numpy().tobytes()).hexdigest()[:16]
+
+    fingerprints = {}
     weights = {}
     for si, (N, K) in enumerate(SHAPES):
         n = N * K
@@ -77,8 +88,14 @@ def main() -> int:
         ncopy = max(2, -(-RING_BYTES // per_copy))
         ring = []
         for c in range(ncopy):
-            g = torch.Generator(device=dev).manual_seed(2000 + 100 * si + c)
-            w = (torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+            if c == 0:
+                w_cpu = (torch.randn(N, K, generator=torch.Generator().manual_seed(2000 + si), dtype=torch.float32) * 0.02).to(torch.bfloat16)
+                fingerprints[f"W[{N},{K}] seed {2000 + si}"] = sha(w_cpu)
+                w = w_cpu.to(dev)
+                del w_cpu
+            else:
+                g = torch.Generator(device=dev).manual_seed(2000 + 100 * si + c)
+                w = (torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
             qw, absmax, _ = ta.quantize_nf4(w, BLOCKSIZE)
             ring.append((qw, absmax))
             del w
@@ -86,8 +103,10 @@ def main() -> int:
     xs, outs = {}, {}
     for mi, M in enumerate(MS):
         for si, (N, K) in enumerate(SHAPES):
-            g = torch.Generator(device=dev).manual_seed(200000 + 100 * si + mi)
-            xs[(M, N, K)] = torch.randn(M, K, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            seed = 200000 + 100 * si + mi
+            x_cpu = torch.randn(M, K, generator=torch.Generator().manual_seed(seed), dtype=torch.float32).to(torch.bfloat16)
+            fingerprints[f"x[{M},{K}] seed {seed}"] = sha(x_cpu)
+            xs[(M, N, K)] = x_cpu.to(dev)
             outs[(M, N, K)] = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     ws_bytes = max(lib.nf4hip_gemv_workspace_bytes(M, N, K) for M in MS for (N, K) in SHAPES)
     ws = torch.zeros(max(ws_bytes, 1 << 20), dtype=torch.uint8, device=dev)
@@ -141,14 +160,33 @@ def main() -> int:
     wall = t1 - t0
     ms_per_step = wall * 1e3 / args.steps
     value = bytes_step * args.steps / wall / 1e9
+
+    # the same calls on ONE copy of every weight (it = 0 throughout): what the Infinity Cache makes of them; reported
+    # next to the cold numbers, never as the metric
+    warm_events = [torch.cuda.Event(enable_timing=True) for _ in range(len(groups) * 10 + 1)]
+    for s_ in range(10):
+        step(0, warm_events, s_)
+    warm_events[-1].record(stream)
+    torch.cuda.synchronize()
+
+    def pct(sorted_vals, q):
+        return sorted_vals[min(len(sorted_vals) - 1, int(q * len(sorted_vals)))]
+
     kernels = []
     for gi, (name, what, calls) in enumerate(groups):
         G = len(groups)
-        ms = sum(events[st * G + gi].elapsed_time(events[st * G + gi + 1]) for st in range(args.steps)) / args.steps
+        per_step = sorted(events[st * G + gi].elapsed_time(events[st * G + gi + 1]) for st in range(args.steps))
+        ms = sum(per_step) / args.steps
+        warm = sorted(warm_events[st * G + gi].elapsed_time(warm_events[st * G + gi + 1]) for st in range(10))
+        per_launch = 1e3 / len(calls)
         kernels.append({
             "kernel": name, "calls": what, "launches_per_step": len(calls),
             "algorithmic_bytes_per_launch": group_bytes[gi] // len(calls),
-            "avg_launch_us": round(ms * 1e3 / len(calls), 3),
+            "avg_launch_us": round(ms * per_launch, 3),
+            "median_launch_us": round(pct(per_step, 0.5) * per_launch, 3),
+            "p10_launch_us": round(pct(per_step, 0.1) * per_launch, 3),
+            "p90_launch_us": round(pct(per_step, 0.9) * per_launch, 3),
+            "warm_median_launch_us": round(pct(warm, 0.5) * per_launch, 3),
             "achieved_GBs": round(group_bytes[gi] / (ms * 1e-3) / 1e9, 1),
             "share_of_step_time": round(ms / ms_per_step, 3),
         })
@@ -172,7 +210,7 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic (seeded bf16 N(0,0.02) weights quantized to NF4 on the GPU, x bf16 N(0,1))",
+        "data": "synthetic (CPU-seeded bf16 N(0,0.02) weights quantized to NF4 by the HIP kernel, x bf16 N(0,1); fingerprints in config.inputs_sha256_16)",
         "config": {
             "workload": "BASELINE config 2: Llama-3-8B projection shapes [4096,4096],[1024,4096],[14336,4096],"
                         "[4096,14336],[128256,4096] as NF4 linears (blocksize 64, fp32 absmax), M in {1,4,16}; "
@@ -180,6 +218,7 @@ def main() -> int:
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
             "algorithmic_bytes_per_step": bytes_step,
             "kernels": kernels,
+            "inputs_sha256_16": fingerprints,
         },
         "roofline": {
             "kernel": f"{dom['kernel']} ({dom['calls']}: the {dom['launches_per_step']} calls per step that take the most time)",
@@ -198,6 +237,7 @@ def main() -> int:
     torch.cuda.empty_cache()
     if not args.no_prefill:
         result["config"]["prefill"] = prefill_section(torch, ta)
+        result["config"]["llama70b_double_quant"] = double_quant_section(torch, ta)
         result["config"]["codec"] = codec_section(torch, ta)
     if args.decode_tokens > 1:
         result["config"]["decode"] = llama_decode(torch, ta, args.decode_tokens)
@@ -210,63 +250,133 @@ def main() -> int:
 MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CUs x 2.4 GHz x 4096 flop/clk/CU
 
 
+def _timed(torch, fn, reps, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / reps
+
+
+def _cpu_seeded(torch, shape, seed, std):
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float32) * std).to(torch.bfloat16)
+
+
 def prefill_section(torch, ta) -> dict:
-    """BASELINE config 3, outside the timed region of the GEMV metric: the Llama-3-8B projection
-    shapes (and the fused gate/up weight [28672, 4096]) with M in {512, 2048, 8192} rows of x through
-    ``matmul_nf4`` -- which routes them to nf4hip_dequantize + the dense library GEMM, or to the fused
-    NF4 GEMM kernel (nf4hip_gemm) for the tall weight at M = 512 -- and the fused kernel forced at
-    M = 2048 for comparison.  TFLOP/s = 2 M N K / time, HIP events bracket 10 calls (3 for the forced
-    fused kernel) after 3 warm-up calls.  ``rows64``: the same weights with 64 rows of x, the router's
-    route (the fused kernel, K split over workgroups) next to the dense route forced."""
+    """BASELINE config 3, outside the timed region of the GEMV metric: the five Llama-3-8B projection shapes (and the
+    fused gate/up weight [28672, 4096]) with M in {512, 2048, 8192} rows of x.  Every case is timed on BOTH routes
+    -- the hand-written fused kernel (nf4hip_gemm: NF4 codes expanded on chip straight into MFMA operands) and
+    nf4hip_dequantize + the dense library GEMM -- and ``router`` names the one ``matmul_nf4`` picks.  TFLOP/s = 2 M N K /
+    time against the bf16 MFMA peak; HIP events bracket 10 calls (4 beyond 4 TFLOP per call) after 3 warm-up calls.
+    ``rows64``: the same weights with 64 rows of x (fused kernel with K split over workgroups vs the dense route)."""
+    dev = torch.device("cuda:0")
+    F = ta.functional
+    L, lib = ta._lib, ta._lib.load()
+    code = ta.nf4_code(dev)
+    sptr = torch.cuda.current_stream().cuda_stream
+    names = {"dequant+gemm": "nf4hip_dequantize + dense GEMM", "gemm": "nf4hip_gemm (fused)"}
+    rows, mid = [], []
+    shapes = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096), (28672, 4096)]
+    for si, (N, K) in enumerate(shapes):
+        w = _cpu_seeded(torch, (N, K), 2000 + si if si < 5 else 2900, 0.02).to(dev)  # configs 2 and 3 share their weights
+        qw, absmax, _ = ta.quantize_nf4(w, BLOCKSIZE)
+        del w
+        for mi, M in enumerate((512, 2048, 8192)):
+            x = _cpu_seeded(torch, (M, K), 300000 + 100 * si + mi, 1.0).to(dev)
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            flops = 2.0 * M * N * K
+            reps = 10 if flops < 4e12 else 4
+            need = lib.nf4hip_gemm_workspace_bytes(M, N, K)
+            ws = torch.zeros(max(need, 16), dtype=torch.uint8, device=dev)
+
+            def fused():
+                L.check(lib.nf4hip_gemm(x.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(), None, N, K, BLOCKSIZE,
+                                        out.data_ptr(), ws.data_ptr(), ws.numel(), sptr))
+
+            def dense():
+                return torch.nn.functional.linear(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)))
+
+            tf, td = _timed(torch, fused, reps), _timed(torch, dense, reps)
+            router = names[F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))]
+            for route, t in ((names["gemm"], tf), (names["dequant+gemm"], td)):
+                rows.append({"N": N, "K": K, "M": M, "route": route, "router_pick": route == router, "us": round(t * 1e6, 1),
+                             "tflops": round(flops / t / 1e12, 1), "frac_of_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+            del x, out
+        # 64 rows of x (between the decode and the prefill regime): the router's choice, which is the fused
+        # kernel with K split over workgroups, next to the dense route (dequantize + library GEMM) forced
+        x = _cpu_seeded(torch, (64, K), 390000 + si, 1.0).to(dev)
+        route = F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))
+        t = _timed(torch, lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 20)
+        td = _timed(torch, lambda: torch.nn.functional.linear(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K))), 20)
+        mid.append({"N": N, "K": K, "M": 64, "route": route, "us": round(t * 1e6, 1), "dense_route_us": round(td * 1e6, 1)})
+        del qw, absmax
+    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows, "rows64": mid}
+
+
+def double_quant_section(torch, ta) -> dict:
+    """BASELINE config 5, outside the timed region of the GEMV metric: Llama-3-70B layer shapes with double-quantised
+    statistics (NF4 blocksize 64, absmax in 8 bits over nested blocks of 256 plus an fp32 offset), M in {1, 16, 2048},
+    through ``matmul_nf4`` on the nested form.  Decode rows are rated against the HBM peak over their algorithmic bytes
+    (codes + 8-bit absmax + nested statistics + x + out), cold (weights rotated through a ring larger than the Infinity
+    Cache); M = 2048 against the bf16 MFMA peak."""
     dev = torch.device("cuda:0")
     F = ta.functional
     code = ta.nf4_code(dev)
+    lib = ta._lib.load()
+    dq_shapes = [(8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672)]
+    ws = torch.zeros(max(1 << 20, max(lib.nf4hip_gemv_workspace_bytes(M, N, K) for M in (1, 16) for (N, K) in dq_shapes)),
+                     dtype=torch.uint8, device=dev)
+    sptr = torch.cuda.current_stream().cuda_stream
+    cases = []
+    for si, (N, K) in enumerate(dq_shapes):
+        n = N * K
+        per_copy = n // 2 + n // BLOCKSIZE
+        ncopy = max(2, -(-RING_BYTES // per_copy))
+        ring = []
+        for c in range(ncopy):
+            if c == 0:
+                w = _cpu_seeded(torch, (N, K), 5000 + si, 0.02).to(dev)
+            else:
+                g = torch.Generator(device=dev).manual_seed(5000 + 100 * si + c)
+                w = (torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+            qw, absmax, _ = ta.quantize_nf4(w, BLOCKSIZE)
+            ring.append((qw, ta.compress_absmax(absmax)))
+            del w, absmax
+        nested_bytes = n // BLOCKSIZE + 4 * -(-(n // BLOCKSIZE) // 256) + 1024 + 4
+        for mi, M in enumerate((1, 16, 2048)):
+            x = _cpu_seeded(torch, (M, K), 500000 + 100 * si + mi, 1.0).to(dev)
+            route = F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))
+            it = [0]
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
 
-    def timed(fn, reps):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / reps
+            def call():
+                qw, nq = ring[it[0] % ncopy]
+                it[0] += 1
+                if M > 16:
+                    return ta.matmul_nf4(x, qw, None, nq, code, BLOCKSIZE, torch.bfloat16, (N, K))
+                # decode rows go straight to the C ABI, as the GEMV metric's own launches do
+                rc = lib.nf4hip_gemv_dq(x.data_ptr(), ta._lib.BF16, M, qw.data_ptr(), nq.q.data_ptr(), nq.absmax2.data_ptr(),
+                                        nq.map256.data_ptr(), float(nq.offset), nq.blocksize, code.data_ptr(), None, N, K,
+                                        BLOCKSIZE, out.data_ptr(), ws.data_ptr(), ws.numel(), sptr)
+                if rc:
+                    ta._lib.check(rc)
 
-    rows, mid = [], []
-    routes = {"dequant+gemm": "nf4hip_dequantize + dense GEMM", "gemm": "nf4hip_gemm (fused)"}
-    for si, (N, K) in enumerate([(4096, 4096), (14336, 4096), (4096, 14336), (28672, 4096)]):
-        g = torch.Generator(device=dev).manual_seed(3000 + si)
-        w = (torch.randn(N, K, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
-        qw, absmax, _ = ta.quantize_nf4(w, BLOCKSIZE)
-        del w
-        for M in (512, 2048, 8192):
-            x = torch.randn(M, K, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-            route = routes[F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))]
-            t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 10)
-            row = {"N": N, "K": K, "M": M, "route": route, "us": round(t * 1e6, 1),
-                   "tflops": round(2.0 * M * N * K / t / 1e12, 1),
-                   "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
-            rows.append(row)
-            if M == 2048:
-                saved, F.DENSE_ROUTE_MIN_M = F.DENSE_ROUTE_MIN_M, 1 << 30
-                try:
-                    assert F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K)) == "gemm"
-                    t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 3)
-                finally:
-                    F.DENSE_ROUTE_MIN_M = saved
-                rows.append({"N": N, "K": K, "M": M, "route": "nf4hip_gemm (fused, forced)", "us": round(t * 1e6, 1),
-                             "tflops": round(2.0 * M * N * K / t / 1e12, 1),
-                             "frac_of_mfma_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
-        # 64 rows of x (between the decode and the prefill regime): the router's choice, which is the fused
-        # kernel with K split over workgroups, next to the dense route (dequantize + library GEMM) forced
-        x = torch.randn(64, K, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        route = F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))
-        t = timed(lambda: ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)), 20)
-        td = timed(lambda: torch.nn.functional.linear(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K))), 20)
-        mid.append({"N": N, "K": K, "M": 64, "route": route, "us": round(t * 1e6, 1), "dense_route_us": round(td * 1e6, 1)})
-    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows, "rows64": mid}
+            t = _timed(torch, call, 20 if M <= 16 else 6, warm=ncopy if M <= 16 else 3)
+            row = {"N": N, "K": K, "M": M, "route": route, "us": round(t * 1e6, 1)}
+            if M <= 16:
+                byts = n // 2 + nested_bytes + 64 + 2 * M * K + 2 * M * N
+                row.update({"algorithmic_bytes": byts, "GBs": round(byts / t / 1e9, 1), "frac_of_hbm_peak": round(byts / t / 1e9 / HBM_PEAK_GBS, 4)})
+            else:
+                flops = 2.0 * M * N * K
+                row.update({"tflops": round(flops / t / 1e12, 1), "frac_of_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+            cases.append(row)
+        del ring
+    return {"note": "decode rows (M <= 16) call nf4hip_gemv_dq through the C ABI; M = 2048 goes through matmul_nf4 and its router", "cases": cases}
 
 
 def codec_section(torch, ta) -> dict:
@@ -361,34 +471,57 @@ def llama_decode(torch, ta, n_new: int) -> dict:
     return out
 
 
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(torch, budget_s: float) -> dict:
     """The reference's CPU route (torch-eager NF4 dequantize, then F.linear) on a bounded sample:
-    BASELINE config 1, one Linear(4096 -> 4096), x [1, 4096]."""
+    BASELINE config 1, one Linear(4096 -> 4096), x [1, 4096], on this box's host cores.  ``value`` is the whole
+    route; the split (dequantize | matmul) and the weights-already-dequantized variant are reported beside it."""
     from oracle import nf4_oracle as O
 
     N, K, M = 4096, 4096, 1
-    g = torch.Generator().manual_seed(1000)
-    w = (torch.randn(N, K, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
-    x = torch.randn(M, K, generator=torch.Generator().manual_seed(100000), dtype=torch.float32).to(torch.bfloat16)
+    w = _cpu_seeded(torch, (N, K), 1000, 0.02)
+    x = _cpu_seeded(torch, (M, K), 100000, 1.0)
     qw, absmax = O.C().quantize(w, BLOCKSIZE)
     lut = O.nf4_lut()
     threads = torch.get_num_threads()
-    O.matmul_4bit_eager(x, qw, None, absmax, lut, BLOCKSIZE, torch.bfloat16, (N, K))  # warm-up
-    times = []
-    t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
-        t0 = time.perf_counter()
-        O.matmul_4bit_eager(x, qw, None, absmax, lut, BLOCKSIZE, torch.bfloat16, (N, K))
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+
+    def median_time(fn, budget, most=200):
+        fn()  # warm-up
+        times, t_end = [], time.perf_counter() + budget
+        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < most):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    whole, n_whole = median_time(lambda: O.matmul_4bit_eager(x, qw, None, absmax, lut, BLOCKSIZE, torch.bfloat16, (N, K)), budget_s * 0.5)
+    deq_t, _ = median_time(lambda: O.dequantize_4bit_eager(qw, absmax, lut, BLOCKSIZE, torch.bfloat16, (N, K)), budget_s * 0.3)
+    wd = O.dequantize_4bit_eager(qw, absmax, lut, BLOCKSIZE, torch.bfloat16, (N, K))
+    mm_t, _ = median_time(lambda: torch.nn.functional.linear(x, wd), budget_s * 0.2)
     return {
-        "value": round(algorithmic_bytes(M, N, K) / med / 1e9, 3),
+        "value": round(algorithmic_bytes(M, N, K) / whole / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"{len(times)} calls of torch-eager dequantize_4bit + F.linear, NF4 Linear(4096->4096), x [1,4096] bf16 "
-                  f"(BASELINE config 1); median {med * 1e3:.1f} ms per call, {os.cpu_count()} host cpus visible",
+        "sample": f"{n_whole} calls of torch-eager dequantize_4bit + F.linear, NF4 Linear(4096->4096), x [1,4096] bf16 "
+                  f"(BASELINE config 1); median {whole * 1e3:.1f} ms per call",
+        "ms_whole_route": round(whole * 1e3, 2),
+        "ms_dequantize_only": round(deq_t * 1e3, 2),
+        "ms_matmul_on_dequantized_weight": round(mm_t * 1e3, 3),
+        "torch_num_threads": threads,
+        "os_cpu_count": os.cpu_count(),
+        "cpu_model": _cpu_model(),
     }
 
 

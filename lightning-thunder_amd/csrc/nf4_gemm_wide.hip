@@ -352,19 +352,64 @@ void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
         if (kt + 2 < ksteps) step(kt + 2, S2{}, c2, c0, std::false_type{});
     }
 
-    // acc[i][g][q] = out[m][n], n = 32 (NG wave + g) + lane % 32, m = 32 i + 8 (q / 4) + 4 (lane / 32) + q % 4
+    // acc[i][g][q] = out[m][n], n = 32 (NG wave + g) + lane % 32, m = 32 i + 8 (q / 4) + 4 (lane / 32) + q % 4.
+    // The tile leaves through LDS (the x stages are free now), half of its rows at a time, so that global memory
+    // sees 16-byte stores that cover whole rows of the tile (512 contiguous bytes per 32 lanes) instead of
+    // 2-byte stores in runs of 64 bytes.  Into LDS: rows q and q + 1 of a lane are rounded to one dword, lanes
+    // l and l ^ 1 exchange dwords (DPP) and v_perm_b32 leaves the even lane with columns (n, n + 1) of row q and
+    // the odd lane with the same columns of row q + 1: one ds_write_b32 per two outputs.  Row r of a half starts at
+    // 512 r; its dword c sits at c ^ 16 f(r), f(r) = r % 2 + 2 (r / 4 % 2), which keeps 16-byte pieces whole and
+    // sends the four rows one write instruction touches (r, r + 1, r + 4, r + 5) to four different bank groups.
+    __syncthreads();  // every wave has issued and received its last fragment reads
+    {
+        constexpr int HALF_ROWS = BM / 2;
+        uint8_t* stage = smem + BOOK_BYTES;
+        const uint32_t sel = (lane & 1) ? 0x03020706u : 0x05040100u;
+        const int wf = (lane & 1) | ((lane >> 5) << 1);
+        const bool vec = (a.N & 7) == 0;
 #pragma unroll
-    for (int g = 0; g < NG; ++g) {
-        const int n = n0 + (wave * NG + g) * 32 + (lane & 31);
-        if (n < a.N) {
-            const float b = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.0f;
+        for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int i = 0; i < T::TI; ++i)
+            for (int g = 0; g < NG; ++g) {
+                const int nl = (wave * NG + g) * 32 + (lane & 31);
+                const int n = n0 + nl;
+                const float b = (a.bias && n < a.N) ? bf16_bits_to_f32(a.bias[n]) : 0.0f;
+                uint8_t* wbase = stage + (4 * (lane >> 5) + (lane & 1)) * 512 + ((((uint32_t)nl >> 1) ^ ((uint32_t)wf << 4)) << 2);
 #pragma unroll
-                for (int q = 0; q < 16; ++q) {
-                    const int m = m0 + i * 32 + 8 * (q >> 2) + 4 * (lane >> 5) + (q & 3);
-                    if (m < a.M) a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(acc[i][g][q] + b);
+                for (int il = 0; il < T::TI / 2; ++il) {
+                    const int i = h * (T::TI / 2) + il;
+#pragma unroll
+                    for (int q = 0; q < 16; q += 2) {
+                        const float2_t f = {acc[i][g][q] + b, acc[i][g][q + 1] + b};
+                        const uint32_t mine = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+                        const uint32_t theirs = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1, 0xf, 0xf, true);
+                        const uint32_t packed = __builtin_amdgcn_perm(theirs, mine, sel);
+                        *reinterpret_cast<uint32_t*>(wbase + (32 * il + 8 * (q >> 2) + (q & 2)) * 512) = packed;
+                    }
                 }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < HALF_ROWS / (T::THREADS / 32); ++it) {
+                const int r = it * (T::THREADS / 32) + (tid >> 5);
+                const int piece = tid & 31;
+                const int fr2 = (r & 1) | (((r >> 2) & 1) << 1);
+                const uint4 v = *reinterpret_cast<const uint4*>(stage + r * 512 + ((piece ^ (fr2 << 2)) << 4));
+                const int m = m0 + h * HALF_ROWS + r;
+                const int n = n0 + piece * 8;
+                if (m < a.M) {
+                    uint16_t* dst = a.out + (int64_t)m * a.N + n;
+                    if (vec) {
+                        if (n < a.N) store16<false>(dst, v.x, v.y, v.z, v.w);
+                    } else {
+                        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (n + e < a.N) dst[e] = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                    }
+                }
+            }
+            if (h == 0) __syncthreads();
         }
     }
 #endif  // __HIP_DEVICE_COMPILE__

@@ -50,8 +50,9 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream);
 // more than 128 rows of x: one wave per SIMD, 256 x 256 or 128 x 256 tiles (nf4_gemm_wide.hip)
-int gemm_wide_tile_rows(int64_t M, int64_t N);
+int gemm_wide_tile_rows(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemm_wide(const MatmulArgs& a, hipStream_t stream);
+size_t gemm_wide_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 // ---------------------------------------------------------------------------------------------
 // device helpers

@@ -378,6 +378,7 @@ hipError_t launch_tile(const MatmulArgs& a, hipStream_t stream) {
 }  // namespace
 
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M > 128) return M * K * 2 < ((int64_t)1 << 32) ? gemm_wide_workspace_bytes(M, N, K) : 0;
     const int splits = gemm_splits(M, N, K);
     if (splits == 1) return 0;
     const int64_t bm = M <= 64 ? 64 : 128;

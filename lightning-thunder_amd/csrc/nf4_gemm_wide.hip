@@ -145,9 +145,27 @@ __device__ __forceinline__ void expansion_step(Expansion& x, int t, uint32_t d, 
 //
 // Order of issue inside a slice: after every MFMA first the LDS reads (the fragment of the next slice once its
 // last user has been issued, book reads), then at most a handful of VALU instructions.
+// How the tiles of one call are spread over workgroups (one workgroup per CU at a time, handed out in the order of
+// their numbers; GRID CUs).
+//   * The first `full` = rounds * GRID tiles are taken whole, one workgroup each.  Tile numbers (m fastest) are
+//     dealt so that every XCD -- workgroup b runs on XCD b % 8 -- owns a contiguous run of them: the x-row tiles
+//     that share a weight tile meet in one L2.
+//   * The remaining `tail_tiles` (fewer than GRID) would leave CUs idle in a last, partial round, so each of them
+//     can be cut into `pieces` equal pieces along k (in quanta of `gran` k steps, qpt per tile), one workgroup per
+//     piece, numbered piece-major (all first pieces, then all second pieces, ...).  The pieces of a tile meet in
+//     the workspace (see the kernel).  pieces == 1: whole tiles.
+struct WideSchedule {
+    int m_tiles, n_tiles;
+    int full, tail_tiles, pieces;
+    int qpt, gran;
+    uint32_t* counters;  // two per tail tile, zero between calls
+    float* partials;     // one slot of BM x 256 floats per piece
+};
+constexpr int GRID = 256;
+
 template <bool NESTED, int BM, int NG>
 __global__ __launch_bounds__(512 / NG) __attribute__((amdgpu_waves_per_eu(3 - NG, 3 - NG)))
-void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
+void gemm_wide_kernel(MatmulArgs a, WideSchedule sch) {
     // The body exists in the device pass only: the host pass cannot instantiate the buffer-resource type
     // it uses and would then leave the kernel's launch stub undefined.
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -170,14 +188,28 @@ void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
     const uint32_t book_lane = (lane & 31) * 8;
     const uint32_t stage0 = BOOK_BYTES;
 
-    const int total = m_tiles * n_tiles;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int chunk = total >> 3, rem = total & 7;
-    const int id = xcd * chunk + min(xcd, rem) + slot;
+    // ---- what this workgroup works on: a whole tile, or one piece of a tail tile ----
+    const int m_tiles = sch.m_tiles;
+    const int ksteps_all = a.K / BK;
+    int id, kfirst = 0, ksteps = ksteps_all, tail_tile = -1, piece = 0;
+    if ((int)blockIdx.x < sch.full) {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        id = xcd * (sch.full >> 3) + slot;
+    } else {
+        const int p = blockIdx.x - sch.full;
+        piece = p / sch.tail_tiles;
+        tail_tile = p - piece * sch.tail_tiles;
+        id = sch.full + tail_tile;
+        if (sch.pieces > 1) {
+            const int q0 = piece * sch.qpt / sch.pieces, q1 = (piece + 1) * sch.qpt / sch.pieces;
+            kfirst = q0 * sch.gran;
+            ksteps = (q1 - q0) * sch.gran;
+        }
+    }
+    const bool partial = sch.pieces > 1 && tail_tile >= 0;
     const int nt = id / m_tiles;
     const int mt = id - nt * m_tiles;
     const int m0 = mt * BM, n0 = nt * BN;
-    const int ksteps = a.K / BK;
 
     f32x16 acc[T::TI][NG];
 #pragma unroll
@@ -203,7 +235,7 @@ void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
         const int c = T::XL * wave + j;
         const int rr = (lane >> 3) ^ (c & 1);
         const int row = min(m0 + 8 * c + rr, a.M - 1);
-        xoff[j] = (uint32_t)row * (uint32_t)(a.K * 2) + (uint32_t)(((lane & 7) ^ rr) << 4);
+        xoff[j] = (uint32_t)row * (uint32_t)(a.K * 2) + (uint32_t)(((lane & 7) ^ rr) << 4) + (uint32_t)(kfirst * (BK * 2));
     }
     auto load_x = [&](int kt, int stage) {  // k step kt into a stage
         const uint32_t st = stage0 + stage * T::STAGE_BYTES + T::XL * wave * CHUNK_BYTES;
@@ -223,7 +255,7 @@ void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
     int64_t e0[NG];
 #pragma unroll
     for (int g = 0; g < NG; ++g)
-        e0[g] = (int64_t)min(n0 + (wave * NG + g) * 32 + (lane & 31), a.N - 1) * a.K + (lane >> 5) * 32;
+        e0[g] = (int64_t)min(n0 + (wave * NG + g) * 32 + (lane & 31), a.N - 1) * a.K + (lane >> 5) * 32 + kfirst * BK;
 
     // Three k steps of x and of codes are under way at any time: stages and code sets rotate with period 3.
     Codes c0[NG], c1[NG], c2[NG];
@@ -361,7 +393,110 @@ void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
     // 512 r; its dword c sits at c ^ 16 f(r), f(r) = r % 2 + 2 (r / 4 % 2), which keeps 16-byte pieces whole and
     // sends the four rows one write instruction touches (r, r + 1, r + 4, r + 5) to four different bank groups.
     __syncthreads();  // every wave has issued and received its last fragment reads
-    {
+
+    // ---- a piece of a tail tile: meet the tile's other pieces in the workspace ----
+    // Pieces are numbered in k order; piece c of tail tile t has a slot of its own (t * pieces + c) for its fp32
+    // partial tile in register order ([i][g][q][thread]: coalesced).  Two counters per tile, zero between calls: P
+    // counts published partials, T hands out tickets.
+    //   * Every piece but the last to finish stores its partial, waits until L2 has it (publish_partials), and only
+    //     then counts itself in P.  Whoever raises P to the number of pieces adds all partials from memory, in k
+    //     order, and writes the tile.
+    //   * Two pieces (the common case): the holder of the second ticket looks at P first; if the other partial is
+    //     published already, it adds it to its registers and writes the tile without storing a partial (a + b = b + a
+    //     exactly, so the result does not depend on who finishes last).  Otherwise it proceeds like everyone else.
+    // No workgroup ever waits for another one.
+    bool write_tile = true;
+    if (partial) {
+        constexpr int SLOT = BM * BN;  // floats
+        constexpr int FR = 16 * T::THREADS;  // floats per accumulator fragment
+        const int pieces = sch.pieces;
+        uint32_t* cP = sch.counters + 2 * tail_tile;
+        uint32_t* cT = cP + 1;
+        auto slot_of = [&](int c) { return sch.partials + (int64_t)(tail_tile * pieces + c) * SLOT; };
+        volatile uint32_t* flag = reinterpret_cast<volatile uint32_t*>(smem + BOOK_BYTES);
+        bool in_registers = false;
+        if (pieces == 2) {
+            if (tid == 0) {
+                const uint32_t ticket = __hip_atomic_fetch_add(cT, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                uint32_t ok = 0;
+                if (ticket == 1) ok = __hip_atomic_load(cP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
+                *flag = ok;
+            }
+            __syncthreads();
+            in_registers = *flag != 0;
+            acquire_partials();
+            __syncthreads();
+        }
+        bool from_memory = false;
+        if (!in_registers) {
+            float* mine = slot_of(piece);
+#pragma unroll
+            for (int i = 0; i < T::TI; ++i)
+#pragma unroll
+                for (int g = 0; g < NG; ++g)
+#pragma unroll
+                    for (int q = 0; q < 16; ++q)
+                        __hip_atomic_store(mine + ((i * NG + g) * 16 + q) * T::THREADS + tid, acc[i][g][q], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+            publish_partials();
+            __syncthreads();
+            if (tid == 0) *flag = __hip_atomic_fetch_add(cP, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+            __syncthreads();
+            from_memory = *flag == (uint32_t)pieces;
+            acquire_partials();
+            __syncthreads();
+        }
+        if (in_registers) {
+            const float* other = slot_of(piece ^ 1);
+            constexpr int B = 4;  // fragments whose loads are in flight together
+#pragma unroll
+            for (int f0 = 0; f0 < T::TI * NG; f0 += B) {
+                float v[B][16];
+#pragma unroll
+                for (int f = 0; f < B; ++f)
+#pragma unroll
+                    for (int q = 0; q < 16; ++q)
+                        v[f][q] = __hip_atomic_load(other + ((f0 + f) * 16 + q) * T::THREADS + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int f = 0; f < B; ++f)
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) acc[(f0 + f) / NG][(f0 + f) % NG][q] += v[f][q];
+            }
+        } else if (from_memory) {
+            constexpr int G = 4;  // pieces whose loads are in flight together
+#pragma unroll
+            for (int f = 0; f < T::TI * NG; ++f) {
+                float sum[16];
+#pragma unroll
+                for (int q = 0; q < 16; ++q) sum[q] = 0.0f;
+#pragma unroll 1
+                for (int c0 = 0; c0 < pieces; c0 += G) {
+                    float v[G][16];
+#pragma unroll
+                    for (int c = 0; c < G; ++c) {
+                        const float* src = slot_of(min(c0 + c, pieces - 1)) + f * FR + tid;
+#pragma unroll
+                        for (int q = 0; q < 16; ++q)
+                            v[c][q] = __hip_atomic_load(src + q * T::THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int c = 0; c < G; ++c)
+                        if (c0 + c < pieces) {
+#pragma unroll
+                            for (int q = 0; q < 16; ++q) sum[q] += v[c][q];
+                        }
+                }
+#pragma unroll
+                for (int q = 0; q < 16; ++q) acc[f / NG][f % NG][q] = sum[q];
+            }
+        }
+        write_tile = in_registers || from_memory;
+        if (write_tile && tid == 0) {
+            __hip_atomic_store(cP, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(cT, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (write_tile) {
         constexpr int HALF_ROWS = BM / 2;
         uint8_t* stage = smem + BOOK_BYTES;
         const uint32_t sel = (lane & 1) ? 0x03020706u : 0x05040100u;
@@ -415,6 +550,41 @@ void gemm_wide_kernel(MatmulArgs a, int m_tiles, int n_tiles) {
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+// Bytes of workspace a cut-up tail needs: the counter region and one partial-tile slot per piece.
+size_t wide_tail_bytes(int tail_tiles, int pieces, int bm) {
+    return (size_t)GEMV_COUNTER_BYTES + (size_t)tail_tiles * pieces * bm * BN * sizeof(float);
+}
+
+// The schedule of a call: a pure function of the shape and of the size of the workspace it is given.  With a
+// workspace that is too small (or none) the tail tiles are taken whole.
+WideSchedule wide_schedule(int64_t M, int64_t N, int64_t K, int bm, size_t workspace_bytes) {
+    WideSchedule s{};
+    s.m_tiles = (int)((M + bm - 1) / bm);
+    s.n_tiles = (int)((N + BN - 1) / BN);
+    const int64_t tiles = (int64_t)s.m_tiles * s.n_tiles;
+    s.full = (int)(tiles / GRID) * GRID;
+    s.tail_tiles = (int)(tiles - s.full);
+    const int ksteps = (int)(K / BK);
+    s.gran = ksteps % 4 == 0 ? 4 : ksteps % 2 == 0 ? 2 : 1;
+    s.qpt = ksteps / s.gran;
+    s.pieces = 1;
+    if (s.tail_tiles == 0 || s.full > 0 || ksteps < 32) return s;
+    const int R = s.tail_tiles;
+    // Cutting pays only where it puts idle CUs to work on pieces that stay long: a call with fewer tiles than CUs,
+    // at most GRID pieces in all, of 16 k steps or more.  Measured without gain: a partial round behind full
+    // rounds cut in two ([28672, 4096], 2048 rows of x: 461 vs 464 us -- the chip is power-limited and a partial
+    // round runs at a higher clock), and more than GRID / 2 tiles cut into a long and a short piece each (the
+    // short pieces cost more in start-up and hand-off than they save).
+    int n = GRID / R;
+    if (n > 8) n = 8;
+    if (n > ksteps / 16) n = ksteps / 16;
+    if (n > s.qpt) n = s.qpt;
+    if (n < 2) return s;
+    s.pieces = n;
+    if (workspace_bytes < wide_tail_bytes(R, s.pieces, bm)) s.pieces = 1;
+    return s;
+}
+
 constexpr int WIDE_NG = 1;
 
 constexpr int MAX_DEVICES = 64;
@@ -434,24 +604,34 @@ hipError_t launch_tile(const MatmulArgs& a, hipStream_t stream) {
         if (e != hipSuccess) return e;
         ready[dev] = true;
     }
-    const int m_tiles = (a.M + BM - 1) / BM;
-    const int n_tiles = (a.N + BN - 1) / BN;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(m_tiles * n_tiles)), dim3(T::THREADS), T::SMEM_BYTES, stream, a, m_tiles, n_tiles);
+    WideSchedule sch = wide_schedule(a.M, a.N, a.K, BM, a.workspace ? a.workspace_bytes : 0);
+    sch.counters = static_cast<uint32_t*>(a.workspace);
+    sch.partials = a.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES) : nullptr;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(sch.full + sch.tail_tiles * sch.pieces)), dim3(T::THREADS), T::SMEM_BYTES, stream, a, sch);
     return hipGetLastError();
 }
 
 }  // namespace
 
-// Rows of x per tile: 256, or 128 when 256-row tiles would leave more than half of a 256-CU chip without
-// a workgroup in the only round (a pure function of the shape).
-int gemm_wide_tile_rows(int64_t M, int64_t N) {
-    const int64_t n_tiles = (N + BN - 1) / BN;
-    return ((M + 255) / 256) * n_tiles <= 128 ? 128 : 256;
+// Rows of x per tile (a pure function of the shape).  The 256-row tile expands every weight half as often, the
+// 128-row tile gives twice the workgroups: 256 rows once that makes 160 tiles or more, or when the k loop is long
+// enough for the pieces of a cut-up tile to stay long (tiles x k steps >= 28672, e.g. 128 tiles of K = 14336);
+// measured on both sides of either bound.
+int gemm_wide_tile_rows(int64_t M, int64_t N, int64_t K) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + BN - 1) / BN);
+    return tiles >= 160 || tiles * (K / BK) >= 28672 ? 256 : 128;
+}
+
+// Workspace of a call: none when no tile is cut up.
+size_t gemm_wide_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int bm = gemm_wide_tile_rows(M, N, K);
+    const WideSchedule s = wide_schedule(M, N, K, bm, ~(size_t)0);
+    return s.pieces > 1 ? wide_tail_bytes(s.tail_tiles, s.pieces, bm) : 0;
 }
 
 hipError_t launch_gemm_wide(const MatmulArgs& a, hipStream_t stream) {
     const bool nested = a.nested.q != nullptr;
-    if (gemm_wide_tile_rows(a.M, a.N) == 128)
+    if (gemm_wide_tile_rows(a.M, a.N, a.K) == 128)
         return nested ? launch_tile<true, 128>(a, stream) : launch_tile<false, 128>(a, stream);
     return nested ? launch_tile<true, 256>(a, stream) : launch_tile<false, 256>(a, stream);
 }

@@ -296,7 +296,7 @@ def matmul_nf4_dq(x, qweight, bias, absmax_q, nested_absmax, nested_quant_map, n
 
 # 40 MiB covers every Llama-3-8B / 70B projection shape on both fused routes (the largest need is the fused
 # GEMM's 33 MB of partial tiles at [16384, 8192], M = 128), so a stream's buffer is normally allocated once.
-_workspace_pool = WorkspacePool(40 << 20, "NF4 matmul")
+_workspace_pool = WorkspacePool(65 << 20, "NF4 matmul")  # 256 partial tiles of 256 x 256 floats + the counter region
 
 
 def _gemv_workspace(device: torch.device, nbytes: int, stream: int | None = None) -> torch.Tensor:
@@ -350,30 +350,54 @@ def _dense_route_us(N: int, K: int) -> float:
     return 20.0 + 0.62 * N * K / 1e6
 
 
+def _wide_schedule(M: int, N: int, K: int) -> tuple[int, int, int]:
+    """(rows of x per tile, tiles, pieces per tile) of the fused GEMM kernel for more than 128 rows of x; mirrors
+    gemm_wide_tile_rows and wide_schedule in csrc/nf4_gemm_wide.hip: the 256-row tile from 160 tiles on or when
+    tiles x k steps >= 28672, else the 128-row tile; a call with fewer tiles than the 256 CUs cuts every tile into
+    up to 8 equal pieces along k (at most 256 pieces in all, 16 k steps or more each) that meet in the workspace."""
+    n_tiles, ksteps = (N + 255) // 256, K // 64
+    tiles256 = ((M + 255) // 256) * n_tiles
+    bm = 256 if tiles256 >= 160 or tiles256 * ksteps >= 28672 else 128
+    tiles = ((M + bm - 1) // bm) * n_tiles
+    pieces = 1
+    if tiles < 256 and ksteps >= 32:
+        gran = 4 if ksteps % 4 == 0 else 2 if ksteps % 2 == 0 else 1
+        pieces = max(1, min(256 // tiles, 8, ksteps // 16, ksteps // gran))
+    return bm, tiles, pieces
+
+
 def _wide_gemm_us(M: int, N: int, K: int) -> float:
-    """Model of the fused GEMM kernel for more than 128 rows of x (csrc/nf4_gemm_wide.hip): tiles of 256 x 256
-    (128 x 256 when the larger tile would leave half the chip without a workgroup) run in rounds of 256
-    workgroups, K / 64 steps each; a step of the 256-row tile takes 1.85 us on a full chip, of the 128-row tile
-    1.0 us, 40 % less on a nearly empty one; 12 us of launch, prologue and epilogue.  Measured / modelled,
-    us: [14336, 4096] M = 256 / 1024 / 2048: 55 / 117 / 232 vs 62 / 124 / 237; [4096, 14336] M = 256 / 1024: 162 / 174 vs 158 /
-    191; [8192, 28672] M = 512: 361 vs 370; lm_head [128256, 4096] M = 1024 / 2048: 978 / 1938 vs 950 / 1890."""
-    n_tiles = (N + 255) // 256
-    bm = 128 if ((M + 255) // 256) * n_tiles <= 128 else 256
-    wgs = ((M + bm - 1) // bm) * n_tiles
+    """Model of the fused GEMM kernel for more than 128 rows of x (csrc/nf4_gemm_wide.hip): workgroups (one per tile
+    or piece of a tile) run in rounds of 256, K / 64 / pieces steps each; a step of the 256-row tile takes 1.85 us
+    on a full chip, of the 128-row tile 1.0 us, up to 40 % less on a sparsely filled one; 12 us of launch, prologue
+    and epilogue; pieces that meet in the workspace add 6 us (128-row tile) or 12 us.  Measured / modelled, us:
+    [4096, 4096] M = 256 / 512 / 1024 / 2048: 30 / 36 / 53 / 75 vs 29 / 37 / 53 / 76; [1024, 4096] M = 256 / 2048: 25 / 34
+    vs 27 / 37; [4096, 14336] M = 256 / 512 / 2048: 52 / 77 / 229 vs 49 / 77 / 233; [8192, 28672] M = 512: 230 vs 233;
+    [14336, 4096] M = 512 / 1024 / 2048: 69 / 113 / 220 vs 68 / 124 / 237; lm_head [128256, 4096] M = 2048: 1940 vs 1890."""
+    bm, tiles, pieces = _wide_schedule(M, N, K)
+    wgs = tiles * pieces
     rounds = (wgs + 255) // 256
     fill = wgs / (rounds * 256.0)
     step = (1.85 if bm == 256 else 1.0) * (0.6 + 0.4 * fill)
-    return 12.0 + rounds * (K // 64) * step
+    merge = 0.0 if pieces == 1 else 6.0 if bm == 128 else 12.0
+    return 12.0 + rounds * (K // 64 // pieces) * step + merge
 
 
 def _dense_gemm_us(M: int, N: int, K: int) -> float:
-    """Model of the dense route for more than 128 rows of x: the dequantize pass (0.56 us per million
-    weights) plus the library GEMM at the rate it reaches for M rows of x on this part -- 0.8 PFLOP/s at
-    256 rows, 1.15 at 512, 1.38 at 1024, 1.45 at 2048, 1.5 beyond (measured / modelled, us: [14336, 4096] M =
-    256 / 1024 / 2048: 70 / 118 / 198 vs 76 / 125 / 204; lm_head M = 1024 / 2048: 1099 / 1831 vs 1079 / 1783; [4096, 14336]
-    M = 256: 80 vs 75)."""
-    rate = 0.8 if M <= 256 else 1.15 if M <= 512 else 1.38 if M <= 1024 else 1.45 if M <= 2048 else 1.5
-    return 5.0 + 0.56 * N * K / 1e6 + 2.0 * M * N * K / (rate * 1e9)
+    """Model of the dense route for more than 128 rows of x, kernel time: the dequantize pass (10 us with the gap to the
+    GEMM + 0.45 us per million weights) plus the library GEMM, 3 us + flops / rate with 1 / rate = 1 / cap(M) + 85 / t in s per PFLOP: cap
+    is the rate the library reaches for M rows of x on a full, power-limited chip (1.0 PFLOP/s at 256 rows, 1.3
+    at 512, 1.4 at 1024, 1.5 at 2048, 1.6 at 4096, 1.68 beyond, times K / (K + 512) for the start and end of the
+    k loop) and t the number of 128 x 128 output tiles (few
+    tiles leave CUs idle).  Measured (kernel trace) / modelled, us: [4096, 4096] M = 512 / 2048 / 8192: 42 / 74 / 217 vs
+    45 / 74 / 214; [1024, 4096] M = 512 / 8192: 25 / 72 vs 30 / 68; [14336, 4096] M = 512 / 2048 / 8192: 89 / 236 / 676 vs 99 /
+    227 / 684; [4096, 14336] M = 512 / 2048: 110 / 250 vs 136 / 232; lm_head M = 512 / 2048 / 8192: 788 / 1850 / 6191 vs 735 /
+    1868 / 6005."""
+    cap = 1.0 if M <= 256 else 1.3 if M <= 512 else 1.4 if M <= 1024 else 1.5 if M <= 2048 else 1.6 if M <= 4096 else 1.68
+    cap *= K / (K + 512.0)
+    t = ((M + 127) // 128) * ((N + 127) // 128)
+    per_pflop = 1.0 / cap + 85.0 / t
+    return 10.0 + 0.45 * N * K / 1e6 + 3.0 + 2.0 * M * N * K * per_pflop / 1e9
 
 
 def _fused_gemm_wins(M: int, N: int, K: int) -> bool:

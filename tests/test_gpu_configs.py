@@ -214,6 +214,41 @@ def test_lm_head_router_takes_fused_kernel(ta, oracle, weights, M):
     _check_against_oracle(y, x, qw, oracle, f"router gemm lm_head M={M}")
 
 
+# Calls with fewer tiles than CUs cut every tile into 2..8 pieces along k that meet in the workspace (two pieces: the
+# later one adds the other's partial to its registers; more: the last to publish adds all of them from memory in k
+# order).  Both tile heights, ragged M and N, nested absmax; every case is also repeated on one workspace and must
+# give the same bits every time (the sum order does not depend on which workgroup finishes last).
+@pytest.mark.parametrize("M,N,K,nested", [
+    (300, 1000, 2048, False),    # 128-row tile, 12 tiles x 2 pieces, ragged M and N
+    (512, 4096, 4096, False),    # 128-row tile, 64 tiles x 4 pieces
+    (256, 1024, 8192, False),    # 128-row tile, 8 tiles x 8 pieces
+    (1024, 4096, 4096, True),    # 128-row tile, 128 tiles x 2 pieces, nested absmax
+    (2048, 4096, 14336, False),  # 256-row tile, 128 tiles x 2 pieces
+    (512, 8192, 28672, False),   # 256-row tile, 64 tiles x 4 pieces
+    (130, 264, 2048 + 64, False),  # 33 k steps: one quantum per k step
+])
+def test_fused_gemm_cut_up_tiles(ta, oracle, M, N, K, nested):
+    print(f"cut-up tiles M={M} [{N},{K}] nested={nested}", flush=True)
+    lib = ta._lib.load()
+    assert lib.nf4hip_gemm_workspace_bytes(M, N, K) > 65536 * 4, "this shape is expected to cut its tiles"
+    qw = QuantizedWeight(ta, N, K, 4242 + M, nested=nested)
+    x = _cpu_acts(M, K, 4243 + N).to(DEV)
+    out_g = Guarded(M * N * 2)
+    _call_matmul(ta, "gemm", x, qw, out_g, M)
+    first = out_g.view(torch.int16, (M, N)).clone()
+    _check_against_oracle(out_g.view(torch.bfloat16, (M, N)), x, qw, oracle, f"nf4hip_gemm cut up [{N},{K}] M={M}")
+    # the ABI insists on the workspace it asked for
+    L = ta._lib
+    if not nested:
+        rc = lib.nf4hip_gemm(x.data_ptr(), L.BF16, M, qw.packed.data_ptr(), qw.absmax.data_ptr(), qw.code.data_ptr(), None, N, K, 64,
+                             out_g.ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+        assert rc == L.E_WORKSPACE
+    for rep in range(4):
+        out_g.body.fill_(0)
+        _call_matmul(ta, "gemm", x, qw, out_g, M)
+        assert torch.equal(out_g.view(torch.int16, (M, N)), first), f"repeat {rep} differs"
+
+
 # ------------------------------------------------------------------------------------------------
 # Llama-3-70B shapes, nested absmax, M in {1, 16, 2048}
 # ------------------------------------------------------------------------------------------------

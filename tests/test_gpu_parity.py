@@ -283,7 +283,7 @@ def fused_gemm(ta, monkeypatch):
     monkeypatch.setattr(ta.functional, "_chunked_gemv_wins", lambda M, N, K: False)
 
 
-@pytest.mark.parametrize("M,N,K", [(200, 128, 4096), (512, 1024, 4096), (2048, 4096, 4096)])
+@pytest.mark.parametrize("M,N,K", [(200, 128, 4096), (129, 1024, 4096), (3000, 1024, 4096)])
 def test_dense_route(ta, oracle, M, N, K):
     """Default route for many rows of x: nf4hip_dequantize + dense GEMM."""
     _sync_print(f"dequant+gemm M={M} N={N} K={K}")

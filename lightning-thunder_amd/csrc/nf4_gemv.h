@@ -10,15 +10,17 @@ constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_TABLE_BYTES = 256 * 256;     // 256 byte values x 64 lanes x 4 B
 constexpr int GEMV_COUNTER_BYTES = (int)GEMV_COUNTER_REGION_BYTES;  // split-K arrival counters at the head of the workspace
 
-// Byte -> (bf16, bf16) table at the start of LDS.  Entry b holds the code values of the two
-// nibbles of b as bf16, the high nibble (even element) in the low half.  It is replicated for the
+// Byte -> (16-bit float, 16-bit float) table at the start of LDS.  Entry b holds the code values of the two
+// nibbles of b, the high nibble (even element) in the low half, as bf16 (F16 = false) or as fp16 (F16 = true:
+// the code book is then exact to 2^-12 instead of 2^-9, see F16Scale).  It is replicated for the
 // 64 lanes with a 256-byte stride: lane l reads byte address (b << 8) | (l * 4), so every lane
 // owns one bank column and a lookup is conflict-free whatever the data.
 // `lut_lane` is lut16[lane & 15], loaded by the caller (early, so that its latency is hidden).
+template <bool F16 = false>
 __device__ __forceinline__ void build_pair_table(uint8_t* smem, float lut_lane, int lane, int wave) {
     // Every entry is one dword replicated over a 256-byte row.  Sixteen lanes write one row with
     // 16-byte stores, so a wave writes four entries per instruction and its 32 entries in eight.
-    const uint32_t lb = f32_to_bf16_bits(lut_lane);
+    const uint32_t lb = F16 ? (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lut_lane) : f32_to_bf16_bits(lut_lane);
     uint4* table = reinterpret_cast<uint4*>(smem);
     const int sub = lane >> 4;
 #pragma unroll
@@ -31,6 +33,41 @@ __device__ __forceinline__ void build_pair_table(uint8_t* smem, float lut_lane, 
         const uint32_t v = first | (second << 16);
         table[e * 16 + (lane & 15)] = make_uint4(v, v, v, v);
     }
+}
+
+// The decode kernels for up to eight rows of x multiply on the matrix pipe in fp16: code-book values rounded to
+// fp16 (11 significant bits) times x.  A lane converts the bf16 values of x it holds once, when it loads them.  A
+// bf16 value is exactly representable in fp16 unless it lies outside fp16's range, so the lane first scales its
+// values by the power of two that puts the largest of them into [2^14, 2^15) and multiplies its partial sums by the
+// inverse afterwards -- both exact in fp32.  Values 2^28 times smaller than the lane's largest lose bits or vanish;
+// their share of the sum is below fp32's resolution of it.
+struct F16Scale {
+    float to_f16;    // multiply x by this before the conversion
+    float from_f16;  // multiply the sums by this
+};
+// `mx`: the largest of the lane's |x| as fp32 bits (bf16 bits << 16)
+__device__ __forceinline__ F16Scale f16_scale_for(uint32_t mx) {
+    // biased exponent e of the largest value: scale by 2^(14 - (e - 127)), at most by 2^126 (largest values below
+    // 2^-112, an all-zero lane)
+    const uint32_t ebits = max(mx >> 23, 141u - 126u);
+    F16Scale s;
+    s.to_f16 = __uint_as_float((268u - ebits) << 23);
+    s.from_f16 = __uint_as_float((ebits - 14u) << 23);
+    return s;
+}
+// running maximum of |x| over bf16 pairs, both halves at once (one v_and, one v_pk_max_u16 per dword) ...
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u16x2_t absmax_of_bf16_pair(uint32_t v, u16x2_t mx) {
+    return __builtin_elementwise_max(mx, __builtin_bit_cast(u16x2_t, v & 0x7fff7fffu));
+}
+// ... and the larger half as fp32 bits
+__device__ __forceinline__ uint32_t absmax_bits(u16x2_t mx) { return (uint32_t)max(mx.x, mx.y) << 16; }
+// two bf16 in a dword -> the same two values times `scale` as fp16 in a dword
+__device__ __forceinline__ uint32_t bf16_pair_to_f16(uint32_t v, float scale) {
+    typedef __fp16 fp16x2_t __attribute__((ext_vector_type(2)));
+    const float lo = __fmul_rn(__uint_as_float(v << 16), scale), hi = __fmul_rn(__uint_as_float(v & 0xffff0000u), scale);
+    const fp16x2_t h = __builtin_amdgcn_cvt_pkrtz(lo, hi);
+    return __builtin_bit_cast(uint32_t, h);
 }
 
 // fp32 variant of the table for the exact kernels: entry b = (lut[b >> 4], lut[b & 15]) as two
@@ -51,12 +88,20 @@ __device__ __forceinline__ void build_pair_table_f32(uint8_t* smem, float lut_la
 }
 
 // K beyond which the decode kernels reproduce the reference's per-weight bf16 rounding exactly.  The cheaper
-// arithmetic (bf16(lut) * x on the matrix pipe, block sums scaled by absmax) differs from bf16(lut * absmax) * x by
-// two independent bf16 roundings per weight, so its distance from the reference grows like sqrt(K): measured
-// sigma 0.0027 / 0.0038 / 0.0047 at K = 4096 / 8192 / 14336 for N(0, 1) activations and N(0, 0.02) weights.  At K = 14336
-// the 2e-2 tolerance is 4.2 sigma and about one output in 40 000 crosses it (seen at [4096, 14336], M = 16), at
-// K = 8192 it is 5.2 sigma (one in five million).
-__host__ __device__ constexpr bool gemv_wants_exact(int64_t K) { return K > 8192; }
+// arithmetic (rounded code-book value * x on the matrix pipe, block sums scaled by absmax) differs from
+// bf16(lut * absmax) * x by the reference's own bf16 rounding of every weight and, where the code book is held in
+// bf16 (the tile kernel), by a second, independent one; its distance from the reference grows like sqrt(K).
+// Measured sigma for N(0, 1) activations and N(0, 0.02) weights, bf16 code book: 0.0027 / 0.0038 / 0.0047 at K = 4096 /
+// 8192 / 14336 -- at K = 14336 the 2e-2 tolerance is 4.2 sigma and about one output in 40 000 crosses it (seen at
+// [4096, 14336], M = 16), at K = 8192 it is 5.2 sigma (one in five million).  fp16 code book (row and quad kernels):
+// 0.0036 at K = 14336 and no output in a million beyond 0.73 of the tolerance; 0.0038 at K = 16384.
+// The kernels therefore come in up to three arithmetic modes, chosen from K: bf16 code book up to K = 8192 (x is
+// used as it is loaded), fp16 code book up to 16384 where the kernel has one (x converted once per lane: a few
+// hundred VALU instructions per wave, which only longer rows repay), exact beyond.
+enum : int { ARITH_BF16 = 0, ARITH_F16 = 1, ARITH_EXACT = 2 };
+__host__ __device__ constexpr int gemv_arith_mode(int64_t K, bool has_f16_mode) {
+    return K <= 8192 ? ARITH_BF16 : (has_f16_mode && K <= 16384) ? ARITH_F16 : ARITH_EXACT;
+}
 
 // Read one table entry.  `addr` is an absolute LDS byte address: the table sits at LDS offset 0
 // (the gemv kernels have no static __shared__ data, so their dynamic segment starts there), which

@@ -38,6 +38,7 @@ namespace nf4 {
 namespace {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -91,8 +92,9 @@ __device__ __forceinline__ float reduce_rows(const float t[4], int lane) {
     return y;
 }
 
-template <int CPW, int U, int XS, bool NESTED, bool EXACT>
+template <int CPW, int U, int XS, bool NESTED, int MODE>
 __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a, QuadPlan p) {
+    constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -121,6 +123,9 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
     const int ks = (int)blockIdx.x % p.splits;
     const int64_t kw0 = (int64_t)(ks * p.waves_k + cw) * (CPW * LOAD_K);
     uint32_t xr[XS][CPW][16];  // x rows `ri`, `ri + 4`, ...: this lane's 32 k of every load
+    float unscale[XS];         // fp16 arithmetic: what undoes the scaling of the lane's x values
+#pragma unroll
+    for (int h = 0; h < XS; ++h) unscale[h] = 1.0f;
 
     auto run_task = [&](const int task, auto first_tag) {
         constexpr bool FIRST = decltype(first_tag)::value;
@@ -199,7 +204,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
             if (EXACT)
                 build_pair_table_f32(smem, lut, lane, wave);
             else
-                build_pair_table(smem, lut, lane, wave);
+                build_pair_table<F16>(smem, lut, lane, wave);
             if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
         }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
@@ -225,6 +230,22 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
 #pragma unroll
                         for (int d = 0; d < 4; ++d) xr[h][c][4 * j + d] = v[j][d];
                 }
+            if (F16) {  // the lane's x values become fp16, scaled into range per row of x
+#pragma unroll
+                for (int h = 0; h < XS; ++h) {
+                    u16x2_t mx = {0, 0};
+#pragma unroll
+                    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+                        for (int q = 0; q < 16; ++q) mx = absmax_of_bf16_pair(xr[h][c][q], mx);
+                    const F16Scale fs = f16_scale_for(absmax_bits(mx));
+#pragma unroll
+                    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+                        for (int q = 0; q < 16; ++q) xr[h][c][q] = bf16_pair_to_f16(xr[h][c][q], fs.to_f16);
+                    unscale[h] = fs.from_f16;
+                }
+            }
         }
 
         for (int i0 = 0; i0 < cnt; i0 += U) {
@@ -275,8 +296,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                         for (int t = 0; t < 8; ++t) {
                             const uint2 wa = make_uint2(pr[2 * t], pr[2 * t + 1]);
                             const uint2 xb = make_uint2(xr[h][c][2 * t], xr[h][c][2 * t + 1]);
-                            acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
-                                                                         __builtin_bit_cast(s16x4, xb), acc, 0, 0, 0);
+                            if (!F16)
+                                acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
+                                                                             __builtin_bit_cast(s16x4, xb), acc, 0, 0, 0);
+                            else
+                                acc = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, wa),
+                                                                         __builtin_bit_cast(f16x4, xb), acc, 0, 0, 0);
                         }
                         if (EXACT) {
 #pragma unroll
@@ -293,6 +318,10 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 const int grow = 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);
 #pragma unroll
                 for (int h = 0; h < XS; ++h) {
+                    if (F16) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) tot[h][i] *= unscale[h];
+                    }
                     // lanes 0..15: row 2*b3+b2 of the group, x row 4h + ri
                     const float total = reduce_rows(tot[h], lane);
                     if (lane < 16 && 4 * h + ri < M && i < cnt)
@@ -400,10 +429,13 @@ QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
 
 template <int CPW, int U, int XS, bool NESTED>
 hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
-    if (gemv_wants_exact(a.K))
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, true>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    const int mode = gemv_arith_mode(a.K, true);
+    if (mode == ARITH_EXACT)
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    else if (mode == ARITH_F16)
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, false>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
@@ -428,10 +460,12 @@ hipError_t launch_n(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_
 template <int CPW, int U, int XS>
 hipError_t allow_lds_cu() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, true>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, true>, SMEM_BYTES);
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, ARITH_EXACT>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, ARITH_EXACT>, SMEM_BYTES);
 }
 
 }  // namespace

@@ -38,6 +38,7 @@ namespace nf4 {
 namespace {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -96,11 +97,13 @@ __device__ __forceinline__ float reduce8(const float v[8], int lane) {
 // pair, bit 2 the second half
 __device__ __forceinline__ int reduce8_id(int lane) { return (lane & 1) | ((lane & 2) ? 2 : 0) | ((lane & 4) ? 4 : 0); }
 
-// EXACT = false: the table holds bf16(lut) pairs and absmax scales the 32-weight partial sum.
-// EXACT = true : the table holds fp32 lut pairs and every weight is rounded like the reference's
+// MODE (gemv_arith_mode): ARITH_BF16 / ARITH_F16: the table holds the code book rounded to bf16 / fp16 in pairs, x is
+//                used as bf16 / converted to fp16 per lane, and absmax scales the 32-weight partial sum.
+//                ARITH_EXACT: the table holds fp32 pairs and every weight is rounded like the reference's
 //                dequantisation, bf16(lut * absmax), before it is multiplied (more VALU work).
-template <int M, int U, bool NESTED, bool EXACT>
+template <int M, int U, bool NESTED, int MODE>
 __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a, RowsPlan p) {
+    constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -143,7 +146,6 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                 if (lane_on) v = *reinterpret_cast<const uint4*>(a.x + m * K + kchunk + klane + 8 * q);
                 xr[m][4 * q + 0] = v.x; xr[m][4 * q + 1] = v.y; xr[m][4 * q + 2] = v.z; xr[m][4 * q + 3] = v.w;
             }
-
         // sq: absmax of the lane's block; nested: its 8-bit code (resolved through the LDS copy of
         // the map when the slot is consumed, so that issuing a load never waits for another) and
         // s2 the second-level absmax
@@ -184,11 +186,29 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
             if (EXACT)
                 build_pair_table_f32(smem, lut_mine, lane, wave);
             else
-                build_pair_table(smem, lut_mine, lane, wave);
+                build_pair_table<F16>(smem, lut_mine, lane, wave);
             if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
             table_built = true;
         }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
+
+        // fp16 arithmetic: the lane's x values become fp16, scaled into range per row of x (here, behind the requests for
+        // the first weights, so that the conversion runs while they are under way)
+        float unscale[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            unscale[m] = 1.0f;
+            if (F16) {
+                u16x2_t mx = {0, 0};
+#pragma unroll
+                for (int q = 0; q < 16; ++q) mx = absmax_of_bf16_pair(xr[m][q], mx);
+                const F16Scale fs = f16_scale_for(absmax_bits(mx));
+#pragma unroll
+                for (int q = 0; q < 16; ++q) xr[m][q] = bf16_pair_to_f16(xr[m][q], fs.to_f16);
+                unscale[m] = fs.from_f16;
+            }
+        }
+
 
         if (cnt > 0) {
             for (int i0 = 0; i0 < cnt; i0 += U) {
@@ -229,14 +249,18 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                         for (int t = 0; t < 8; ++t) {
                             const uint2 wa = make_uint2(pr[2 * t], pr[2 * t + 1]);
                             const uint2 xb = make_uint2(xr[m][2 * t], xr[m][2 * t + 1]);
-                            c = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
-                                                                       __builtin_bit_cast(s16x4, xb), c, 0, 0, 0);
+                            if (!F16)
+                                c = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, wa),
+                                                                           __builtin_bit_cast(s16x4, xb), c, 0, 0, 0);
+                            else
+                                c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, wa),
+                                                                       __builtin_bit_cast(f16x4, xb), c, 0, 0, 0);
                         }
                         // diagonal element of this lane's 4x4 block
                         const float c01 = (lane & 1) ? c[1] : c[0];
                         const float c23 = (lane & 1) ? c[3] : c[2];
                         const float diag = (lane & 2) ? c23 : c01;
-                        res[u * M + m] = EXACT ? diag : diag * s;
+                        res[u * M + m] = EXACT ? diag : diag * (s * unscale[m]);
                     }
                 }
                 // reduce the U*M per-lane results over the wave, 8 at a time
@@ -338,10 +362,13 @@ RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
 
 template <int M, int U, bool NESTED>
 hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
-    if (gemv_wants_exact(a.K))
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, true>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    const int mode = gemv_arith_mode(a.K, true);
+    if (mode == ARITH_EXACT)
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+    else if (mode == ARITH_F16)
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, false>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
@@ -366,10 +393,12 @@ hipError_t launch_n(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_
 template <int M, int U>
 hipError_t allow_lds_mu() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, true, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, true>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_rows_kernel<M, U, true, true>, SMEM_BYTES);
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, true, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, true, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, ARITH_EXACT>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_rows_kernel<M, U, true, ARITH_EXACT>, SMEM_BYTES);
 }
 
 template <int M>

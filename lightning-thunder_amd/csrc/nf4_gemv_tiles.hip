@@ -770,7 +770,7 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
     const int n = rows_held(a.M) == 8 ? list_length<10>(G, nsl, last) : list_length<5>(G, nsl, last);
     if (n > ITEMS_MAX) return hipErrorInvalidValue;
     const bool steady = n >= STEADY_MIN_ITEMS;
-    if (gemv_wants_exact(a.K))
+    if (gemv_arith_mode(a.K, false) == ARITH_EXACT)
         return rows_held(a.M) == 8 ? launch_r<8, true>(a, p, grid, steady, stream)
                                    : launch_r<16, true>(a, p, grid, steady, stream);
     return rows_held(a.M) == 8 ? launch_r<8, false>(a, p, grid, steady, stream)

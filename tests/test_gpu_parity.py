@@ -216,6 +216,45 @@ def test_gemv_shapes(ta, oracle, N, K, M):
     _matmul_case(ta, oracle, M, N, K, seed=N + K + M)
 
 
+@pytest.mark.parametrize("K", [2048, 10240])
+@pytest.mark.parametrize("M", [1, 2, 4, 8])
+def test_gemv_x_outside_fp16_range(ta, oracle, M, K):
+    """For 8192 < K <= 16384 the row and quad kernels multiply in fp16 after scaling each lane's x values into
+    range (K = 10240; K = 2048 takes the bf16 arithmetic): rows of x far above fp16's largest value, far below its
+    smallest, of mixed magnitudes, and with the largest finite bf16."""
+    _sync_print(f"gemv x outside the fp16 range M={M} K={K}")
+    N = 192
+    w = _weights((N, K), seed=77)
+    qw, absmax = oracle.C().quantize(w, 64)
+    lut = oracle.nf4_lut()
+    base = _acts((M, K), seed=78 + M).float()
+    scales = [1e6, 2.0**100, 2.0**-60, 70000.0]
+    for case in range(5):
+        x = base.clone()
+        if case < 4:
+            x *= scales[case]
+        else:  # one huge value per row among ordinary ones, and the largest finite bf16 in row 0
+            x[:, 5::211] *= 1e8
+            x[0, 1000] = 3.3895313892515355e38
+        x = x.to(torch.bfloat16)
+        y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None, absmax.to(DEV), lut.to(DEV), 64, torch.bfloat16, (N, K))
+        ref = oracle.matmul_4bit_f64(x, qw, None, absmax, lut, 64, torch.float32, (N, K)).double()
+        got = y.cpu().double()
+        assert bool(torch.isfinite(got).all()), f"case {case}: non-finite output"
+        # the tolerance of the matmul, scaled with the magnitude of each row of x
+        mag = x.double().abs().amax(dim=1, keepdim=True).clamp_min(1e-300)
+        typical = x.double().pow(2).mean(dim=1, keepdim=True).sqrt()
+        tol = 2e-2 * typical + 2e-2 * ref.abs() + 1e-6 * mag
+        assert bool(((got - ref).abs() <= tol).all()), f"case {case}: max excess {((got - ref).abs() - tol).max().item():.3g}"
+    # infinities and NaNs in x reach the outputs of their row
+    x = base.clone().to(torch.bfloat16)
+    x[0, 3] = float("inf")
+    y = ta.matmul_nf4(x.to(DEV), qw.to(DEV), None, absmax.to(DEV), lut.to(DEV), 64, torch.bfloat16, (N, K)).cpu()
+    assert not bool(torch.isfinite(y[0].float()).any())
+    if M > 1:
+        assert bool(torch.isfinite(y[1:].float()).all())
+
+
 @pytest.mark.parametrize("blocksize", [128, 512, 4096])
 @pytest.mark.parametrize("M", [3, 7])
 def test_gemv_blocksizes(ta, oracle, blocksize, M):

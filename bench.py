@@ -251,16 +251,20 @@ MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CUs x 2.4 GHz x 4096 flop/clk/CU
 
 
 def _timed(torch, fn, reps, warm=3):
+    """Seconds per call: the median of three event-bracketed batches of ``reps`` calls after ``warm`` untimed ones."""
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / reps
+    per = []
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        per.append(e0.elapsed_time(e1) * 1e-3 / reps)
+    return sorted(per)[1]
 
 
 def _cpu_seeded(torch, shape, seed, std):
@@ -350,7 +354,7 @@ def double_quant_section(torch, ta) -> dict:
         nested_bytes = n // BLOCKSIZE + 4 * -(-(n // BLOCKSIZE) // 256) + 1024 + 4
         for mi, M in enumerate((1, 16, 2048)):
             x = _cpu_seeded(torch, (M, K), 500000 + 100 * si + mi, 1.0).to(dev)
-            route = F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))
+            route = F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K), nested=True)
             it = [0]
             out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
 

@@ -17,6 +17,9 @@
  *     queued on `stream` has finished.  Outputs are caller-allocated.
  *   - `stream` is a hipStream_t (NULL = the default stream).  Nothing here synchronises the
  *     device, allocates or frees memory, or blocks the host.
+ *   - Alignment (else NF4HIP_E_ALIGN): tensors that the kernels read or write in 128-bit pieces -- x, w, packed,
+ *     absmax, absmax_q, absmax2, out, workspace -- must be 16-byte aligned; the small tables read element by
+ *     element need their natural alignment only: lut16 and map256 4 bytes, bias 2 bytes.
  *   - dtype codes: NF4HIP_BF16 = 0, NF4HIP_F16 = 1, NF4HIP_F32 = 2.
  *   - Weight layout: the [N, K] weight is flattened row-major into n = N*K elements; quantisation
  *     blocks are `blocksize` consecutive elements of that flat view.  `packed` holds two 4-bit
@@ -44,7 +47,7 @@ extern "C" {
 #define NF4HIP_E_DTYPE (-2)     /* dtype code unknown or unsupported by this entry point */
 #define NF4HIP_E_BLOCKSIZE (-3) /* blocksize not one of 64,128,256,512,1024,2048,4096 */
 #define NF4HIP_E_SHAPE (-4)     /* a size is negative/zero where it may not be, or violates a fast-path rule */
-#define NF4HIP_E_ALIGN (-5)     /* a pointer is not 16-byte aligned */
+#define NF4HIP_E_ALIGN (-5)     /* a pointer is not aligned as the rules above ask */
 #define NF4HIP_E_WORKSPACE (-6) /* workspace missing or smaller than nf4hip_*_workspace_bytes() */
 #define NF4HIP_E_HIP (-7)       /* a HIP runtime call failed; text in nf4hip_last_error() */
 

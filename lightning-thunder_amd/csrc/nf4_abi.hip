@@ -63,6 +63,7 @@ int hip_fail(const char* what, hipError_t e) {
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 // log2 of a supported blocksize, or -1
 int block_log2(int blocksize) {
@@ -85,8 +86,8 @@ int check_nested(const uint8_t* absmax_q, const float* absmax2, const float* map
     if (!absmax_q || !absmax2 || !map256) return fail(NF4HIP_E_NULL, "nested absmax: null pointer");
     *nested_log2 = block_log2(nested_blocksize);
     if (*nested_log2 < 0) return fail(NF4HIP_E_BLOCKSIZE, "nested_blocksize %d unsupported", nested_blocksize);
-    if (!aligned16(absmax_q) || !aligned16(absmax2) || !aligned16(map256))
-        return fail(NF4HIP_E_ALIGN, "nested absmax: pointer not 16-byte aligned");
+    if (!aligned16(absmax_q) || !aligned16(absmax2) || !aligned4(map256))
+        return fail(NF4HIP_E_ALIGN, "nested absmax: absmax_q / absmax2 not 16-byte aligned or map256 not 4-byte aligned");
     return NF4HIP_OK;
 }
 
@@ -120,8 +121,9 @@ int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const 
     if (!(kind == GEMV && M <= 4) && K % blocksize)
         return fail(NF4HIP_E_SHAPE, "%s: blocksize %d does not divide K = %lld", name, blocksize, (long long)K);
     if (!aligned16(x) || !aligned16(packed) || !aligned16(out) || (absmax && !aligned16(absmax)) ||
-        (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
-        return fail(NF4HIP_E_ALIGN, "%s: pointer not 16-byte aligned", name);
+        (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) || !aligned4(lut16))
+        return fail(NF4HIP_E_ALIGN, "%s: x / packed / absmax / out not 16-byte aligned, lut16 not 4-byte or bias not 2-byte aligned",
+                    name);
     const size_t need = kind == GEMV ? nf4::gemv_workspace_bytes(M, N, K) : nf4::gemm_workspace_bytes(M, N, K);
     if (use_static) {
         if (need > (size_t)NF4HIP_STATIC_SCRATCH_BYTES)
@@ -192,8 +194,8 @@ int nf4hip_dequantize(const uint8_t* packed, const float* absmax, const float* l
     if (bl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dequantize: blocksize %d unsupported", blocksize);
     if (n == 0) return NF4HIP_OK;
     if (!packed || !absmax || !lut16 || !out) return fail(NF4HIP_E_NULL, "nf4hip_dequantize: null pointer");
-    if (!aligned16(packed) || !aligned16(absmax) || !aligned16(out))
-        return fail(NF4HIP_E_ALIGN, "nf4hip_dequantize: pointer not 16-byte aligned");
+    if (!aligned16(packed) || !aligned16(absmax) || !aligned16(out) || !aligned4(lut16))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_dequantize: packed / absmax / out not 16-byte aligned or lut16 not 4-byte aligned");
     const nf4::NestedAbsmax none{nullptr, nullptr, nullptr, 0.0f, 0};
     const hipError_t e =
         nf4::launch_dequantize(packed, absmax, none, lut16, n, bl, out, out_dtype, static_cast<hipStream_t>(stream));
@@ -208,6 +210,8 @@ int nf4hip_dq_compress(const float* absmax, int64_t nblocks, int nested_blocksiz
     if (nl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dq_compress: nested_blocksize %d unsupported", nested_blocksize);
     if (nblocks == 0) return NF4HIP_OK;
     if (!absmax || !map256 || !absmax_q || !absmax2) return fail(NF4HIP_E_NULL, "nf4hip_dq_compress: null pointer");
+    if (!aligned16(absmax) || !aligned16(absmax_q) || !aligned16(absmax2) || !aligned4(map256))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_dq_compress: absmax / absmax_q / absmax2 not 16-byte aligned or map256 not 4-byte aligned");
     const hipError_t e =
         nf4::launch_dq_compress(absmax, nblocks, nl, map256, offset, absmax_q, absmax2, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail("nf4hip_dq_compress", e);
@@ -222,6 +226,8 @@ int nf4hip_dq_reconstruct(const uint8_t* absmax_q, const float* absmax2, const f
         return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_dq_reconstruct: nested_blocksize %d unsupported", nested_blocksize);
     if (nblocks == 0) return NF4HIP_OK;
     if (!absmax_q || !absmax2 || !map256 || !absmax) return fail(NF4HIP_E_NULL, "nf4hip_dq_reconstruct: null pointer");
+    if (!aligned16(absmax) || !aligned16(absmax_q) || !aligned16(absmax2) || !aligned4(map256))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_dq_reconstruct: absmax / absmax_q / absmax2 not 16-byte aligned or map256 not 4-byte aligned");
     const nf4::NestedAbsmax nq{absmax_q, absmax2, map256, offset, nl};
     const hipError_t e = nf4::launch_dq_reconstruct(nq, nblocks, absmax, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail("nf4hip_dq_reconstruct", e);
@@ -240,8 +246,8 @@ int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const f
     int nl = 0;
     const int rc = check_nested(absmax_q, absmax2, map256, nested_blocksize, &nl);
     if (rc) return rc;
-    if (!aligned16(packed) || !aligned16(out))
-        return fail(NF4HIP_E_ALIGN, "nf4hip_dequantize_dq: pointer not 16-byte aligned");
+    if (!aligned16(packed) || !aligned16(out) || !aligned4(lut16))
+        return fail(NF4HIP_E_ALIGN, "nf4hip_dequantize_dq: packed / out not 16-byte aligned or lut16 not 4-byte aligned");
     const nf4::NestedAbsmax nq{absmax_q, absmax2, map256, offset, nl};
     const hipError_t e =
         nf4::launch_dequantize(packed, nullptr, nq, lut16, n, bl, out, out_dtype, static_cast<hipStream_t>(stream));

@@ -400,7 +400,7 @@ def _dense_gemm_us(M: int, N: int, K: int) -> float:
     return 10.0 + 0.45 * N * K / 1e6 + 3.0 + 2.0 * M * N * K * per_pflop / 1e9
 
 
-def _fused_gemm_wins(M: int, N: int, K: int) -> bool:
+def _fused_gemm_wins(M: int, N: int, K: int, nested: bool = False) -> bool:
     """Is the fused GEMM kernel faster than dequantize + dense GEMM?  Both sides are modelled from
     measurements on MI355X.  Up to 128 rows of x (one tile of x rows, K split over workgroups) the fused kernel's
     time hardly depends on N while the chip is not full, the dense route's grows with the weight (M = 64, us:
@@ -413,7 +413,9 @@ def _fused_gemm_wins(M: int, N: int, K: int) -> bool:
     which needs no transient bf16 weight."""
     if M <= 128:
         return _fused_gemm_us(M, N, K) < _dense_route_us(N, K)
-    return _wide_gemm_us(M, N, K) <= 1.03 * _dense_gemm_us(M, N, K)
+    # nested absmax: the fused kernel resolves an 8-bit code through two more look-ups per block and k step and runs
+    # 15-30 % longer ([8192, 8192] 2048 rows: 275 vs 235 us; [8192, 28672]: 1045 vs 784), the dequantize pass hardly does
+    return _wide_gemm_us(M, N, K) * (1.25 if nested else 1.0) <= 1.03 * _dense_gemm_us(M, N, K)
 
 
 def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
@@ -435,7 +437,7 @@ def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
     return t < 0.8 * _dense_route_us(N, K)
 
 
-def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape) -> str:
+def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape, nested: bool = False) -> str:
     """Which kernel serves this call: ``"gemv"``, ``"gemv-chunks"`` (the decode kernel once per 16
     rows of x), ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP
     dequantize, then the dense library GEMM, because that is the faster of the two for many rows
@@ -465,7 +467,7 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
     if K % 512 == 0 and _chunked_gemv_wins(M, N, K):
         return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
-    if _fused_gemm_wins(M, N, K):
+    if _fused_gemm_wins(M, N, K, nested):
         return "gemm"  # expanding the weight tiles in registers beats writing the bf16 weight out
     # the fused GEMM kernel streams K sequentially per tile: beyond LONG_K even a few rows of x are
     # served faster by dequantize + dense GEMM
@@ -481,7 +483,7 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
     N, K = shape
     assert x.shape[-1] == K, f"{x.shape=}, rhs {shape=}"
     _require_gpu(x, qweight, quant_map, bias)
-    route = fused_route(x, bias, blocksize, dtype, shape)
+    route = fused_route(x, bias, blocksize, dtype, shape, isinstance(absmax, NestedAbsmax))
     if route in ("dequant+linear", "dequant+gemm"):
         w = dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape).to(x.dtype)
         return torch.nn.functional.linear(x, w, bias)

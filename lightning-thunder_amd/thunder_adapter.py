@@ -24,6 +24,7 @@ from types import SimpleNamespace
 import torch
 
 from . import functional
+from .transforms import quantization
 
 EXECUTOR_NAME = "quant_hip_nf4"
 
@@ -44,7 +45,8 @@ def install():
             assert x.shape[-1] == shape[1], f"{x.shape=}, rhs {shape=}"
             return thunder.TensorProxy(like=x, shape=(*x.shape[:-1], shape[0]))
 
-        ex.register_operator("hip_matmul_nf4", meta=hip_matmul_nf4_meta, fn=functional.matmul_nf4)
+        # resolved at call time, so that whoever replaces functional.matmul_nf4 (a test's stand-in) is honoured
+        ex.register_operator("hip_matmul_nf4", meta=hip_matmul_nf4_meta, fn=lambda *args: functional.matmul_nf4(*args))
         thunder.extend.register_executor(ex)
     hip_matmul_nf4 = ex.opmap["hip_matmul_nf4"]
 
@@ -58,11 +60,14 @@ def install():
             self.blocksize = blocksize
 
         def quantize_weight(self, w):
+            # the reference's device policy (quantization.py:53-63): meta stands for zeros on the GPU, a weight
+            # elsewhere is copied there, a GPU weight is used where it is
+            work = torch.device(quantization.WORK_DEVICE)
             if w.device.type == "meta":
-                w_work = torch.zeros_like(w, device="cuda")
-            elif w.device.type != "cuda":
+                w_work = torch.zeros_like(w, device=work)
+            elif w.device.type != work.type:
                 with torch.no_grad():
-                    w_work = w.to("cuda")
+                    w_work = w.to(work)
             else:
                 w_work = w
             qw, absmax, code = functional.quantize_nf4(w_work, self.blocksize)

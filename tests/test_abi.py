@@ -78,6 +78,12 @@ def test_matmul_argument_errors(ta):
     assert "512" in _err(ta)
     assert gemm(K=100) == L.E_SHAPE and gemm(K=192, bs=128) == L.E_SHAPE
     assert gemv(x=A + 4) == L.E_ALIGN and gemm(packed=A + 1) == L.E_ALIGN and gemv(bias=A + 1) == L.E_ALIGN
+    assert gemv(lut=A + 2) == L.E_ALIGN
+    # the small tables need their natural alignment only: these calls get past the alignment check (and stop at the next one)
+    assert gemv(lut=A + 4, w=None) == L.E_WORKSPACE and gemv(bias=A + 2, w=None) == L.E_WORKSPACE
+    assert lib.nf4hip_dq_compress(A + 4, 512, 256, A, 0.0, A, A, None) == L.E_ALIGN
+    assert lib.nf4hip_dq_reconstruct(A, A + 8, A, 0.0, 512, 256, A, None) == L.E_ALIGN
+    assert lib.nf4hip_dq_compress(A, 512, 256, A + 2, 0.0, A, A, None) == L.E_ALIGN
     assert gemv(w=None) == L.E_WORKSPACE and gemv(wb=16) == L.E_WORKSPACE
     assert "workspace" in _err(ta)
     # the entry point that brings its own scratch: same checks, and a shape whose partial sums exceed the

@@ -314,6 +314,49 @@ def test_gemv_repeatable_and_workspace_reuse(ta, oracle):
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
+def test_split_k_hand_off_holds_over_many_launches(ta):
+    """2000 launches on ONE workspace, alternating between four calls whose partial sums cross workgroups (decode
+    tile kernel with K split eight ways, row kernel with a long K, fused GEMM with K split, fused GEMM with cut-up
+    tiles): every result must equal the first of its kind bit for bit and every arrival counter must be back at
+    zero.  The comparison runs on the device; the host looks at the verdict every 100 launches and stops at the
+    first mismatch."""
+    _sync_print("split-K hand-off, 2000 launches on one workspace")
+    L, lib = ta._lib, ta._lib.load()
+    code = ta.nf4_code(DEV)
+    g = torch.Generator(device=DEV).manual_seed(7)
+    calls = []
+    for kind, M, N, K in [("gemv", 16, 4096, 4096), ("gemv", 1, 512, 32768), ("gemm", 64, 1024, 4096), ("gemm", 512, 1024, 4096)]:
+        n = N * K
+        packed = torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=DEV, generator=g)
+        absmax = torch.rand(n // 64, device=DEV, generator=g) * 0.05 + 0.01
+        x = torch.randn(M, K, device=DEV, generator=g).to(torch.bfloat16)
+        need = (lib.nf4hip_gemv_workspace_bytes if kind == "gemv" else lib.nf4hip_gemm_workspace_bytes)(M, N, K)
+        assert need > 65536 * 4, f"{kind} M={M} [{N},{K}] is expected to split K over workgroups"
+        calls.append((kind, M, N, K, packed, absmax, x, need, torch.empty(M, N, dtype=torch.bfloat16, device=DEV)))
+    ws = torch.zeros(max(c[7] for c in calls), dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch(c):
+        kind, M, N, K, packed, absmax, x, _, out = c
+        fn = lib.nf4hip_gemv if kind == "gemv" else lib.nf4hip_gemm
+        L.check(fn(x.data_ptr(), L.BF16, M, packed.data_ptr(), absmax.data_ptr(), code.data_ptr(), None, N, K, 64,
+                   out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+
+    first = []
+    for c in calls:
+        launch(c)
+        first.append(c[8].clone())
+    bad = torch.zeros((), dtype=torch.bool, device=DEV)
+    for it in range(2000):
+        c = calls[it % len(calls)]
+        c[8].zero_()
+        launch(c)
+        bad |= (c[8].view(torch.int16) != first[it % len(calls)].view(torch.int16)).any()
+        if it % 100 == 99:
+            assert not bool(bad), f"a result changed between launches {it - 99} and {it}"
+    assert not bool(ws[: 65536 * 4].any()), "arrival counters not back at zero"
+
+
 @pytest.fixture
 def fused_gemm(ta, monkeypatch):
     """Route every M > 16 call to the fused GEMM kernel (the default router prefers HIP dequantize

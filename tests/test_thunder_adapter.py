@@ -1,0 +1,91 @@
+"""thunder_adapter.install() against a minimal stand-in `thunder` package (tests/fake_thunder): host logic only.
+
+What a real Thunder would exercise and this cannot: tracing, the dispatch pass keeping the bound symbol, execution
+of a compiled module.  What it does check: the executor and operator are registered once and found again, the
+operator's meta function infers the output shape the way the reference's does (quantization.py:29-32), the
+transform subclass never runs the reference's bitsandbytes-importing __init__, quantize_weight follows the
+reference's device policy and returns the (qweight, state) pair the class reads, and the trace hook runs with the
+module global pointing at the HIP symbol and restores whatever was there -- also when the hook raises, and also
+when the global did not exist."""
+
+import importlib
+import os
+import sys
+import types
+
+import pytest
+import torch
+
+import fake_backend
+
+FAKE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fake_thunder")
+
+
+@pytest.fixture
+def fake_thunder():
+    saved = {k: v for k, v in sys.modules.items() if k == "thunder" or k.startswith("thunder.")}
+    for k in saved:
+        del sys.modules[k]
+    sys.path.insert(0, FAKE)
+    try:
+        yield importlib.import_module("thunder")
+    finally:
+        sys.path.remove(FAKE)
+        for k in [k for k in sys.modules if k == "thunder" or k.startswith("thunder.")]:
+            del sys.modules[k]
+        sys.modules.update(saved)
+
+
+def test_install_without_thunder_says_so(ta):
+    if importlib.util.find_spec("thunder") is not None:
+        pytest.skip("a thunder package is importable here")
+    adapter = importlib.import_module("lightning-thunder_amd.thunder_adapter")
+    with pytest.raises(ImportError, match="lightning-thunder"):
+        adapter.install()
+
+
+def test_install_on_a_stand_in_thunder(ta, fake_thunder):
+    adapter = importlib.import_module("lightning-thunder_amd.thunder_adapter")
+    ref = importlib.import_module("thunder.transforms.quantization")
+    T = adapter.install()
+    ex = fake_thunder.extend.get_executor("quant_hip_nf4")
+    assert ex is T.executor and set(ex.opmap) == {"hip_matmul_nf4"}
+    assert adapter.install().executor is ex  # a second install finds the executor, registers nothing twice
+    sym = ex.opmap["hip_matmul_nf4"]
+
+    # meta: [..., K] x weight [N, K] -> [..., N]; a wrong K is refused
+    x = types.SimpleNamespace(shape=(2, 5, 64), dtype=torch.bfloat16, device="cuda")
+    out = sym.meta(x, None, None, None, None, 64, torch.bfloat16, (48, 64))
+    assert out.shape == (2, 5, 48)
+    with pytest.raises(AssertionError):
+        sym.meta(x, None, None, None, None, 64, torch.bfloat16, (48, 32))
+
+    t = T(blocksize=128)  # must not reach the reference's __init__
+    assert issubclass(T, ref.BitsAndBytesLinearQuant4bit)
+    assert t.quant_states == {} and t.quantized_submodule_names == set() and t.blocksize == 128
+
+    with fake_backend.installed(ta):
+        w = (torch.randn(48, 256, generator=torch.Generator().manual_seed(1)) * 0.02).to(torch.bfloat16)
+        qw, state = t.quantize_weight(w)
+        assert qw.dtype == torch.uint8 and qw.numel() == 48 * 256 // 2
+        assert state.shape == (48, 256) and state.dtype == torch.bfloat16 and state.blocksize == 128
+        assert state.absmax.numel() == 48 * 256 // 128 and state.code.numel() == 16
+        qz, sz = t.quantize_weight(torch.empty(48, 256, dtype=torch.bfloat16, device="meta"))  # meta stands for zeros
+        assert qz.device.type == "cpu" and not bool(sz.absmax.any())
+        # the registered implementation is the package's matmul (here: its CPU stand-in)
+        xr = torch.randn(3, 256, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+        y = sym(xr, qw, None, state.absmax, state.code, 128, torch.bfloat16, (48, 256))
+        assert y.shape == (3, 48)
+        deq = ta.functional.dequantize_nf4(qw, state.absmax, state.code, 128, torch.bfloat16, (48, 256))
+        torch.testing.assert_close(y.float(), (xr.float() @ deq.float().t()), rtol=2e-2, atol=2e-2)
+
+    # the trace hook sees the HIP symbol under the reference's global name, and the name is restored afterwards
+    assert not hasattr(ref, "bnb_matmul_nf4")
+    _, (comp, bound), _ = t.transform_traces_pre_prologue("p", "c", "e")
+    assert comp == "c" and bound is sym and not hasattr(ref, "bnb_matmul_nf4")
+    ref.bnb_matmul_nf4 = "theirs"
+    _, (_, bound), _ = t.transform_traces_pre_prologue("p", "c", "e")
+    assert bound is sym and ref.bnb_matmul_nf4 == "theirs"
+    with pytest.raises(RuntimeError, match="trace rewrite failed"):
+        t.transform_traces_pre_prologue("p", "c", "e", fail=True)
+    assert ref.bnb_matmul_nf4 == "theirs"

@@ -1,7 +1,7 @@
 // Dispatch of the decode-shape fused NF4 dequant-matmul (M <= 16) between its three kernels:
 // row-streaming (M = 1, 2, nf4_gemv_rows.hip), four weight rows per lane quad (M = 3, 4, and
-// M = 5..8 on weights of at most 2^26 elements, nf4_gemv_quad.hip) and MFMA tiles (the rest up to
-// M = 16, nf4_gemv_tiles.hip).
+// M = 5..8 on weights of at most 2^26 elements, and M = 9..16 as two halves of x on weights of at most 2^24,
+// nf4_gemv_quad.hip) and MFMA tiles (the rest up to M = 16, nf4_gemv_tiles.hip).
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -37,12 +37,20 @@ hipError_t device_setup(int* cus_out) {
 // 8192), the tile kernel streams faster once the weights are large; they cross near 2^26 weights.
 bool quad_serves(int64_t M, int64_t N, int64_t K) { return M <= 4 || (M <= 8 && N * K <= ((int64_t)1 << 26)); }
 
+// Nine to sixteen rows of x on a small weight (up to 2^24 elements): the quad kernel on two halves of x, whose
+// start-up is shorter than the tile kernel's (measured, 16 rows: [1024, 4096] 7.6 vs 10.5 us, [4096, 4096] 10.6 vs 11.5;
+// [6144, 4096] 14.6 vs 11.9 the other way round).
+bool quad_halves_serve(int64_t M, int64_t N, int64_t K) {
+    return M > 8 && N * K <= ((int64_t)1 << 24) && gemv_quad_halves_possible(N, K);
+}
+
 }  // namespace
 
 // ---- dispatch -------------------------------------------------------------------------------
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 2) return gemv_rows_workspace_bytes(M, N, K);
+    if (quad_halves_serve(M, N, K)) return gemv_quad_workspace_bytes(8, N, K);
     return quad_serves(M, N, K) ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
 }
 
@@ -51,6 +59,7 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;
     if (a.M <= 2) return launch_gemv_rows(a, cus, stream);
+    if (quad_halves_serve(a.M, a.N, a.K)) return launch_gemv_quad_halves(a, cus, stream);
     return quad_serves(a.M, a.N, a.K) ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
 }
 

@@ -112,6 +112,14 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
 
+    // Nine to sixteen rows of x on a small weight: two workgroups per task, blockIdx.y picks rows 0..7 or 8..15 of x
+    // (the launcher only does this when K is not split across workgroups, so the halves share nothing)
+    if (gridDim.y > 1) {
+        const int mb = 8 * (int)blockIdx.y;
+        a.x += (int64_t)mb * a.K;
+        a.out += (int64_t)mb * a.N;
+        a.M = min(a.M - mb, 8);
+    }
     const int cw = wave % p.waves_k;
     const int rg = wave / p.waves_k;
     const int64_t K = a.K;
@@ -428,27 +436,28 @@ QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
 }
 
 template <int CPW, int U, int XS, bool NESTED>
-hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
+hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
     const int mode = gemv_arith_mode(a.K, true);
+    const dim3 g((unsigned)grid, (unsigned)halves);
     if (mode == ARITH_EXACT)
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else if (mode == ARITH_F16)
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
 // U = row groups in flight per wave: U * CPW 16-byte loads per lane, at most 8 (4 with eight rows of x)
 template <int CPW, int XS, bool NESTED>
-hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
+hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
     const int cnt = p.groups_per_band / p.row_groups;  // groups per wave and task
     constexpr int UMAX = 8 / (CPW * XS);
     if constexpr (UMAX >= 8)
-        if (cnt >= 8) return launch_u<CPW, 8, XS, NESTED>(a, p, grid, stream);
+        if (cnt >= 8) return launch_u<CPW, 8, XS, NESTED>(a, p, grid, stream, halves);
     if constexpr (UMAX >= 4 && !(NESTED && CPW == 2))  // nested: one more register per load in flight
-        if (cnt >= 4) return launch_u<CPW, 4, XS, NESTED>(a, p, grid, stream);
-    return launch_u<CPW, 2, XS, NESTED>(a, p, grid, stream);
+        if (cnt >= 4) return launch_u<CPW, 4, XS, NESTED>(a, p, grid, stream, halves);
+    return launch_u<CPW, 2, XS, NESTED>(a, p, grid, stream, halves);
 }
 
 template <bool NESTED>
@@ -484,6 +493,20 @@ hipError_t gemv_quad_setup() {
     if ((e = allow_lds_cu<2, 2, 1>()) != hipSuccess) return e;
     if ((e = allow_lds_cu<1, 4, 2>()) != hipSuccess) return e;
     return allow_lds_cu<1, 2, 2>();
+}
+
+// Nine to sixteen rows of x as two halves of up to eight, one workgroup each per task (the weight is read twice, the
+// second time mostly from the caches): for small weights, where the tile kernel's start-up costs more than that.
+bool gemv_quad_halves_possible(int64_t N, int64_t K) { return K % LOAD_K == 0 && quad_splits(8, K) == 1; }
+
+hipError_t launch_gemv_quad_halves(const MatmulArgs& a, int cus, hipStream_t stream) {
+    if (a.M <= 8 || a.M > 16 || !gemv_quad_halves_possible(a.N, a.K)) return hipErrorInvalidValue;
+    // each half has the chip to itself in the plan: the two halves of a task then run side by side
+    int slots = cus;
+    const QuadPlan p = make_quad_plan(8, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
+    if (p.splits != 1) return hipErrorInvalidValue;
+    int grid = p.ntasks < slots ? p.ntasks : slots;
+    return a.nested.q ? launch_c<1, 2, true>(a, p, grid, stream, 2) : launch_c<1, 2, false>(a, p, grid, stream, 2);
 }
 
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {

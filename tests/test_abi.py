@@ -101,7 +101,8 @@ def test_matmul_argument_errors(ta):
     assert lib.nf4hip_gemv_workspace_bytes(16, 128256, 4096) == COUNTERS                  # big N: K is not split
     assert lib.nf4hip_gemv_workspace_bytes(1, 4096, 4096) == COUNTERS
     assert lib.nf4hip_gemv_workspace_bytes(4, 8192, 28672) == COUNTERS + 4 * 4 * 8192 * 4  # K split over 4 workgroups
-    assert lib.nf4hip_gemv_workspace_bytes(16, 1024, 4096) > COUNTERS                        # tile kernel splits K
+    assert lib.nf4hip_gemv_workspace_bytes(16, 1024, 4096) == COUNTERS                       # small weight: quad kernel on two halves of x
+    assert lib.nf4hip_gemv_workspace_bytes(16, 6144, 4096) > COUNTERS                        # tile kernel splits K
     assert lib.nf4hip_gemm_workspace_bytes(2048, 4096, 4096) == 0
 
 

@@ -325,7 +325,7 @@ def test_split_k_hand_off_holds_over_many_launches(ta):
     code = ta.nf4_code(DEV)
     g = torch.Generator(device=DEV).manual_seed(7)
     calls = []
-    for kind, M, N, K in [("gemv", 16, 4096, 4096), ("gemv", 1, 512, 32768), ("gemm", 64, 1024, 4096), ("gemm", 512, 1024, 4096)]:
+    for kind, M, N, K in [("gemv", 16, 6144, 4096), ("gemv", 1, 512, 32768), ("gemm", 64, 1024, 4096), ("gemm", 512, 1024, 4096)]:
         n = N * K
         packed = torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=DEV, generator=g)
         absmax = torch.rand(n // 64, device=DEV, generator=g) * 0.05 + 0.01

@@ -46,7 +46,7 @@ def _both(ta, M, N, K, seed, with_bias):
 # the scratch array is really used: M = 16 on short weights (MFMA tile kernel), M = 4 / 2 on a long K
 # (quad and row-streaming kernels)
 PAIRS = [
-    ((16, 4096, 4096), (16, 1024, 4096)),
+    ((16, 6144, 4096), (16, 2048, 4096 + 512)),
     ((16, 4096, 14336), (9, 1000, 4096)),
     ((4, 8192, 28672), (2, 512, 28672)),
     ((8, 8192, 8192), (1, 4096, 4096)),

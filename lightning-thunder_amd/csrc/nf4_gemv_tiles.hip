@@ -39,6 +39,7 @@ namespace nf4 {
 namespace {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 constexpr int THREADS = GEMV_THREADS;
@@ -48,7 +49,8 @@ constexpr int PHASE_K = 512;                 // k per phase
 constexpr int XBYTES_MAX = 80 * 1024;        // resident x operands
 constexpr int ITEMS_MAX = 512;               // longest work list of a workgroup (one entry per thread)
 constexpr int ITEMS_OFFSET = TABLE_BYTES + XBYTES_MAX;
-constexpr int SMEM_BYTES = ITEMS_OFFSET + ITEMS_MAX * 16;
+constexpr int UNSCALE_OFFSET = ITEMS_OFFSET + ITEMS_MAX * 16;  // fp16 mode: 16 floats, what undoes the scaling of each row of x
+constexpr int SMEM_BYTES = UNSCALE_OFFSET + 64;
 constexpr int COUNTER_BYTES = GEMV_COUNTER_BYTES;
 constexpr int SLOTS = 4;                     // ring slots = accumulator sets = largest batch
 
@@ -308,10 +310,11 @@ __device__ __forceinline__ void prepare_phase(const MatmulArgs& a, PhaseRegs& r,
 // MFMA j = 4p + q of the phase covers k [32j, 32j + 32) and uses d[q][p].
 // EXACT (K > 8192): fp32 table, every weight rounded as bf16(lut * absmax) before the MFMA -- the
 // reference's dequantisation bit for bit -- and the MFMAs accumulate straight into acc.
-template <int R, bool EXACT>
+template <int R, int MODE>
 __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uint8_t* xph, int lane, f32x4& acc) {
     typedef float f32x2_t __attribute__((ext_vector_type(2)));
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     const uint32_t lane4 = (uint32_t)lane * 4u;
     const uint32_t lane8 = (uint32_t)(lane & 31) * 8u;
     const int gg = lane >> 4, m = lane & 15;
@@ -364,8 +367,12 @@ __device__ __forceinline__ void contract_phase(const PhaseOperands& o, const uin
                                                           acc, 0, 0, 0);
         } else {
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            blk[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f.xa),
-                                                             __builtin_bit_cast(bf16x8, wb), qq ? blk[h] : zero, 0, 0, 0);
+            if (F16)
+                blk[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, f.xa),
+                                                                __builtin_bit_cast(f16x8, wb), qq ? blk[h] : zero, 0, 0, 0);
+            else
+                blk[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f.xa),
+                                                                 __builtin_bit_cast(bf16x8, wb), qq ? blk[h] : zero, 0, 0, 0);
             // the block of the PREVIOUS pair that just completed is scaled here, one MFMA later
             if (qq == 1 && h == 1) {
 #pragma unroll
@@ -408,14 +415,47 @@ __device__ __forceinline__ void store_x_slice(const MatmulArgs& a, const uint4 (
     }
 }
 
+// fp16 mode (the launcher picks it only when the workgroup's K range is ONE slice, so that a row of x keeps one scale
+// for everything its accumulators see): a wave holds whole rows of the slice -- row `wave` in units [0, CAP), row
+// wave + 8 in units [CAP, 2 CAP) -- finds each row's largest |x|, scales the row into fp16's range by a power of two
+// (f16_scale_for), converts it, and leaves what undoes the scaling in `unscale[row]` for the end of the batch.
+template <int R>
+__device__ __forceinline__ void scale_x_slice_to_f16(uint4 (&v)[XUNITS], int n, uint8_t* unscale, int lane, int wave) {
+    constexpr int CAP = XBYTES_MAX / (R * 1024);
+#pragma unroll
+    for (int rg = 0; rg < XUNITS / CAP; ++rg) {
+        u16x2_t mx = {0, 0};
+#pragma unroll
+        for (int pp = 0; pp < CAP; ++pp) {
+            const uint4& w = v[rg * CAP + pp];
+            if (pp < n) {  // units beyond the slice hold a re-read valid unit: harmless, but keep the maximum the slice's own
+                mx = absmax_of_bf16_pair(w.x, mx); mx = absmax_of_bf16_pair(w.y, mx);
+                mx = absmax_of_bf16_pair(w.z, mx); mx = absmax_of_bf16_pair(w.w, mx);
+            }
+        }
+        uint32_t m = absmax_bits(mx);
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off));
+        const F16Scale fs = f16_scale_for(m);
+#pragma unroll
+        for (int pp = 0; pp < CAP; ++pp) {
+            uint4& w = v[rg * CAP + pp];
+            w.x = bf16_pair_to_f16(w.x, fs.to_f16); w.y = bf16_pair_to_f16(w.y, fs.to_f16);
+            w.z = bf16_pair_to_f16(w.z, fs.to_f16); w.w = bf16_pair_to_f16(w.w, fs.to_f16);
+        }
+        if (lane == 0) reinterpret_cast<float*>(unscale)[wave + 8 * rg] = fs.from_f16;
+    }
+}
+
 // STEADY (long work lists): the slots are refilled without branches and groups of four entries that
 // follow each other without a restage or a batch end run in an inner loop that holds nothing else.
 // The compiler can then count the loads in flight and waits for ONE slot where it otherwise waits for
 // everything in flight at the top of every group (loads under branches, and the stores of a batch
 // end, which complete out of order with loads).  The price is a drain when that loop is entered and
 // switched-off requests at the end of the list, which short lists cannot afford.
-template <bool B64, bool NESTED, int R, bool EXACT, bool STEADY>
+template <bool B64, bool NESTED, int R, int MODE, bool STEADY>
 __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Plan p) {
+    constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int CAP = XBYTES_MAX / (R * 1024);  // phases of x that fit
     const int tid = threadIdx.x;
@@ -491,7 +531,8 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
         if (EXACT)
             build_pair_table_f32(smem, lut_lane, lane, wave);
         else
-            build_pair_table(smem, lut_lane, lane, wave);
+            build_pair_table<F16>(smem, lut_lane, lane, wave);
+        if (F16) scale_x_slice_to_f16<R>(xv, nph0, smem + UNSCALE_OFFSET, lane, wave);
         store_x_slice<R>(a, xv, smem + TABLE_BYTES, nph0, lane, wave);
         __syncthreads();
     }
@@ -533,7 +574,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                         load_phase<B64, NESTED>(a, ring[j], ll, first_row(refill ? nx.tg : ls.tg0),
                                                 refill ? nx.kabs : ls.r0 * PHASE_K, refill ? 0xffffffffu : 0u);
                         if (!(it.info & ITEM_GAP)) {
-                            contract_phase<R, EXACT>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane,
+                            contract_phase<R, MODE>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane,
                                                      acc[j]);
                             if (it.info & ITEM_END) {
                                 end_info = it.info;
@@ -557,7 +598,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                     prepare_phase<B64, NESTED, false>(a, ring[j], lane, o);
                     // the slot's registers are free again: refill before the long part of the work
                     if (!(nx.info & ITEM_GAP)) load_phase<B64, NESTED>(a, ring[j], ll, first_row(nx.tg), nx.kabs);
-                    contract_phase<R, EXACT>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane, acc[j]);
+                    contract_phase<R, MODE>(o, smem + TABLE_BYTES + (it.info & ITEM_PHS_MASK) * (R * 1024), lane, acc[j]);
                     if (it.info & ITEM_END) {
                         end_info = it.info;
                         end_tg = it.tg;
@@ -578,6 +619,13 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
         } else if (fin_nb == 2) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[0][i] += acc[2][i], acc[1][i] += acc[3][i];
+        }
+        if (F16) {  // back from the per-row scaling of x (rows 4 g .. 4 g + 3 are this lane's)
+            const float4 us = *reinterpret_cast<const float4*>(smem + UNSCALE_OFFSET + 16 * g);
+#pragma unroll
+            for (int t = 0; t < SLOTS; ++t) {
+                acc[t][0] *= us.x; acc[t][1] *= us.y; acc[t][2] *= us.z; acc[t][3] *= us.w;
+            }
         }
 #pragma unroll
         for (int t = 0; t < SLOTS; ++t) {
@@ -721,10 +769,12 @@ size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 template <bool B64, bool NESTED, bool STEADY>
 hipError_t allow_rx() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, false, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, false, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, true, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, true, STEADY>, SMEM_BYTES);
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, ARITH_BF16, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, ARITH_BF16, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, ARITH_F16, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, ARITH_F16, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 8, ARITH_EXACT, STEADY>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_tiles_kernel<B64, NESTED, 16, ARITH_EXACT, STEADY>, SMEM_BYTES);
 }
 
 template <bool B64, bool NESTED>
@@ -741,20 +791,25 @@ hipError_t gemv_tiles_setup() {
     return allow_both<true, true>();
 }
 
-template <int R, bool EXACT, bool STEADY>
+template <int R, int MODE, bool STEADY>
 hipError_t launch_rs(const MatmulArgs& a, const Plan& p, int grid, hipStream_t stream) {
     const bool b64 = a.block_log2 == 6;
     const bool nested = a.nested.q != nullptr;
-    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R, EXACT, STEADY> : gemv_tiles_kernel<true, false, R, EXACT, STEADY>)
-                    : (nested ? gemv_tiles_kernel<false, true, R, EXACT, STEADY>
-                              : gemv_tiles_kernel<false, false, R, EXACT, STEADY>);
+    auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R, MODE, STEADY> : gemv_tiles_kernel<true, false, R, MODE, STEADY>)
+                    : (nested ? gemv_tiles_kernel<false, true, R, MODE, STEADY>
+                              : gemv_tiles_kernel<false, false, R, MODE, STEADY>);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
-template <int R, bool EXACT>
+template <int R, int MODE>
 hipError_t launch_r(const MatmulArgs& a, const Plan& p, int grid, bool steady, hipStream_t stream) {
-    return steady ? launch_rs<R, EXACT, true>(a, p, grid, stream) : launch_rs<R, EXACT, false>(a, p, grid, stream);
+    return steady ? launch_rs<R, MODE, true>(a, p, grid, stream) : launch_rs<R, MODE, false>(a, p, grid, stream);
+}
+
+template <int MODE>
+hipError_t launch_m(const MatmulArgs& a, const Plan& p, int grid, bool steady, hipStream_t stream) {
+    return rows_held(a.M) == 8 ? launch_r<8, MODE>(a, p, grid, steady, stream) : launch_r<16, MODE>(a, p, grid, steady, stream);
 }
 
 hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
@@ -770,11 +825,12 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
     const int n = rows_held(a.M) == 8 ? list_length<10>(G, nsl, last) : list_length<5>(G, nsl, last);
     if (n > ITEMS_MAX) return hipErrorInvalidValue;
     const bool steady = n >= STEADY_MIN_ITEMS;
-    if (gemv_arith_mode(a.K, false) == ARITH_EXACT)
-        return rows_held(a.M) == 8 ? launch_r<8, true>(a, p, grid, steady, stream)
-                                   : launch_r<16, true>(a, p, grid, steady, stream);
-    return rows_held(a.M) == 8 ? launch_r<8, false>(a, p, grid, steady, stream)
-                               : launch_r<16, false>(a, p, grid, steady, stream);
+    // fp16 arithmetic needs one scale per row of x for everything an accumulator sees: only when the workgroup's K
+    // range is a single slice of x (otherwise the exact variant serves 8192 < K <= 16384 too)
+    const int mode = gemv_arith_mode(a.K, nsl == 1);
+    if (mode == ARITH_EXACT) return launch_m<ARITH_EXACT>(a, p, grid, steady, stream);
+    if (mode == ARITH_F16) return launch_m<ARITH_F16>(a, p, grid, steady, stream);
+    return launch_m<ARITH_BF16>(a, p, grid, steady, stream);
 }
 
 }  // namespace nf4

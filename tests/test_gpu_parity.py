@@ -217,11 +217,12 @@ def test_gemv_shapes(ta, oracle, N, K, M):
 
 
 @pytest.mark.parametrize("K", [2048, 10240])
-@pytest.mark.parametrize("M", [1, 2, 4, 8])
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 11, 16])
 def test_gemv_x_outside_fp16_range(ta, oracle, M, K):
-    """For 8192 < K <= 16384 the row and quad kernels multiply in fp16 after scaling each lane's x values into
-    range (K = 10240; K = 2048 takes the bf16 arithmetic): rows of x far above fp16's largest value, far below its
-    smallest, of mixed magnitudes, and with the largest finite bf16."""
+    """For 8192 < K <= 16384 the decode kernels multiply in fp16 after scaling x into range -- per lane in the row and
+    quad kernels, per row of x in the tile kernel (M = 11, 16) -- (K = 10240; K = 2048 takes the bf16 arithmetic): rows
+    of x far above fp16's largest value, far below its smallest, of mixed magnitudes, and with the largest finite
+    bf16."""
     _sync_print(f"gemv x outside the fp16 range M={M} K={K}")
     N = 192
     w = _weights((N, K), seed=77)

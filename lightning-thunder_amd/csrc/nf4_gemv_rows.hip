@@ -101,7 +101,12 @@ __device__ __forceinline__ int reduce8_id(int lane) { return (lane & 1) | ((lane
 //                used as bf16 / converted to fp16 per lane, and absmax scales the 32-weight partial sum.
 //                ARITH_EXACT: the table holds fp32 pairs and every weight is rounded like the reference's
 //                dequantisation, bf16(lut * absmax), before it is multiplied (more VALU work).
-template <int M, int U, bool NESTED, int MODE>
+// PAIRED (fp32 absmax, K a multiple of the blocksize): one absmax load serves TWO rows in flight -- the two lanes
+//                that share a block fetch that block's absmax of the even and of the odd slot's row, and each slot
+//                reads its value from the right lane through a DPP operand.  The 4-byte loads cost more than their
+//                share of the bytes (a vector memory instruction per KB of codes: the lm_head ran 5 us faster without
+//                them); this halves their number (lm_head 59.7 -> 58.4 us, [28672, 8192] 29.8 -> 28.0 with one row of x).
+template <int M, int U, bool NESTED, int MODE, bool PAIRED>
 __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a, RowsPlan p) {
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -172,8 +177,13 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                     if (NESTED) {
                         sq[u] = __uint_as_float((uint32_t)a.nested.q[blk]);
                         s2[u] = a.nested.absmax2[blk >> a.nested.nested_log2];
-                    } else {
+                    } else if (!PAIRED) {
                         sq[u] = a.absmax[blk];
+                    } else if ((u & 1) == 0) {
+                        // even lanes: this row; odd lanes: the row of slot u + 1 (the wave's next row, if it has one)
+                        const int row2 = r_begin + rl + min(i + 1, cnt - 1) * step;
+                        const int64_t blk2 = (((int64_t)row2 * K + kchunk) >> a.block_log2) + (klane >> a.block_log2);
+                        sq[u] = a.absmax[(lane & 1) ? blk2 : blk];
                     }
                 }
             };
@@ -213,10 +223,20 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
         if (cnt > 0) {
             for (int i0 = 0; i0 < cnt; i0 += U) {
                 float res[U * M];
+                float s_odd = 0.0f;
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const uint32_t d[4] = {wq[u].x, wq[u].y, wq[u].z, wq[u].w};
                     float s = sq[u];
+                    if (PAIRED) {
+                        if ((u & 1) == 0) {
+                            const int both = __builtin_bit_cast(int, sq[u]);
+                            s = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(both, both, 0xA0, 0xf, 0xf, true));  // quad_perm [0,0,2,2]
+                            s_odd = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(both, both, 0xF5, 0xf, 0xf, true));  // quad_perm [1,1,3,3]
+                        } else {
+                            s = s_odd;
+                        }
+                    }
                     if (NESTED)
                         s = __fadd_rn(__fmul_rn(reinterpret_cast<const float*>(smem + MAP_OFFSET)[__float_as_uint(s)], s2[u]),
                                       a.nested.offset);
@@ -360,16 +380,23 @@ RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
     return p;
 }
 
-template <int M, int U, bool NESTED>
-hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
+template <int M, int U, bool NESTED, bool PAIRED>
+hipError_t launch_p(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int mode = gemv_arith_mode(a.K, true);
     if (mode == ARITH_EXACT)
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT, PAIRED>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else if (mode == ARITH_F16)
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16, PAIRED>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16, PAIRED>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
+}
+
+template <int M, int U, bool NESTED>
+hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
+    if constexpr (!NESTED && M == 1)  // measured: 1-2 us on weights of 30 MB and more with one row of x, a loss with two
+        if (p.aligned) return launch_p<M, U, false, true>(a, p, grid, stream);
+    return launch_p<M, U, NESTED, false>(a, p, grid, stream);
 }
 
 // U = rows in flight per wave: as many as the wave has to do, within the register budget
@@ -390,15 +417,21 @@ hipError_t launch_n(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_
     return a.M == 2 ? launch_m<2, NESTED>(a, p, grid, stream) : launch_m<1, NESTED>(a, p, grid, stream);
 }
 
+template <int M, int U, int MODE>
+hipError_t allow_lds_mode() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, MODE, false>, SMEM_BYTES)) != hipSuccess) return e;
+    if constexpr (M == 1)
+        if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, MODE, true>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_rows_kernel<M, U, true, MODE, false>, SMEM_BYTES);
+}
+
 template <int M, int U>
 hipError_t allow_lds_mu() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, true, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, true, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, ARITH_EXACT>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_rows_kernel<M, U, true, ARITH_EXACT>, SMEM_BYTES);
+    if ((e = allow_lds_mode<M, U, ARITH_BF16>()) != hipSuccess) return e;
+    if ((e = allow_lds_mode<M, U, ARITH_F16>()) != hipSuccess) return e;
+    return allow_lds_mode<M, U, ARITH_EXACT>();
 }
 
 template <int M>

@@ -50,8 +50,8 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-constexpr int NORM_THREADS = 256;
-constexpr int NORM_MAX_CHUNKS = 8;  // 8 elements per chunk: d <= 256 * 8 * 8 = 16384
+constexpr int NORM_THREADS = 512;
+constexpr int NORM_MAX_CHUNKS = 4;  // 8 elements per chunk: d <= 512 * 4 * 8 = 16384
 
 // x <- bf16(x + delta) (delta may be null), y <- bf16(x * rsqrt(mean(x^2) + eps) * weight); one
 // workgroup per row.
@@ -63,16 +63,28 @@ __global__ __launch_bounds__(NORM_THREADS) void add_rmsnorm_kernel(uint16_t* x, 
     const int64_t row = blockIdx.x;
     uint16_t* xr = x + row * d;
     const int chunks = d / 8;
+    // every load of the kernel goes out first, the norm weight included: nothing waits on memory twice
+    uint4 xv[NORM_MAX_CHUNKS], dv[NORM_MAX_CHUNKS], wv[NORM_MAX_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < NORM_MAX_CHUNKS; ++c) {
+        const int ch = tid + c * NORM_THREADS;
+        xv[c] = dv[c] = wv[c] = make_uint4(0, 0, 0, 0);
+        if (ch < chunks) {
+            xv[c] = *reinterpret_cast<const uint4*>(xr + ch * 8);
+            if (delta) dv[c] = *reinterpret_cast<const uint4*>(delta + row * d + ch * 8);
+            wv[c] = *reinterpret_cast<const uint4*>(weight + ch * 8);
+        }
+    }
     float v[NORM_MAX_CHUNKS][8];
     float ss = 0.0f;
 #pragma unroll
     for (int c = 0; c < NORM_MAX_CHUNKS; ++c) {
         const int ch = tid + c * NORM_THREADS;
         if (ch < chunks) {
-            unpack8(*reinterpret_cast<const uint4*>(xr + ch * 8), v[c]);
+            unpack8(xv[c], v[c]);
             if (delta) {
                 float dl[8];
-                unpack8(*reinterpret_cast<const uint4*>(delta + row * d + ch * 8), dl);
+                unpack8(dv[c], dl);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[c][i] = bf16_to_f32(f32_to_bf16(v[c][i] + dl[i]));
                 *reinterpret_cast<uint4*>(xr + ch * 8) = pack8(v[c]);
@@ -93,7 +105,7 @@ __global__ __launch_bounds__(NORM_THREADS) void add_rmsnorm_kernel(uint16_t* x, 
         const int ch = tid + c * NORM_THREADS;
         if (ch < chunks) {
             float w[8], o[8];
-            unpack8(*reinterpret_cast<const uint4*>(weight + ch * 8), w);
+            unpack8(wv[c], w);
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = v[c][i] * rstd * w[i];
             *reinterpret_cast<uint4*>(y + row * d + ch * 8) = pack8(o);

@@ -52,6 +52,13 @@ int nf4hip_decode_attention(const void* qkv, const int64_t* pos, const float* co
  * gate_up[rows, 2 dff], dff % 8 == 0. */
 int nf4hip_decode_silu_mul(const void* gate_up, int64_t rows, int64_t dff, void* out, void* stream);
 
+/* Greedy sampling: out[r] <- index of the largest element of logits[r, 0 .. vocab-1] (bf16), the lowest index among
+ * equals, a NaN counting as the largest value (torch.argmax's answer).  One workgroup per row, no scratch.
+ * pos_or_null: a device counter that the call advances by one after the rows are done (the position of the decode
+ * step, so that sampling and bookkeeping are one launch); NULL to leave it out.
+ * Several rows need vocab % 8 == 0 (every row 16-byte aligned). */
+int nf4hip_decode_argmax(const void* logits, int64_t rows, int64_t vocab, int64_t* out, int64_t* pos_or_null, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -333,6 +333,63 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* gate_up, 
     *reinterpret_cast<uint4*>(out + r * dff + c * 8) = pack8(o);
 }
 
+constexpr int ARGMAX_THREADS = 1024;
+
+// Largest element of each row, lowest index on ties, NaN counted as the largest value (what torch.argmax returns);
+// one workgroup per row.  Every element becomes a 64-bit key -- the value's bits in an order-preserving form above
+// the complemented index -- and the row's answer is the largest key, so the order of the reduction does not matter.
+// `pos` (may be null): a position counter that workgroup 0 advances by one, the decode step's bookkeeping.
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_kernel(const uint16_t* logits, int64_t vocab, int64_t* out,
+                                                                 int64_t* pos) {
+    __shared__ unsigned long long red[ARGMAX_THREADS / 64];
+    const int tid = threadIdx.x;
+    const uint16_t* row = logits + (int64_t)blockIdx.x * vocab;
+    auto key_of = [](uint32_t bf, int64_t idx) -> unsigned long long {
+        const uint32_t bits = bf << 16;
+        uint32_t ord = (bits & 0x80000000u) ? ~bits : bits | 0x80000000u;
+        if ((bits & 0x7fffffffu) > 0x7f800000u) ord = 0xffffffffu;  // NaN
+        return ((unsigned long long)ord << 32) | (uint32_t)(0xffffffffu - (uint32_t)idx);
+    };
+    unsigned long long best = 0;
+    const int64_t chunks = vocab / 8;
+    for (int64_t c0 = tid; c0 < chunks; c0 += 4 * ARGMAX_THREADS) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {  // four requests in flight; a request past the end re-reads the thread's first
+            const int64_t c = c0 + (int64_t)u * ARGMAX_THREADS;
+            v[u] = *reinterpret_cast<const uint4*>(row + (c < chunks ? c : c0) * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t c = c0 + (int64_t)u * ARGMAX_THREADS;
+            if (c >= chunks) break;
+            const uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const unsigned long long k0 = key_of(d[i] & 0xffffu, c * 8 + 2 * i), k1 = key_of(d[i] >> 16, c * 8 + 2 * i + 1);
+                best = best > k0 ? best : k0;
+                best = best > k1 ? best : k1;
+            }
+        }
+    }
+    for (int64_t i = chunks * 8 + tid; i < vocab; i += ARGMAX_THREADS) {  // vocab % 8 elements at the end
+        const unsigned long long k = key_of(row[i], i);
+        best = best > k ? best : k;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(best, o, 64);
+        best = best > other ? best : other;
+    }
+    if ((tid & 63) == 0) red[tid >> 6] = best;
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < ARGMAX_THREADS / 64; ++w) best = best > red[w] ? best : red[w];
+        out[blockIdx.x] = (int64_t)(0xffffffffu - (uint32_t)best);
+        if (pos && blockIdx.x == 0) *pos += 1;
+    }
+}
+
 thread_local char g_err[256] = "";
 
 int fail(const char* msg) {
@@ -443,6 +500,20 @@ __attribute__((visibility("default"))) int nf4hip_decode_silu_mul(const void* ga
     hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t*>(gate_up), rows, dff, static_cast<uint16_t*>(out));
     return hipGetLastError() == hipSuccess ? 0 : fail("nf4hip_decode_silu_mul: launch failed");
+}
+
+__attribute__((visibility("default"))) int nf4hip_decode_argmax(const void* logits, int64_t rows, int64_t vocab, int64_t* out,
+                                                                int64_t* pos_or_null, void* stream) {
+    if (!logits || !out) return fail("nf4hip_decode_argmax: null pointer");
+    if (rows <= 0 || vocab <= 0 || rows > INT32_MAX || vocab > 0xffffffffLL)
+        return fail("nf4hip_decode_argmax: need 0 < rows < 2^31 and 0 < vocab < 2^32");
+    if (!aligned16(logits) || (rows > 1 && vocab % 8))
+        return fail("nf4hip_decode_argmax: logits not 16-byte aligned, or several rows whose length is no multiple of 8");
+    if ((reinterpret_cast<uintptr_t>(out) & 7u) || (reinterpret_cast<uintptr_t>(pos_or_null) & 7u))
+        return fail("nf4hip_decode_argmax: out / pos not 8-byte aligned");
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(ARGMAX_THREADS), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(logits), vocab, out, pos_or_null);
+    return hipGetLastError() == hipSuccess ? 0 : fail("nf4hip_decode_argmax: launch failed");
 }
 
 }  // extern "C"

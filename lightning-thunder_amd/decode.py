@@ -249,8 +249,13 @@ def greedy_decode(model, cfg: LlamaConfig, prompt: torch.Tensor, n_new: int, use
     out[0] = first[:, 0]
 
     def step():
-        nxt = model(tok, pos, kcache, vcache).argmax(-1, keepdim=True)
-        tok.copy_(nxt)
+        logits = model(tok, pos, kcache, vcache)
+        if cfg.hip_glue and logits.is_cuda and logits.dtype == torch.bfloat16:
+            from . import glue
+
+            glue.argmax_into(logits, tok.view(-1), pos)  # the next token and pos += 1 in one launch
+            return
+        tok.copy_(logits.argmax(-1, keepdim=True))
         pos.add_(1)
 
     graph = None

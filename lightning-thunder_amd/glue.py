@@ -27,6 +27,7 @@ SYMBOLS = {
     "nf4hip_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32]),
     "nf4hip_decode_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, ctypes.c_size_t, _vp]),
     "nf4hip_decode_silu_mul": (_i32, [_vp, _i64, _i64, _vp, _vp]),
+    "nf4hip_decode_argmax": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp]),
 }
 
 _lib = None
@@ -136,3 +137,18 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     with torch.cuda.device(gate_up.device):
         _check(lib, lib.nf4hip_decode_silu_mul(gate_up.data_ptr(), rows, dff, out.data_ptr(), _stream(gate_up)))
     return out
+
+
+def argmax_into(logits: torch.Tensor, out: torch.Tensor, pos: torch.Tensor | None = None) -> None:
+    """``out[r] = logits[r].argmax()`` for ``logits`` [rows, vocab] bf16 and ``out`` int64 with ``rows`` elements;
+    ``pos`` (a one-element int64 tensor on the GPU), when given, is advanced by one in the same launch."""
+    lib = load()
+    _bf16_cuda(logits)
+    rows, vocab = logits.shape
+    if not (out.is_cuda and out.dtype == torch.int64 and out.is_contiguous() and out.numel() == rows):
+        raise ValueError(f"out must be a contiguous int64 GPU tensor of {rows} elements, got {out.dtype} {tuple(out.shape)}")
+    if pos is not None and not (pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1):
+        raise ValueError("pos must be a one-element int64 tensor on the GPU")
+    with torch.cuda.device(logits.device):
+        _check(lib, lib.nf4hip_decode_argmax(logits.data_ptr(), rows, vocab, out.data_ptr(), None if pos is None else pos.data_ptr(),
+                                             _stream(logits)))

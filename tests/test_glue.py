@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol(glue):
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     declared = sorted(set(re.findall(r"\b(nf4hip_decode_\w+)\s*\(", text)))
     lib = glue.load()
-    assert len(declared) == 5
+    assert len(declared) == 6
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/nf4hip_decode.h but not exported"
     assert sorted(glue.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
@@ -51,6 +51,9 @@ def test_argument_errors_come_before_any_hip_call(glue):
     assert lib.nf4hip_decode_attention_workspace_bytes(64, 32, 128) == 0  # one workgroup per (sequence, head) is plenty
     assert lib.nf4hip_decode_silu_mul(A, 1, 12, A, None) == -1 and "multiple of 8" in err()
     assert lib.nf4hip_decode_silu_mul(A, 0, 16, A, None) == -1
+    assert lib.nf4hip_decode_argmax(None, 1, 64, A, None, None) == -1 and "null" in err()
+    assert lib.nf4hip_decode_argmax(A, 2, 63, A, None, None) == -1 and "multiple of 8" in err()
+    assert lib.nf4hip_decode_argmax(A, 1, 64, A + 4, None, None) == -1 and "8-byte" in err()
 
 
 def test_missing_library_fails_loudly(glue, tmp_path):
@@ -89,6 +92,30 @@ def test_silu_mul(glue, rows, dff):
     torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1e-3)  # two bf16 roundings
     torch_glue = (torch.nn.functional.silu(gu[:, :dff]) * gu[:, dff:]).float()
     assert ((out.float() - torch_glue).abs() <= 8e-3 * torch_glue.abs() + 1e-6).all()  # at most one bf16 ulp apart
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,vocab", [(1, 128256), (8, 128256), (3, 1024), (1, 1003), (2, 8)])
+def test_argmax(glue, rows, vocab):
+    """torch.argmax's answer: the first index of the largest value; ties, +-inf and a NaN are put into the rows."""
+    print(f"argmax rows={rows} vocab={vocab}", flush=True)
+    x = _randn((rows, vocab), 9, 3.0)
+    x[0, vocab // 2] = x[0].max()          # a tie: the lower index wins
+    x[0, 1] = float("-inf")
+    if rows > 1:
+        x[1, vocab - 1] = float("inf")
+    if rows > 2:
+        x[2, 5] = float("nan")             # NaN counts as the largest
+        x[2, 7] = float("inf")
+    xd = x.to(DEV)
+    out = torch.full((rows,), -1, dtype=torch.int64, device=DEV)
+    pos = torch.tensor([41], dtype=torch.int64, device=DEV)
+    glue.argmax_into(xd, out, pos)
+    assert torch.equal(out.cpu(), x.float().argmax(-1))
+    assert torch.equal(out, xd.argmax(-1))
+    assert int(pos) == 42
+    glue.argmax_into(xd, out)  # without the counter
+    assert int(pos) == 42 and torch.equal(out.cpu(), x.float().argmax(-1))
 
 
 def _rope_ref(x, cos, sin):  # x [..., hd] fp32, cos/sin [hd]

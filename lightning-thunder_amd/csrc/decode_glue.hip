@@ -1,6 +1,6 @@
 // The three operations between the 4-bit linears of a Llama decode step (one new token per
 // sequence), each as one kernel for gfx950: residual add + RMSNorm, rotary embedding + KV-cache
-// update + grouped-query attention over the cache, SiLU(gate) * up.  In the reference these run as
+// update + grouped-query attention over the cache, SiLU(gate) * up; and greedy sampling (row argmax).  In the reference these run as
 // fusions of its other executors around the quantized linear (thunder/executors/sdpaex.py for the
 // attention, the nvFuser / torch.compile executors for the element-wise and norm work); here they
 // exist so that the decode-step harness is bound by the NF4 kernels rather than by ~18 small

@@ -7,8 +7,9 @@ decoding loop whose single-token step is captured in a HIP graph, the way the re
 tagged as static inputs (thunder/transforms/quantization.py:178,186).  Everything that is not a
 linear (norms, rotary embedding, attention, sampling) is plain PyTorch by default: it is plumbing
 around the path, not part of it.  With ``LlamaConfig.hip_glue`` the single-token step runs that work in
-three HIP kernels instead (``glue.py``: residual add + RMSNorm, rotary + cache update + attention,
-SiLU * up), so that the step is bound by the 4-bit linears rather than by ~18 small launches per layer.
+HIP kernels instead (``glue.py``: residual add + RMSNorm, rotary + cache update + attention,
+SiLU * up; greedy sampling as a fourth), so that the step is bound by the 4-bit linears rather than by ~18 small
+launches per layer.
 
 ``fused_projections=True`` builds Q/K/V and gate/up as ONE linear each ([6144, 4096] and
 [28672, 4096] for Llama-3-8B).  NF4 blocks are 64 consecutive elements of a row, so the packed

@@ -1,8 +1,8 @@
 """Decode-step glue: ctypes binding of ``libnf4hip_decode.so`` (C ABI in ``include/nf4hip_decode.h``).
 
 Three kernels for the work between the 4-bit linears of a Llama decode step -- residual add +
-RMSNorm, rotary embedding + KV-cache update + grouped-query attention, SiLU(gate) * up -- used by
-``decode.Llama`` when ``LlamaConfig.hip_glue`` is set.  The reference leaves this work to its other
+RMSNorm, rotary embedding + KV-cache update + grouped-query attention, SiLU(gate) * up -- and a row
+argmax for greedy sampling, used by ``decode.Llama`` / ``decode.greedy_decode`` when ``LlamaConfig.hip_glue`` is set.  The reference leaves this work to its other
 executors (thunder/executors/sdpaex.py, nvFuser / torch.compile fusions); it is not part of the
 bitsandbytes path.  There is no CPU fallback: without the built library these functions raise.
 """

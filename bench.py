@@ -444,14 +444,16 @@ def llama_decode(torch, ta, n_new: int) -> dict:
     HIP graph, Q/K/V and gate/up as one linear each."""
     D = importlib.import_module("lightning-thunder_amd.decode")
     dev = torch.device("cuda:0")
-    cfg = D.LlamaConfig.llama3_8b(fused_projections=True)
+    cfg = D.LlamaConfig.llama3_8b(fused_projections=True, gate_up_interleaved=True)
     model = D.build_llama(cfg, device=dev, seed=4000)
     jm = ta.jit(model, transforms=[ta.BitsAndBytesLinearQuant4bit()])
     nweights = sum(m.weight.numel() for m in model.modules() if isinstance(m, torch.nn.Linear))
     out = {
         "model": "Llama-3-8B architecture (32 layers, d 4096, 32q/8kv heads, FFN 14336, vocab 128256), random init, "
-                 "all 161 linears NF4 (QKV and gate/up fused), prompt 512, greedy, HIP-graph decode step; norms / rotary + attention / SiLU*up between the linears as 3 HIP kernels "
-                 "(decode_tok_per_s) or as PyTorch ops (decode_tok_per_s_torch_glue)",
+                 "all 161 linears NF4 (QKV and gate/up fused, gate and up rows interleaved), prompt 512, greedy, HIP-graph decode step; "
+                 "decode_tok_per_s: residual add + RMSNorm + SiLU*up in the epilogues of the NF4 decode kernels (up to two rows of x), "
+                 "rotary + cache + attention and sampling as HIP glue kernels; _separate_glue: all of that work as HIP glue kernels "
+                 "between the linears; _torch_glue: as PyTorch ops",
         "new_tokens": n_new,
         "linear_weight_bytes_per_token": int(nweights * 0.5625),
         "hbm_bound_tok_per_s_batch1": round(HBM_PEAK_GBS * 1e9 / (nweights * 0.5625), 1),
@@ -461,12 +463,13 @@ def llama_decode(torch, ta, n_new: int) -> dict:
         prompt = torch.randint(0, cfg.vocab, (B, 512), generator=g, device=dev)
         D.greedy_decode(jm, cfg, prompt, n_new=1, use_graph=False)  # untimed: library start-up, GEMM heuristics
         res = {}
-        # the single-token step with the HIP glue kernels (norm, rotary + cache + attention, SiLU * up)
-        # around the NF4 linears, and with plain PyTorch ops in their place
-        for key, glue in (("", True), ("_torch_glue", False)):
-            if B > 8 and not glue:
-                continue
-            cfg.hip_glue = glue
+        # the single-token step with residual add / RMSNorm / SiLU * up done by the epilogues of the NF4 decode kernels
+        # where those take them (up to two rows of x; rotary + cache + attention and sampling as HIP glue kernels), with
+        # all of that work as HIP glue kernels of its own, and with plain PyTorch ops in its place
+        for key, glue, epi in (("", True, True), ("_separate_glue", True, False), ("_torch_glue", False, False)):
+            if (B > 8 and not glue) or (B > 2 and glue and not epi):
+                continue  # beyond two rows of x the first variant already is the second
+            cfg.hip_glue, cfg.linear_epilogues = glue, epi
             _, st = D.greedy_decode(jm, cfg, prompt, n_new=n_new, use_graph=True)
             res[f"decode_tok_per_s{key}"] = round(st["decode_tok_per_s"], 1)
             res[f"ms_per_step{key}"] = round(st["decode_s"] / st["decode_steps"] * 1e3, 3)

@@ -117,6 +117,47 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
                    size_t workspace_bytes, void* stream);
 
 /*
+ * nf4hip_gemv with an epilogue: the thread that finishes an output also does the element-wise / normalising step
+ * that follows (or precedes) the linear in a decoder layer, so that a decode step needs one launch per linear instead
+ * of two.  In the reference these steps are fusions of its other executors around bnb_matmul_nf4
+ * (thunder/transforms/quantization.py:34-39 has no epilogue); at one to sixteen rows of x each of them costs a launch
+ * that takes as long as a small linear.  Every output is finished by exactly one thread, so nothing is computed twice.
+ * fp32 absmax only; same rules as nf4hip_gemv otherwise.  A case the serving kernel does not take (rows of x beyond
+ * two, K too long for one workgroup, odd N with pairs) returns NF4HIP_E_SHAPE: run nf4hip_gemv and the step by itself.
+ *
+ *   NF4HIP_EPI_SILU_PAIRS   weight rows 2j and 2j+1 are row j of the gate and of the up projection; out is [M, N/2]:
+ *                           out[m][j] = bf16( bf16(silu(g)) * u ), g = bf16(sum[m][2j]), u = bf16(sum[m][2j+1])
+ *                           -- what SiLU(gate) * up on the bf16 output of nf4hip_gemv gives, bit for bit.
+ *   NF4HIP_EPI_RESID_NORM   d = bf16(sum[m][n] + bias[n]); r = bf16(resid_in[m][n] + d) -> resid_out[m][n];
+ *                           bf16(r * norm_weight[n]) -> xnext_out[m][n]; the sum of r^2 over the outputs of one
+ *                           workgroup -> out_sumsq[m * parts + workgroup], parts = nf4hip_gemv_norm_parts(M, N, K).
+ *                           `out` is not written (NULL accepted).  resid_out may be resid_in.
+ *   NF4HIP_EPI_ROWSCALE     x is the xnext_out of a RESID_NORM call and in_sumsq / in_parts its out_sumsq / parts:
+ *                           sum[m][n] is multiplied by 1 / sqrt(sum_p in_sumsq[m][p] / K + eps) before the bias, i.e.
+ *                           out = linear(rms_norm(r) * norm_weight) with the per-row factor applied to the finished
+ *                           sums instead of to every element.  May be combined with SILU_PAIRS.
+ */
+#define NF4HIP_EPI_ROWSCALE 1
+#define NF4HIP_EPI_SILU_PAIRS 2
+#define NF4HIP_EPI_RESID_NORM 4
+typedef struct nf4hip_epilogue {
+    int flags; /* NF4HIP_EPI_* */
+    float eps;
+    const float* in_sumsq; /* ROWSCALE: [M, in_parts] */
+    int in_parts;
+    const void* resid_in;    /* RESID_NORM: [M, N] bf16 */
+    const void* norm_weight; /* RESID_NORM: [N] bf16 */
+    void* resid_out;         /* RESID_NORM: [M, N] bf16 */
+    void* xnext_out;         /* RESID_NORM: [M, N] bf16 */
+    float* out_sumsq;        /* RESID_NORM: [M, nf4hip_gemv_norm_parts(M, N, K)] */
+} nf4hip_epilogue;
+/* partial sums per row of x that a RESID_NORM call on the current device writes (0: the shape is not served) */
+int nf4hip_gemv_norm_parts(int64_t M, int64_t N, int64_t K);
+int nf4hip_gemv_epilogue(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
+                         const float* lut16, const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out,
+                         void* workspace, size_t workspace_bytes, const nf4hip_epilogue* epilogue, void* stream);
+
+/*
  * nf4hip_gemv for callers that cannot allocate or own a workspace (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference:
  * bitsandbytes' gemv_4bit needs no scratch, and the workspace of nf4hip_gemv is this library's own

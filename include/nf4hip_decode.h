@@ -51,6 +51,10 @@ int nf4hip_decode_attention(const void* qkv, const int64_t* pos, const float* co
 /* out[rows, dff] <- bf16(bf16(silu(gate)) * up) with gate = gate_up[:, :dff], up = gate_up[:, dff:];
  * gate_up[rows, 2 dff], dff % 8 == 0. */
 int nf4hip_decode_silu_mul(const void* gate_up, int64_t rows, int64_t dff, void* out, void* stream);
+/* The same for gate and up interleaved: gate_up[:, 2j] = gate[:, j], gate_up[:, 2j+1] = up[:, j] -- the output of a linear
+ * whose weight rows alternate between the gate and the up projection (the layout nf4hip_gemv_epilogue's
+ * NF4HIP_EPI_SILU_PAIRS expects). */
+int nf4hip_decode_silu_mul_pairs(const void* gate_up, int64_t rows, int64_t dff, void* out, void* stream);
 
 /* Greedy sampling: out[r] <- index of the largest element of logits[r, 0 .. vocab-1] (bf16), the lowest index among
  * equals, a NaN counting as the largest value (torch.argmax's answer).  One workgroup per row, no scratch.

@@ -35,6 +35,17 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libnf4hip.s
 _vp, _i32, _i64, _f32, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t
 _MATMUL = [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp, _sz, _vp]
 _MATMUL_DQ = [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _f32, _i32, _vp, _vp, _i64, _i64, _i32, _vp, _vp, _sz, _vp]
+
+
+class Epilogue(ctypes.Structure):
+    """``nf4hip_epilogue`` of include/nf4hip.h."""
+
+    _fields_ = [("flags", _i32), ("eps", _f32), ("in_sumsq", _vp), ("in_parts", _i32), ("resid_in", _vp),
+                ("norm_weight", _vp), ("resid_out", _vp), ("xnext_out", _vp), ("out_sumsq", _vp)]
+
+
+EPI_ROWSCALE, EPI_SILU_PAIRS, EPI_RESID_NORM = 1, 2, 4
+
 SYMBOLS = {
     "nf4hip_abi_version": (_i32, []),
     "nf4hip_last_error": (ctypes.c_char_p, []),
@@ -46,6 +57,8 @@ SYMBOLS = {
     "nf4hip_gemv_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "nf4hip_gemv": (_i32, _MATMUL),
     "nf4hip_gemv_dq": (_i32, _MATMUL_DQ),
+    "nf4hip_gemv_epilogue": (_i32, _MATMUL[:-1] + [ctypes.POINTER(Epilogue), _vp]),
+    "nf4hip_gemv_norm_parts": (_i32, [_i64, _i64, _i64]),
     "nf4hip_gemv_static": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp]),
     "nf4hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "nf4hip_gemm": (_i32, _MATMUL),

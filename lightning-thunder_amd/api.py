@@ -60,9 +60,12 @@ class _QuantWeight(torch.Tensor):
     sees the plain uint8 tensor."""
 
     @staticmethod
-    def __new__(cls, packed: torch.Tensor, call):
+    def __new__(cls, packed: torch.Tensor, call, operator=None):
         t = packed.detach().as_subclass(cls)
         t._planned_call = call
+        # (operator name, packed weight, the operator's arguments after bias): for callers that run a variant of the
+        # planned operator on this weight (the decode step's linears with an epilogue)
+        t._planned_operator = operator
         return t
 
     @classmethod
@@ -130,7 +133,7 @@ def _plan_call(tm: ThunderModule, cd: CompileData, cs: CompileStats) -> _Plan:
         def call(x, bias, _b=b, _packed=packed, _rest=rest):
             return _b(x, _packed, bias, *_rest)
 
-        wrappers[w_name] = _QuantWeight(packed, call)
+        wrappers[w_name] = _QuantWeight(packed, call, (b.sym.name, packed, rest))
     for t in cd.transforms:
         comp = t.transform_trace_post_optimization(comp, executors_list=cd.executors_list)
     plan.prologue_trace, plan.computation_trace, plan.epilogue_trace = pro, comp, epi

@@ -9,7 +9,10 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <string>
+
 #include "../../include/nf4hip_decode.h"
+#include "decode_math.h"
 
 namespace {
 
@@ -86,7 +89,7 @@ __global__ __launch_bounds__(NORM_THREADS) void add_rmsnorm_kernel(uint16_t* x, 
                 float dl[8];
                 unpack8(dv[c], dl);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[c][i] = bf16_to_f32(f32_to_bf16(v[c][i] + dl[i]));
+                for (int i = 0; i < 8; ++i) v[c][i] = nf4x::resid_add(v[c][i], dl[i]);
                 *reinterpret_cast<uint4*>(xr + ch * 8) = pack8(v[c]);
             }
 #pragma unroll
@@ -319,17 +322,30 @@ __global__ __launch_bounds__(ATTN_THREADS) void attention_decode_kernel(const ui
     if (tid == 0) __hip_atomic_store(&counters[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// out <- bf16(bf16(silu(gate)) * up), gate = gate_up[:, :dff], up = gate_up[:, dff:]
+// out <- bf16(bf16(silu(gate)) * up).  PAIRS false: gate = gate_up[:, :dff], up = gate_up[:, dff:]; true: gate and up
+// interleaved, gate_up[:, 2j] = gate[:, j], gate_up[:, 2j + 1] = up[:, j] (a thread's 8 outputs come from 32 contiguous bytes)
+template <bool PAIRS>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* gate_up, int64_t rows, int64_t dff, uint16_t* out) {
     const int64_t per_row = dff / 8;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= rows * per_row) return;
     const int64_t r = i / per_row, c = i - r * per_row;
     float g[8], u[8], o[8];
-    unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * dff + c * 8), g);
-    unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * dff + dff + c * 8), u);
+    if (PAIRS) {
+        float a[8], b[8];
+        unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * dff + c * 16), a);
+        unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * dff + c * 16 + 8), b);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) o[k] = bf16_to_f32(f32_to_bf16(g[k] / (1.0f + __expf(-g[k])))) * u[k];
+        for (int k = 0; k < 4; ++k) {
+            g[k] = a[2 * k]; u[k] = a[2 * k + 1];
+            g[4 + k] = b[2 * k]; u[4 + k] = b[2 * k + 1];
+        }
+    } else {
+        unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * dff + c * 8), g);
+        unpack8(*reinterpret_cast<const uint4*>(gate_up + r * 2 * dff + dff + c * 8), u);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = bf16_to_f32(nf4x::silu_mul_bf16(g[k], u[k]));
     *reinterpret_cast<uint4*>(out + r * dff + c * 8) = pack8(o);
 }
 
@@ -491,15 +507,29 @@ __attribute__((visibility("default"))) int nf4hip_decode_attention(const void* q
     return hipGetLastError() == hipSuccess ? 0 : fail("nf4hip_decode_attention: launch failed");
 }
 
+static int silu_mul_launch(const char* name, bool pairs, const void* gate_up, int64_t rows, int64_t dff, void* out, void* stream) {
+    if (!gate_up || !out) return fail((std::string(name) + ": null pointer").c_str());
+    if (rows <= 0 || dff <= 0 || dff % 8) return fail((std::string(name) + ": need rows > 0 and dff a multiple of 8").c_str());
+    if (!aligned16(gate_up) || !aligned16(out)) return fail((std::string(name) + ": pointer not 16-byte aligned").c_str());
+    const int64_t n = rows * (dff / 8);
+    const dim3 grid((unsigned)((n + 255) / 256));
+    if (pairs)
+        hipLaunchKernelGGL(silu_mul_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(gate_up), rows, dff, static_cast<uint16_t*>(out));
+    else
+        hipLaunchKernelGGL(silu_mul_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(gate_up), rows, dff, static_cast<uint16_t*>(out));
+    return hipGetLastError() == hipSuccess ? 0 : fail((std::string(name) + ": launch failed").c_str());
+}
+
 __attribute__((visibility("default"))) int nf4hip_decode_silu_mul(const void* gate_up, int64_t rows, int64_t dff, void* out,
                                                                   void* stream) {
-    if (!gate_up || !out) return fail("nf4hip_decode_silu_mul: null pointer");
-    if (rows <= 0 || dff <= 0 || dff % 8) return fail("nf4hip_decode_silu_mul: need rows > 0 and dff a multiple of 8");
-    if (!aligned16(gate_up) || !aligned16(out)) return fail("nf4hip_decode_silu_mul: pointer not 16-byte aligned");
-    const int64_t n = rows * (dff / 8);
-    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint16_t*>(gate_up), rows, dff, static_cast<uint16_t*>(out));
-    return hipGetLastError() == hipSuccess ? 0 : fail("nf4hip_decode_silu_mul: launch failed");
+    return silu_mul_launch("nf4hip_decode_silu_mul", false, gate_up, rows, dff, out, stream);
+}
+
+__attribute__((visibility("default"))) int nf4hip_decode_silu_mul_pairs(const void* gate_up, int64_t rows, int64_t dff, void* out,
+                                                                        void* stream) {
+    return silu_mul_launch("nf4hip_decode_silu_mul_pairs", true, gate_up, rows, dff, out, stream);
 }
 
 __attribute__((visibility("default"))) int nf4hip_decode_argmax(const void* logits, int64_t rows, int64_t vocab, int64_t* out,

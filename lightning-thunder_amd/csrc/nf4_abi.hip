@@ -97,8 +97,8 @@ enum MatmulKind { GEMV, GEMM };
 int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
                   const nf4::NestedAbsmax* nested, const float* lut16, const void* bias, int64_t N, int64_t K,
                   int blocksize, void* out, void* workspace, size_t workspace_bytes, void* stream,
-                  bool use_static = false) {
-    const char* name = use_static ? "nf4hip_gemv_static" : kind == GEMV ? "nf4hip_gemv" : "nf4hip_gemm";
+                  bool use_static = false, const nf4hip_epilogue* epi = nullptr) {
+    const char* name = epi ? "nf4hip_gemv_epilogue" : use_static ? "nf4hip_gemv_static" : kind == GEMV ? "nf4hip_gemv" : "nf4hip_gemm";
     if (!x || !packed || !lut16 || !out) return fail(NF4HIP_E_NULL, "%s: null pointer", name);
     if (!nested && !absmax) return fail(NF4HIP_E_NULL, "%s: absmax is null", name);
     if (x_dtype != NF4HIP_BF16)
@@ -152,6 +152,27 @@ int matmul_common(MatmulKind kind, const void* x, int x_dtype, int64_t M, const 
     a.block_log2 = bl;
     a.workspace = workspace;
     a.workspace_bytes = workspace_bytes;
+    a.epi = nf4::Epilogue{nf4::EPI_NONE, 0.0f, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (epi && epi->flags) {
+        const int f = epi->flags;
+        const bool scale = f & NF4HIP_EPI_ROWSCALE, pairs = f & NF4HIP_EPI_SILU_PAIRS, resid = f & NF4HIP_EPI_RESID_NORM;
+        if ((f & ~(NF4HIP_EPI_ROWSCALE | NF4HIP_EPI_SILU_PAIRS | NF4HIP_EPI_RESID_NORM)) || (resid && (scale || pairs)))
+            return fail(NF4HIP_E_SHAPE, "%s: flags %d: RESID_NORM stands alone, ROWSCALE and SILU_PAIRS may be combined", name, f);
+        if (scale && (!epi->in_sumsq || epi->in_parts <= 0))
+            return fail(NF4HIP_E_NULL, "%s: ROWSCALE needs in_sumsq and in_parts > 0", name);
+        if (resid && (!epi->resid_in || !epi->norm_weight || !epi->resid_out || !epi->xnext_out || !epi->out_sumsq))
+            return fail(NF4HIP_E_NULL, "%s: RESID_NORM needs resid_in, norm_weight, resid_out, xnext_out and out_sumsq", name);
+        if ((scale && !aligned4(epi->in_sumsq)) || (resid && !aligned4(epi->out_sumsq)) ||
+            (resid && ((reinterpret_cast<uintptr_t>(epi->resid_in) | reinterpret_cast<uintptr_t>(epi->norm_weight) |
+                        reinterpret_cast<uintptr_t>(epi->resid_out) | reinterpret_cast<uintptr_t>(epi->xnext_out)) & 1u)))
+            return fail(NF4HIP_E_ALIGN, "%s: an epilogue tensor is not aligned to its element size", name);
+        a.epi = nf4::Epilogue{f, epi->eps, epi->in_sumsq, epi->in_parts, static_cast<const uint16_t*>(epi->resid_in),
+                              static_cast<const uint16_t*>(epi->norm_weight), static_cast<uint16_t*>(epi->resid_out),
+                              static_cast<uint16_t*>(epi->xnext_out), epi->out_sumsq};
+        if (!nf4::gemv_epilogue_possible(a))
+            return fail(NF4HIP_E_SHAPE, "%s: M = %lld, N = %lld, K = %lld with flags %d is not served (run nf4hip_gemv and the operation by itself)",
+                        name, (long long)M, (long long)N, (long long)K, f);
+    }
     if (use_static) {
         const hipError_t es = static_scratch(&a.workspace, static_cast<hipStream_t>(stream));
         if (es != hipSuccess) return hip_fail(name, es);
@@ -270,6 +291,21 @@ int nf4hip_gemv_static(const void* x, int x_dtype, int64_t M, const uint8_t* pac
                        void* stream) {
     return matmul_common(GEMV, x, x_dtype, M, packed, absmax, nullptr, lut16, bias_or_null, N, K, blocksize, out,
                          nullptr, 0, stream, true);
+}
+
+int nf4hip_gemv_epilogue(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
+                         const float* lut16, const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out,
+                         void* workspace, size_t workspace_bytes, const nf4hip_epilogue* epilogue, void* stream) {
+    if (!epilogue) return fail(NF4HIP_E_NULL, "nf4hip_gemv_epilogue: epilogue is null");
+    // RESID_NORM writes resid_out / xnext_out instead of out
+    if (!out && (epilogue->flags & NF4HIP_EPI_RESID_NORM)) out = epilogue->xnext_out;
+    return matmul_common(GEMV, x, x_dtype, M, packed, absmax, nullptr, lut16, bias_or_null, N, K, blocksize, out,
+                         workspace, workspace_bytes, stream, false, epilogue);
+}
+
+int nf4hip_gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || M > 16) return 0;
+    return nf4::gemv_norm_parts(M, N, K);
 }
 
 int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,

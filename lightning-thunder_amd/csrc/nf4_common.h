@@ -17,6 +17,27 @@ struct NestedAbsmax {
     int nested_log2;       // log2(nested_blocksize)
 };
 
+// What a decode-shape matmul does with its finished sums besides rounding them (fp32 absmax, K not split over
+// workgroups).  Each output is finished by exactly one thread, so nothing here is computed twice.
+//   EPI_ROWSCALE    sum[m][n] *= 1 / sqrt(mean_sq[m] + eps) before bias: x is bf16(r * norm_weight) written by an
+//                   EPI_RESID_NORM call, in_sumsq [M, in_parts] that call's partial sums of r^2 (mean over this K).
+//   EPI_SILU_PAIRS  weight rows 2j / 2j+1 are gate row j / up row j: out [M, N/2], out[m][j] = silu(gate) * up
+//                   with the roundings of bf16 linear outputs, a bf16 SiLU and a bf16 product.
+//   EPI_RESID_NORM  d = bf16(sum + bias); r = bf16(resid_in + d) -> resid_out; bf16(r * norm_weight) -> xnext_out;
+//                   the workgroup's sum of r^2 per row of x -> out_sumsq[m * parts + band]; `out` is not written.
+enum : int { EPI_NONE = 0, EPI_ROWSCALE = 1, EPI_SILU_PAIRS = 2, EPI_RESID_NORM = 4 };
+struct Epilogue {
+    int flags;
+    float eps;
+    const float* in_sumsq;
+    int in_parts;
+    const uint16_t* resid_in;     // [M, N]
+    const uint16_t* norm_weight;  // [N]
+    uint16_t* resid_out;          // [M, N]
+    uint16_t* xnext_out;          // [M, N]
+    float* out_sumsq;             // [M, gemv_norm_parts(M, N, K)]
+};
+
 struct MatmulArgs {
     const uint16_t* x;    // [M, K] bf16
     const uint8_t* packed;  // [N*K/2]
@@ -29,6 +50,7 @@ struct MatmulArgs {
     int block_log2;  // log2(blocksize)
     void* workspace;
     size_t workspace_bytes;
+    Epilogue epi;
 };
 
 // Launchers (defined next to their kernels).  They assume validated arguments and return the
@@ -47,6 +69,8 @@ constexpr size_t GEMV_COUNTER_REGION_BYTES = 65536 * 4;
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream);
+bool gemv_epilogue_possible(const MatmulArgs& a);  // does the kernel that serves (M, N, K) take a.epi?
+int gemv_norm_parts(int64_t M, int64_t N, int64_t K);  // partial sums per row of x an EPI_RESID_NORM call writes (0: not served)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream);
 // more than 128 rows of x: one wave per SIMD, 256 x 256 or 128 x 256 tiles (nf4_gemm_wide.hip)

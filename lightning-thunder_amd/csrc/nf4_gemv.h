@@ -148,6 +148,8 @@ hipError_t gemv_allow_lds(K kern, int bytes) {
 size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_rows_setup();
 hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream);
+bool gemv_rows_epilogue_possible(const MatmulArgs& a);
+int gemv_rows_norm_parts(int64_t M, int64_t N, int64_t K, int cus);
 
 // four-weight-rows-per-quad kernel, 3 <= M <= 8 (nf4_gemv_quad.hip)
 size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K);

@@ -54,7 +54,23 @@ size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return quad_serves(M, N, K) ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
 }
 
+bool gemv_epilogue_possible(const MatmulArgs& a) {
+    if (a.epi.flags == EPI_NONE) return true;
+    if (a.M <= 2) return gemv_rows_epilogue_possible(a);
+    return false;
+}
+
+// The number of partial sums is the number of bands of the launch plan, which depends on the device's CU count: the
+// current device's (256, the part this library is written for, where no device answers).
+int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
+    int cus = 256;
+    if (device_setup(&cus) != hipSuccess) cus = 256;
+    if (M <= 2) return gemv_rows_norm_parts(M, N, K, cus);
+    return 0;
+}
+
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
+    if (!gemv_epilogue_possible(a)) return hipErrorNotSupported;
     int cus = 0;
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;

@@ -32,6 +32,7 @@
 //  * K > 16384 is split over two or more workgroups; partial sums cross workgroups through
 //    agent-scope relaxed atomics and a counter (no L2-wide fences), added in a fixed order by the
 //    last workgroup to arrive.
+#include "decode_math.h"
 #include "nf4_gemv.h"
 
 namespace nf4 {
@@ -49,6 +50,11 @@ constexpr int CHUNK_K = 2048;          // k covered by one wave-wide 16-byte loa
 constexpr int FLAG_OFFSET = GEMV_TABLE_BYTES + PART_BYTES - 16;
 constexpr int MAP_BYTES = 1024;         // nested absmax only: the 256-entry map, taken from the end of the partial sums
 constexpr int MAP_OFFSET = FLAG_OFFSET - MAP_BYTES;
+// kernels with an epilogue (fp32 absmax only): sums of squares per (row of x, wave), below the flag
+constexpr int SUMSQ_BYTES = 2 * GEMV_WAVES * 4;
+constexpr int SUMSQ_OFFSET = FLAG_OFFSET - 16 - SUMSQ_BYTES;
+constexpr int PRE_BYTES = GEMV_THREADS * 4;  // EPI_RESID_NORM: a dword per thread
+constexpr int PRE_OFFSET = SUMSQ_OFFSET - PRE_BYTES;
 
 struct RowsPlan {
     int chunks;         // k chunks handled by one workgroup (waves along K)
@@ -106,8 +112,14 @@ __device__ __forceinline__ int reduce8_id(int lane) { return (lane & 1) | ((lane
 //                reads its value from the right lane through a DPP operand.  The 4-byte loads cost more than their
 //                share of the bytes (a vector memory instruction per KB of codes: the lm_head ran 5 us faster without
 //                them); this halves their number (lm_head 59.7 -> 58.4 us, [28672, 8192] 29.8 -> 28.0 with one row of x).
-template <int M, int U, bool NESTED, int MODE, bool PAIRED>
+// EPI (Epilogue flags; fp32 absmax, K not split over workgroups): what the thread that finishes an output does with
+//                it.  EPI_ROWSCALE: the producer's partial sums of squares are added up once per workgroup (one per
+//                thread, butterfly per wave, waves in order) while the first weights are on their way.
+//                EPI_RESID_NORM: a thread's outputs all belong to one row of x (M divides the workgroup size), so its
+//                squares add up in a register; lanes of equal m are added by a butterfly, waves in order.
+template <int M, int U, bool NESTED, int MODE, bool PAIRED, int EPI = EPI_NONE>
 __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a, RowsPlan p) {
+    static_assert(EPI == EPI_NONE || (!NESTED && GEMV_THREADS % M == 0 && M <= 2), "epilogues: fp32 absmax, M = 1, 2");
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -129,6 +141,8 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
     const int rl = wave / p.chunks;   // this wave's row lane
     const int64_t K = a.K;
     const int step = p.row_lanes;
+    float* sumsq_s = reinterpret_cast<float*>(smem + SUMSQ_OFFSET);
+    uint32_t* pre_s = reinterpret_cast<uint32_t*>(smem + PRE_OFFSET);
 
     for (int task = blockIdx.x; task < p.ntasks; task += gridDim.x) {
         const int band = task / p.splits;
@@ -141,6 +155,22 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
         const bool lane_on = wave_on && kchunk + klane < K;
         const int cnt = wave_on ? (r_end - r_begin - rl + step - 1) / step : 0;  // rows of this wave
 
+        // What the epilogue needs from memory is requested first and parked in LDS before the first barrier (the
+        // oldest requests of the wave: waiting for them waits for nothing else), so that no register holds it while
+        // the weights stream.  EPI_ROWSCALE (first task): this thread's share of the producer's partial sums of
+        // squares.  EPI_RESID_NORM: residual and norm weight of the thread's first output (it rarely has a second).
+        const bool first_task = !table_built;
+        float ssp[M];
+        uint32_t pre_res = 0, pre_w = 0;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            ssp[m] = 0.0f;
+            if ((EPI & EPI_ROWSCALE) && first_task && tid < a.epi.in_parts) ssp[m] = a.epi.in_sumsq[m * a.epi.in_parts + tid];
+        }
+        if ((EPI & EPI_RESID_NORM) && tid < (r_end - r_begin) * M) {
+            pre_res = a.epi.resid_in[(int64_t)(tid % M) * a.N + r_begin + tid / M];
+            pre_w = a.epi.norm_weight[r_begin + tid / M];
+        }
         // x for this lane's 32 k, all M rows
         uint32_t xr[M][16];
 #pragma unroll
@@ -200,6 +230,16 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
             if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
             table_built = true;
         }
+        if ((EPI & EPI_ROWSCALE) && first_task) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float ss = ssp[m];
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                if (lane == 0) sumsq_s[m * GEMV_WAVES + wave] = ss;
+            }
+        }
+        if (EPI & EPI_RESID_NORM) pre_s[tid] = pre_res | (pre_w << 16);  // a slot per thread, read back by the same thread
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
 
         // fp16 arithmetic: the lane's x values become fp16, scaled into range per row of x (here, behind the requests for
@@ -304,14 +344,61 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
         const int nrows = r_end - r_begin;
         // the last split may own fewer chunks than the others
         const int nchunks = min(p.chunks, (int)((K + CHUNK_K - 1) / CHUNK_K) - ks * p.chunks);
-        if (p.splits == 1) {
+        float rstd[M];  // EPI_ROWSCALE: 1 / rms of every row of x, from the wave sums left in LDS by the first task
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            rstd[m] = 1.0f;
+            if (EPI & EPI_ROWSCALE) {
+                float tot = 0.0f;
+#pragma unroll
+                for (int w = 0; w < GEMV_WAVES; ++w) tot += sumsq_s[m * GEMV_WAVES + w];
+                rstd[m] = rsqrtf(tot / (float)K + a.epi.eps);
+            }
+        }
+        // finished sum of output (r, m) of this band, bias included
+        auto finished = [&](int r, int m) {
+            float sum = 0.0f;
+            for (int c = 0; c < nchunks; ++c) sum += part[(r * p.chunks + c) * M + m];
+            if (EPI & EPI_ROWSCALE) sum *= rstd[m];
+            if (a.bias) sum += bf16_bits_to_f32(a.bias[r_begin + r]);
+            return sum;
+        };
+        if (EPI & EPI_SILU_PAIRS) {
+            // rows 2j, 2j + 1 of the band: gate j, up j (bands start and end on even rows)
+            for (int idx = tid; idx < (nrows / 2) * M; idx += GEMV_THREADS) {
+                const int j = idx / M, m = idx - j * M;
+                const float g = nf4x::round_bf16(finished(2 * j, m)), u = nf4x::round_bf16(finished(2 * j + 1, m));
+                a.out[(int64_t)m * (a.N / 2) + r_begin / 2 + j] = (uint16_t)nf4x::silu_mul_bf16(g, u);
+            }
+        } else if (EPI & EPI_RESID_NORM) {
+            float ss = 0.0f;  // every output of this thread has m = tid % M
             for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
                 const int r = idx / M, m = idx - r * M;
-                float sum = 0.0f;
-                for (int c = 0; c < nchunks; ++c) sum += part[(r * p.chunks + c) * M + m];
-                const int n = r_begin + r;
-                if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
-                a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
+                const int64_t at = (int64_t)m * a.N + r_begin + r;
+                const float d = nf4x::round_bf16(finished(r, m));
+                const bool pre = idx == tid;
+                const uint32_t parked = pre_s[tid];
+                const float old = bf16_bits_to_f32(pre ? parked & 0xffffu : (uint32_t)a.epi.resid_in[at]);
+                const float nw = bf16_bits_to_f32(pre ? parked >> 16 : (uint32_t)a.epi.norm_weight[r_begin + r]);
+                const float res = nf4x::resid_add(old, d);
+                a.epi.resid_out[at] = (uint16_t)f32_to_bf16_bits(res);
+                a.epi.xnext_out[at] = (uint16_t)f32_to_bf16_bits(res * nw);
+                ss = fmaf(res, res, ss);
+            }
+#pragma unroll
+            for (int o = 32; o >= M; o >>= 1) ss += __shfl_xor(ss, o, 64);  // lanes of equal m (M = 1, 2)
+            if (lane < M) sumsq_s[lane * GEMV_WAVES + wave] = ss;
+            __syncthreads();
+            if (tid < M) {
+                float tot = 0.0f;
+#pragma unroll
+                for (int w = 0; w < GEMV_WAVES; ++w) tot += sumsq_s[tid * GEMV_WAVES + w];
+                a.epi.out_sumsq[tid * p.nbands + band] = tot;
+            }
+        } else if (p.splits == 1) {
+            for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                const int r = idx / M, m = idx - r * M;
+                a.out[(int64_t)m * a.N + r_begin + r] = (uint16_t)f32_to_bf16_bits(finished(r, m));
             }
         } else {
             for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
@@ -352,77 +439,94 @@ int rows_splits(int64_t K) {
     return (int)((nch + GEMV_WAVES - 1) / GEMV_WAVES);
 }
 
-RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested) {
+RowsPlan make_rows_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested, int epi = EPI_NONE) {
     RowsPlan p;
     p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
     const int nch = (int)((K + CHUNK_K - 1) / CHUNK_K);
     p.splits = rows_splits(K);
     p.chunks = (nch + p.splits - 1) / p.splits;
     p.row_lanes = GEMV_WAVES / p.chunks;
-    const int part_bytes = PART_BYTES - 64 - (nested ? MAP_BYTES : 0);
-    const int cap = (part_bytes / (p.chunks * M * 4)) / p.row_lanes * p.row_lanes;
+    // rows of a band come in multiples of `unit`: the row lanes, and whole (gate, up) pairs where those are merged
+    const int unit = (epi & EPI_SILU_PAIRS) && p.row_lanes % 2 ? 2 * p.row_lanes : p.row_lanes;
+    const int part_bytes = PART_BYTES - 64 - (nested ? MAP_BYTES : 0) - (epi ? SUMSQ_BYTES + 16 + PRE_BYTES : 0);
+    const int cap = (part_bytes / (p.chunks * M * 4)) / unit * unit;
     int bands_target = slots / p.splits;
     if (bands_target < 1) bands_target = 1;
     // one task per resident workgroup if its partial sums fit in LDS, else 2, 3, ... balanced rounds
     int64_t rpb = cap;
     for (int rounds = 1; rounds <= 64; ++rounds) {
         int64_t r = (N + (int64_t)rounds * bands_target - 1) / ((int64_t)rounds * bands_target);
-        r = (r + p.row_lanes - 1) / p.row_lanes * p.row_lanes;
+        r = (r + unit - 1) / unit * unit;
         if (r <= cap) {
             rpb = r;
             break;
         }
     }
-    if (rpb < p.row_lanes) rpb = p.row_lanes;
+    if (rpb < unit) rpb = unit;
     p.rows_per_band = (int)rpb;
     p.nbands = (int)((N + rpb - 1) / rpb);
     p.ntasks = p.nbands * p.splits;
     return p;
 }
 
-template <int M, int U, bool NESTED, bool PAIRED>
+template <int M, int U, bool NESTED, bool PAIRED, int EPI>
 hipError_t launch_p(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int mode = gemv_arith_mode(a.K, true);
     if (mode == ARITH_EXACT)
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT, PAIRED>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else if (mode == ARITH_F16)
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16, PAIRED>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16, PAIRED>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
-template <int M, int U, bool NESTED>
+template <int M, int U, bool NESTED, int EPI>
 hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     if constexpr (!NESTED && M == 1)  // measured: 1-2 us on weights of 30 MB and more with one row of x, a loss with two
-        if (p.aligned) return launch_p<M, U, false, true>(a, p, grid, stream);
-    return launch_p<M, U, NESTED, false>(a, p, grid, stream);
+        if (p.aligned) return launch_p<M, U, false, true, EPI>(a, p, grid, stream);
+    return launch_p<M, U, NESTED, false, EPI>(a, p, grid, stream);
 }
 
 // U = rows in flight per wave: as many as the wave has to do, within the register budget
 // (8 only for M = 1).
-template <int M, bool NESTED>
+template <int M, bool NESTED, int EPI>
 hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int cnt = p.rows_per_band / p.row_lanes;  // rows per wave and task
-    if constexpr (M == 1)
-        if (!NESTED && cnt >= 8) return launch_u<1, 8, NESTED>(a, p, grid, stream);  // nested: one more register per slot
+    // eight rows in flight fill the register file to the last register: one more live value (nested absmax: a register
+    // per slot; an epilogue: its pointers and flags) spills, and a kernel that uses scratch memory starts 2-3 us later
+    if constexpr (M == 1 && !NESTED && EPI == EPI_NONE)
+        if (cnt >= 8) return launch_u<1, 8, NESTED, EPI>(a, p, grid, stream);
     if constexpr (M <= 2)
-        if (cnt >= 4) return launch_u<M, 4, NESTED>(a, p, grid, stream);
-    return launch_u<M, 2, NESTED>(a, p, grid, stream);
+        if (cnt >= 4) return launch_u<M, 4, NESTED, EPI>(a, p, grid, stream);
+    return launch_u<M, 2, NESTED, EPI>(a, p, grid, stream);
 }
 
-template <bool NESTED>
+template <bool NESTED, int EPI>
 hipError_t launch_n(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     // M = 3 and 4 are served by the four-rows-per-quad kernel
-    return a.M == 2 ? launch_m<2, NESTED>(a, p, grid, stream) : launch_m<1, NESTED>(a, p, grid, stream);
+    return a.M == 2 ? launch_m<2, NESTED, EPI>(a, p, grid, stream) : launch_m<1, NESTED, EPI>(a, p, grid, stream);
+}
+
+template <int M, int U, int MODE, int EPI>
+hipError_t allow_lds_epi() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, MODE, false, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    if constexpr (M == 1)
+        if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, MODE, true, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    return hipSuccess;
 }
 
 template <int M, int U, int MODE>
 hipError_t allow_lds_mode() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, MODE, false>, SMEM_BYTES)) != hipSuccess) return e;
-    if constexpr (M == 1)
-        if ((e = gemv_allow_lds(gemv_rows_kernel<M, U, false, MODE, true>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = allow_lds_epi<M, U, MODE, EPI_NONE>()) != hipSuccess) return e;
+    if constexpr (U <= 4) {
+        if ((e = allow_lds_epi<M, U, MODE, EPI_ROWSCALE>()) != hipSuccess) return e;
+        if ((e = allow_lds_epi<M, U, MODE, EPI_ROWSCALE | EPI_SILU_PAIRS>()) != hipSuccess) return e;
+        if ((e = allow_lds_epi<M, U, MODE, EPI_SILU_PAIRS>()) != hipSuccess) return e;
+        if ((e = allow_lds_epi<M, U, MODE, EPI_RESID_NORM>()) != hipSuccess) return e;
+    }
     return gemv_allow_lds(gemv_rows_kernel<M, U, true, MODE, false>, SMEM_BYTES);
 }
 
@@ -457,14 +561,37 @@ hipError_t gemv_rows_setup() {
     return allow_lds_m<2>();
 }
 
-hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {
+// epilogues of the row kernel: fp32 absmax, whole rows of x in one workgroup; (gate, up) pairs need an even N
+bool gemv_rows_epilogue_possible(const MatmulArgs& a) {
+    if (a.epi.flags == EPI_NONE) return true;
+    if (a.nested.q || rows_splits(a.K) != 1) return false;
+    if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > GEMV_THREADS) return false;
+    return !(a.epi.flags & EPI_SILU_PAIRS) || a.N % 2 == 0;
+}
+
+int gemv_rows_norm_parts(int64_t M, int64_t N, int64_t K, int cus) {
+    if (rows_splits(K) != 1) return 0;
     int slots = 2 * cus;
     if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
-    const RowsPlan p = make_rows_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
+    return make_rows_plan((int)M, N, K, 6, slots, false, EPI_RESID_NORM).nbands;
+}
+
+hipError_t launch_gemv_rows(const MatmulArgs& a, int cus, hipStream_t stream) {
+    if (!gemv_rows_epilogue_possible(a)) return hipErrorNotSupported;
+    int slots = 2 * cus;
+    if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
+    const RowsPlan p = make_rows_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr, a.epi.flags);
     // one arrival counter per band when K is split across workgroups
     if (p.splits > 1 && p.nbands > GEMV_COUNTER_BYTES / 4) return hipErrorInvalidValue;
     const int grid = p.ntasks < slots ? p.ntasks : slots;
-    return a.nested.q ? launch_n<true>(a, p, grid, stream) : launch_n<false>(a, p, grid, stream);
+    switch (a.epi.flags) {
+        case EPI_NONE: return a.nested.q ? launch_n<true, EPI_NONE>(a, p, grid, stream) : launch_n<false, EPI_NONE>(a, p, grid, stream);
+        case EPI_ROWSCALE: return launch_n<false, EPI_ROWSCALE>(a, p, grid, stream);
+        case EPI_ROWSCALE | EPI_SILU_PAIRS: return launch_n<false, EPI_ROWSCALE | EPI_SILU_PAIRS>(a, p, grid, stream);
+        case EPI_SILU_PAIRS: return launch_n<false, EPI_SILU_PAIRS>(a, p, grid, stream);
+        case EPI_RESID_NORM: return launch_n<false, EPI_RESID_NORM>(a, p, grid, stream);
+    }
+    return hipErrorNotSupported;
 }
 
 }  // namespace nf4

@@ -40,6 +40,11 @@ class LlamaConfig:
     max_seq: int = 640
     fused_projections: bool = False
     hip_glue: bool = False
+    # with fused_projections: rows 2j / 2j+1 of the gate-up weight are row j of the gate / of the up projection (instead
+    # of gate rows first, up rows after), so that the thread finishing a pair of outputs can apply SiLU(gate) * up itself
+    gate_up_interleaved: bool = False
+    # with hip_glue: let the 4-bit decode kernels' epilogues do the residual add, RMSNorm and SiLU * up where they can
+    linear_epilogues: bool = True
 
     @property
     def head_dim(self) -> int:
@@ -117,7 +122,10 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(cfg.d_ff, cfg.d_model, bias=False)
 
     def forward(self, x):
-        if self.cfg.fused_projections:
+        if self.cfg.fused_projections and self.cfg.gate_up_interleaved:
+            gu = self.gate_up_proj(x)
+            gate, up = gu[..., 0::2], gu[..., 1::2]
+        elif self.cfg.fused_projections:
             gate, up = self.gate_up_proj(x).chunk(2, dim=-1)
         else:
             gate, up = self.gate_proj(x), self.up_proj(x)
@@ -163,6 +171,10 @@ class Llama(nn.Module):
         cfg = self.cfg
         H, Hkv, eps = cfg.n_head, cfg.n_kv_head, cfg.norm_eps
         x = self.wte(idx)[:, 0, :].contiguous()
+        if cfg.linear_epilogues and cfg.fused_projections and cfg.gate_up_interleaved and x.shape[0] <= 2:
+            out = self._decode_step_epilogues(x, pos, kcache, vcache)
+            if out is not None:
+                return out
         delta = None
         for i, blk in enumerate(self.blocks):
             h = glue.add_rmsnorm(x, delta, blk.norm_1.weight, eps)
@@ -176,8 +188,40 @@ class Llama(nn.Module):
             h = glue.add_rmsnorm(x, delta, blk.norm_2.weight, eps)
             m = blk.mlp
             gate_up = m.gate_up_proj(h) if cfg.fused_projections else torch.cat((m.gate_proj(h), m.up_proj(h)), dim=-1)
-            delta = m.down_proj(glue.silu_mul(gate_up))
+            delta = m.down_proj(glue.silu_mul(gate_up, pairs=cfg.fused_projections and cfg.gate_up_interleaved))
         return self.lm_head(glue.add_rmsnorm(x, delta, self.norm_f.weight, eps))
+
+    def _decode_step_epilogues(self, x, pos, kcache, vcache):
+        """The single-token forward with the neighbours of every linear done in that linear's epilogue
+        (``hip_matmul_nf4_epilogue``): the output and down projections add the residual, write the next norm's
+        input times its weight and leave partial sums of squares; the QKV, gate-up and lm_head projections scale their
+        sums by the 1 / rms those give, and the gate-up projection applies SiLU(gate) * up to its pairs of outputs.
+        Per layer four linears and the attention kernel.  Returns None (before anything is launched) unless every
+        linear runs as the 4-bit operator with fp32 absmax at a shape the kernels take."""
+        from . import glue
+        from .transforms import quantization as Q
+
+        cfg = self.cfg
+        H, Hkv, eps = cfg.n_head, cfg.n_kv_head, cfg.norm_eps
+        lins = [l for blk in self.blocks for l in (blk.attn.qkv_proj, blk.attn.o_proj, blk.mlp.gate_up_proj, blk.mlp.down_proj)]
+        args = {id(l): _planned_nf4(l) for l in lins + [self.lm_head]}
+        if any(a is None for a in args.values()) or not _epilogues_served(x.shape[0], lins + [self.lm_head]):
+            return None
+        ep = Q.hip_matmul_nf4_epilogue
+        r = x
+        xn = ss = None
+        for i, blk in enumerate(self.blocks):
+            a, m = blk.attn, blk.mlp
+            if i == 0:
+                qkv = a.qkv_proj(glue.add_rmsnorm(r, None, blk.norm_1.weight, eps))
+            else:
+                qkv = ep(xn, *args[id(a.qkv_proj)], rowscale=(ss, eps))
+            y = glue.attention_decode(qkv, pos, self.rope_cos, self.rope_sin, kcache[i], vcache[i], H, Hkv)
+            r, xn, ss = ep(y, *args[id(a.o_proj)], resid_norm=(r, blk.norm_2.weight))
+            h = ep(xn, *args[id(m.gate_up_proj)], rowscale=(ss, eps), silu_pairs=True)
+            nxt = self.blocks[i + 1].norm_1.weight if i + 1 < len(self.blocks) else self.norm_f.weight
+            r, xn, ss = ep(h, *args[id(m.down_proj)], resid_norm=(r, nxt))
+        return ep(xn, *args[id(self.lm_head)], rowscale=(ss, eps))
 
     def forward(self, idx, pos, kcache, vcache):
         if self.cfg.hip_glue and idx.shape[1] == 1 and idx.is_cuda and self.wte.weight.dtype == torch.bfloat16:
@@ -191,6 +235,25 @@ class Llama(nn.Module):
         for i, blk in enumerate(self.blocks):
             x = blk(x, pos, cos, sin, bias, kcache[i], vcache[i])
         return self.lm_head(self.norm_f(x[:, -1:, :])).squeeze(1)
+
+
+def _planned_nf4(lin: nn.Linear):
+    """``(qweight, bias, absmax, quant_map, blocksize, dtype, shape)`` when ``lin`` runs as the operator
+    ``hip_matmul_nf4`` (4-bit weight, fp32 absmax) in the compiled module, else None."""
+    planned = getattr(lin.weight, "_planned_operator", None)
+    if planned is None or planned[0] != "hip_matmul_nf4":
+        return None
+    _, packed, rest = planned
+    return (packed, lin.bias, *rest)
+
+
+def _epilogues_served(rows: int, linears) -> bool:
+    """Do the decode kernels take an epilogue at ``rows`` rows of x on every one of these weights?  (Asked of the
+    library through its own planning function, before the step launches anything.)"""
+    from . import _lib
+
+    lib = _lib.load()
+    return all(lib.nf4hip_gemv_norm_parts(rows, l.out_features, l.in_features) > 0 for l in linears)
 
 
 def build_llama(cfg: LlamaConfig, device="cuda", dtype=torch.bfloat16, seed: int = 0) -> Llama:
@@ -308,7 +371,11 @@ def fuse_state_dict(sd: dict, cfg: LlamaConfig) -> dict:
             out[base + "qkv_proj.weight"] = torch.cat([v, sd[base + "k_proj.weight"], sd[base + "v_proj.weight"]], dim=0)
         elif k.endswith("gate_proj.weight"):
             base = k[: -len("gate_proj.weight")]
-            out[base + "gate_up_proj.weight"] = torch.cat([v, sd[base + "up_proj.weight"]], dim=0)
+            up = sd[base + "up_proj.weight"]
+            if cfg.gate_up_interleaved:  # rows 2j / 2j+1 = gate row j / up row j
+                out[base + "gate_up_proj.weight"] = torch.stack([v, up], dim=1).reshape(2 * v.shape[0], v.shape[1])
+            else:
+                out[base + "gate_up_proj.weight"] = torch.cat([v, up], dim=0)
         else:
             out[k] = v
     return out

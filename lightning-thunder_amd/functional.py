@@ -13,6 +13,7 @@ queued on ``torch.cuda.current_stream()`` and nothing synchronises.
 
 from __future__ import annotations
 
+import ctypes
 import math
 from dataclasses import dataclass
 
@@ -530,3 +531,78 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
                 _lib.check(fn(x2.data_ptr() + 2 * m0 * K, _lib.BF16, mc, qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(), bptr,
                               N, K, blocksize, out.data_ptr() + 2 * m0 * N, ws_ptr, ws_bytes, stream))  # fmt: skip
     return out.reshape(*x.shape[:-1], N)
+
+
+# ---- the decode kernels with an epilogue ---------------------------------------------------------------------
+
+
+def matmul_nf4_epilogue(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, *, rowscale=None, silu_pairs=False,
+                        resid_norm=None):
+    """``matmul_nf4`` at decode shapes with the step that follows (or precedes) the linear in a decoder layer done by
+    the thread that finishes each output (``nf4hip_gemv_epilogue``), one launch instead of two:
+
+    * ``resid_norm=(resid, norm_weight)``: ``r = resid + linear(x)``; returns ``(r, xnext, sumsq)`` with
+      ``xnext = r * norm_weight`` (not yet divided by the rms) and ``sumsq`` [rows, parts] partial sums of ``r**2``.
+    * ``rowscale=(sumsq, eps)``: ``x`` is such an ``xnext``; the sums are multiplied by ``rsqrt(sumsq.sum(-1) / K + eps)``,
+      which makes the result ``linear(rms_norm(r) * norm_weight)``.
+    * ``silu_pairs``: weight rows 2j / 2j+1 are gate row j / up row j; returns ``silu(gate) * up`` [rows, N/2].
+
+    Returns None where the library does not serve the case (more than two rows of x, nested absmax, K beyond one
+    workgroup's reach, other dtypes): the caller then runs ``matmul_nf4`` and the step by itself."""
+    N, K = (int(s) for s in shape)
+    x2 = x.reshape(-1, K)
+    M = x2.shape[0]
+    if isinstance(absmax, NestedAbsmax) or M > 16 or not x2.is_cuda:
+        return None
+    if fused_route(x2, bias, blocksize, dtype, (N, K)) != "gemv":
+        return None
+    lib = _lib.load()
+    _require_gpu(x2, qweight, quant_map, bias, absmax)
+    x2, qweight = _aligned(x2), _aligned(qweight)
+    quant_map, absmax = _aligned(quant_map.to(torch.float32)), _aligned(absmax.to(torch.float32))
+    if qweight.numel() < N * K // 2 or absmax.numel() < N * K // blocksize:
+        raise ValueError(f"qweight / absmax hold {qweight.numel()} / {absmax.numel()} entries, too few for {shape}")
+    b = None if bias is None else bias.contiguous()
+    epi = _lib.Epilogue()
+    keep = []  # tensors whose addresses the struct holds
+    with _on_device(x2.device):
+        out = None
+        if rowscale is not None:
+            sumsq, eps = rowscale
+            if sumsq.dtype != torch.float32 or sumsq.dim() != 2 or sumsq.shape[0] != M or not sumsq.is_contiguous():
+                raise ValueError(f"rowscale: sumsq must be a contiguous fp32 [rows, parts] tensor, got {sumsq.dtype} {tuple(sumsq.shape)}")
+            epi.flags |= _lib.EPI_ROWSCALE
+            epi.eps, epi.in_sumsq, epi.in_parts = float(eps), sumsq.data_ptr(), sumsq.shape[1]
+            keep.append(sumsq)
+        if silu_pairs:
+            if N % 2:
+                return None
+            epi.flags |= _lib.EPI_SILU_PAIRS
+        if resid_norm is not None:
+            resid, norm_weight = resid_norm
+            if resid.shape != (M, N) or resid.dtype != torch.bfloat16 or norm_weight.shape != (N,) or norm_weight.dtype != torch.bfloat16:
+                raise ValueError(f"resid_norm: need bf16 resid [{M}, {N}] and norm_weight [{N}], got {tuple(resid.shape)} {resid.dtype}, "
+                                 f"{tuple(norm_weight.shape)} {norm_weight.dtype}")
+            parts = lib.nf4hip_gemv_norm_parts(M, N, K)
+            if parts <= 0:
+                return None
+            resid, norm_weight = resid.contiguous(), norm_weight.contiguous()
+            r_out, xnext = torch.empty_like(resid), torch.empty_like(resid)
+            out_sumsq = torch.empty((M, parts), dtype=torch.float32, device=x2.device)
+            epi.flags |= _lib.EPI_RESID_NORM
+            epi.resid_in, epi.norm_weight = resid.data_ptr(), norm_weight.data_ptr()
+            epi.resid_out, epi.xnext_out, epi.out_sumsq = r_out.data_ptr(), xnext.data_ptr(), out_sumsq.data_ptr()
+            keep += [resid, norm_weight]
+        else:
+            out = torch.empty((M, N // 2 if silu_pairs else N), dtype=torch.bfloat16, device=x2.device)
+        stream = _stream()
+        ws = _gemv_workspace(x2.device, lib.nf4hip_gemv_workspace_bytes(M, N, K), stream)
+        rc = lib.nf4hip_gemv_epilogue(x2.data_ptr(), _lib.BF16, M, qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(),
+                                      None if b is None else b.data_ptr(), N, K, blocksize, None if out is None else out.data_ptr(),
+                                      ws.data_ptr(), ws.numel(), ctypes.byref(epi), stream)
+    if rc == _lib.E_SHAPE:
+        return None
+    _lib.check(rc)
+    if resid_norm is not None:
+        return r_out, xnext, out_sumsq
+    return out.reshape(*x.shape[:-1], out.shape[-1])

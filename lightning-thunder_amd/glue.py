@@ -27,6 +27,7 @@ SYMBOLS = {
     "nf4hip_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32]),
     "nf4hip_decode_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, ctypes.c_size_t, _vp]),
     "nf4hip_decode_silu_mul": (_i32, [_vp, _i64, _i64, _vp, _vp]),
+    "nf4hip_decode_silu_mul_pairs": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "nf4hip_decode_argmax": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp]),
 }
 
@@ -127,15 +128,17 @@ def attention_decode(qkv: torch.Tensor, pos: torch.Tensor, cos: torch.Tensor, si
     return out
 
 
-def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """``silu(gate) * up`` for ``gate_up`` [rows, 2 dff] = (gate | up).  Returns [rows, dff]."""
+def silu_mul(gate_up: torch.Tensor, pairs: bool = False) -> torch.Tensor:
+    """``silu(gate) * up`` for ``gate_up`` [rows, 2 dff] = (gate | up), or with ``pairs`` gate and up interleaved
+    (column 2j = gate j, column 2j + 1 = up j).  Returns [rows, dff]."""
     lib = load()
     _bf16_cuda(gate_up)
     rows, two = gate_up.shape
     dff = two // 2
     out = torch.empty((rows, dff), dtype=torch.bfloat16, device=gate_up.device)
+    fn = lib.nf4hip_decode_silu_mul_pairs if pairs else lib.nf4hip_decode_silu_mul
     with torch.cuda.device(gate_up.device):
-        _check(lib, lib.nf4hip_decode_silu_mul(gate_up.data_ptr(), rows, dff, out.data_ptr(), _stream(gate_up)))
+        _check(lib, fn(gate_up.data_ptr(), rows, dff, out.data_ptr(), _stream(gate_up)))
     return out
 
 

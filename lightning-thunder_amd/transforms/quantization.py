@@ -36,6 +36,9 @@ hip_matmul_nf4: extend.Symbol | None = None
 hip_quantize_nf4: extend.Symbol | None = None
 hip_dequantize_nf4: extend.Symbol | None = None
 hip_matmul_nf4_dq: extend.Symbol | None = None
+# hip_matmul_nf4 with an epilogue: the residual add / RMSNorm / SiLU * up next to the linear done by the decode kernel
+# (no counterpart in the reference, whose other executors fuse those steps around bnb_matmul_nf4)
+hip_matmul_nf4_epilogue: extend.Symbol | None = None
 hip_quantize_nf4_dq: extend.Symbol | None = None
 hip_dequantize_nf4_dq: extend.Symbol | None = None
 
@@ -82,6 +85,25 @@ def hip_matmul_nf4_dq_impl(x, qweight, bias, absmax_q, nested_absmax, nested_qua
                                     blocksize, nested_blocksize, dtype, shape)
 
 
+def hip_matmul_nf4_epilogue_meta(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=None, silu_pairs=False,
+                                 resid_norm=None):
+    _check_matmul_shapes(x, shape)
+    n = shape[0] // 2 if silu_pairs else shape[0]
+    out = TensorProxy(like=x, shape=(*x.shape[:-1], n))
+    if resid_norm is None:
+        return out
+    rows = _numel(x.shape[:-1])
+    return out, TensorProxy(like=x, shape=(*x.shape[:-1], n)), _plain(x, (rows, 512), torch.float32)
+
+
+def hip_matmul_nf4_epilogue_impl(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=None, silu_pairs=False,
+                                 resid_norm=None):
+    """``hip_matmul_nf4`` with the decoder layer's neighbouring step done in the kernel's epilogue
+    (``functional.matmul_nf4_epilogue``); None where the kernels do not serve the case."""
+    return functional.matmul_nf4_epilogue(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=rowscale,
+                                          silu_pairs=silu_pairs, resid_norm=resid_norm)
+
+
 def hip_quantize_nf4_impl(w, blocksize=64):
     return functional.quantize_nf4(w, blocksize)
 
@@ -121,13 +143,15 @@ def get_hip_nf4_executor() -> extend.OperatorExecutor:
     (thunder/transforms/quantization.py:19-44).  Loading the HIP library is part of it: a missing
     or mismatching ``libnf4hip.so`` fails here, not at the first forward."""
     global hip_nf4_executor, hip_matmul_nf4, hip_quantize_nf4, hip_dequantize_nf4
-    global hip_matmul_nf4_dq, hip_quantize_nf4_dq, hip_dequantize_nf4_dq
+    global hip_matmul_nf4_dq, hip_quantize_nf4_dq, hip_dequantize_nf4_dq, hip_matmul_nf4_epilogue
     if hip_nf4_executor is None:
         from .. import _lib
 
         _lib.load()
         ex = extend.OperatorExecutor("quant_hip_nf4", version=0.1)
         hip_matmul_nf4 = ex.register_operator("hip_matmul_nf4", meta=hip_matmul_nf4_meta, fn=hip_matmul_nf4_impl)
+        hip_matmul_nf4_epilogue = ex.register_operator("hip_matmul_nf4_epilogue", meta=hip_matmul_nf4_epilogue_meta,
+                                                       fn=hip_matmul_nf4_epilogue_impl)
         hip_quantize_nf4 = ex.register_operator("hip_quantize_nf4", meta=_quantize_meta, fn=hip_quantize_nf4_impl)
         hip_dequantize_nf4 = ex.register_operator("hip_dequantize_nf4", meta=_dequantize_meta, fn=hip_dequantize_nf4_impl)
         hip_matmul_nf4_dq = ex.register_operator("hip_matmul_nf4_dq", meta=hip_matmul_nf4_dq_meta, fn=hip_matmul_nf4_dq_impl)

@@ -171,3 +171,29 @@ def test_fused_route_rules(ta):
     assert route(1, 2, 2) == "dequant+linear"
     assert route(1, 64, 4096, bias=torch.zeros(64)) == "dequant+linear"  # fp32 bias with bf16 x
     _ = ctypes  # (imported for readers who want to poke at the library by hand)
+
+
+def test_epilogue_argument_errors(ta):
+    """nf4hip_gemv_epilogue validates its struct before any HIP call; what the kernels do not serve is E_SHAPE."""
+    import ctypes
+
+    L = ta._lib
+    lib = L.load()
+    A = 1 << 20  # fake, aligned device address: validation dereferences nothing
+    ws = lib.nf4hip_gemv_workspace_bytes(1, 64, 4096)
+    args = (A, L.BF16, 1, A, A, A, None, 64, 4096, 64, A, A, ws)
+    err = lambda: lib.nf4hip_last_error().decode()
+    call = lambda e, a=args: lib.nf4hip_gemv_epilogue(*a, ctypes.byref(e), None)
+    assert lib.nf4hip_gemv_epilogue(*args, None, None) == L.E_NULL
+    assert call(L.Epilogue(8)) == L.E_SHAPE and "flags" in err()
+    assert call(L.Epilogue(L.EPI_RESID_NORM | L.EPI_ROWSCALE)) == L.E_SHAPE and "stands alone" in err()
+    assert call(L.Epilogue(L.EPI_ROWSCALE)) == L.E_NULL and "in_sumsq" in err()
+    assert call(L.Epilogue(L.EPI_ROWSCALE, 1e-5, A + 2, 8)) == L.E_ALIGN
+    assert call(L.Epilogue(L.EPI_RESID_NORM, 0.0, None, 0, A, A, A, None, A)) == L.E_NULL and "xnext_out" in err()
+    assert call(L.Epilogue(L.EPI_RESID_NORM, 0.0, None, 0, A, A, A + 1, A, A)) == L.E_ALIGN
+    args3 = (A, L.BF16, 3, A, A, A, None, 64, 4096, 64, A, A, 1 << 30)
+    assert call(L.Epilogue(L.EPI_SILU_PAIRS), args3) == L.E_SHAPE and "not served" in err()
+    long_k = (A, L.BF16, 1, A, A, A, None, 64, 20480, 64, A, A, 1 << 30)
+    assert call(L.Epilogue(L.EPI_SILU_PAIRS), long_k) == L.E_SHAPE and "not served" in err()
+    assert call(L.Epilogue(L.EPI_ROWSCALE, 1e-5, A, 513)) == L.E_SHAPE  # more partial sums than a workgroup has threads
+    assert lib.nf4hip_gemv_norm_parts(3, 64, 4096) == 0 and lib.nf4hip_gemv_norm_parts(1, 64, 20480) == 0

@@ -1,0 +1,209 @@
+"""GPU tests of the decode kernels' epilogues (nf4hip_gemv_epilogue), called through the C ABI by
+``functional.matmul_nf4_epilogue``.
+
+What an epilogue does to a finished sum is element-wise arithmetic on bf16 values, so wherever the two-step route
+(nf4hip_gemv, then the step as a kernel of its own) computes the same thing the bits must agree: SiLU * up on pairs of
+outputs, the new residual, the next norm's input times its weight.  The row scale (1 / rms applied to the finished
+sums instead of to every element of x) is floating-point work in another order: held to the matmul's bar,
+rtol = atol = 2e-2 against float64 on the same inputs.
+"""
+
+import importlib
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def _randn(shape, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * std).to(torch.bfloat16)
+
+
+@pytest.fixture(scope="module")
+def F(ta):
+    return ta.functional
+
+
+@pytest.fixture(scope="module")
+def glue():
+    return importlib.import_module("lightning-thunder_amd.glue")
+
+
+def _quantized(ta, N, K, seed):
+    qw, absmax, code = ta.quantize_nf4(_randn((N, K), seed, 0.02).to(DEV))
+    return qw, absmax, code
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16)
+
+
+# (N, K): small, the Llama-3-8B gate-up and down shapes, K in the fp16-code-book range, ragged sizes
+PAIR_SHAPES = [(1024, 512), (28672, 4096), (2048, 14336), (272, 2080)]
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("shape", PAIR_SHAPES)
+def test_silu_pairs_gives_the_two_step_bits(ta, F, glue, M, shape):
+    N, K = shape
+    print(f"epilogue silu_pairs M={M} N={N} K={K}", flush=True)
+    qw, absmax, code = _quantized(ta, N, K, seed=N + K)
+    x = _randn((M, K), seed=3 * N + M).to(DEV)
+    bias = _randn((N,), seed=N, std=0.5).to(DEV) if N == 272 else None
+    two_step = glue.silu_mul(F.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K)), pairs=True)
+    out = F.matmul_nf4_epilogue(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K), silu_pairs=True)
+    torch.cuda.synchronize()
+    assert out is not None and out.shape == (M, N // 2)
+    assert torch.equal(_bits(out), _bits(two_step))
+
+
+# (N, K): Llama-3-8B output and down projections, ragged, the longest K one workgroup holds
+RESID_SHAPES = [(4096, 4096), (4096, 14336), (517, 1056), (256, 16384)]
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("shape", RESID_SHAPES)
+def test_resid_norm_epilogue(ta, F, M, shape):
+    N, K = shape
+    print(f"epilogue resid_norm M={M} N={N} K={K}", flush=True)
+    qw, absmax, code = _quantized(ta, N, K, seed=N + K + 1)
+    x = _randn((M, K), seed=5 * N + M).to(DEV)
+    resid = _randn((M, N), seed=7 * N + M, std=2.0).to(DEV)
+    nw = (1.0 + _randn((N,), seed=N, std=0.1).float()).to(torch.bfloat16).to(DEV)
+    bias = _randn((N,), seed=N + 1, std=0.5).to(DEV) if N == 517 else None
+    resid_before = resid.clone()
+    got = F.matmul_nf4_epilogue(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw))
+    assert got is not None
+    r, xnext, sumsq = got
+    delta = F.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))  # the plain kernel's bf16 output
+    torch.cuda.synchronize()
+    r_ref = (resid_before.float() + delta.float()).to(torch.bfloat16)
+    assert torch.equal(resid, resid_before)
+    assert torch.equal(_bits(r), _bits(r_ref)), "resid_out is not bf16(resid + bf16(linear))"
+    assert torch.equal(_bits(xnext), _bits((r_ref.float() * nw.float()).to(torch.bfloat16))), "xnext is not bf16(r * norm_weight)"
+    assert sumsq.shape == (M, ta._lib.load().nf4hip_gemv_norm_parts(M, N, K))
+    torch.testing.assert_close(sumsq.double().sum(-1), r_ref.double().pow(2).sum(-1), rtol=1e-5, atol=0)
+
+
+def _deq(oracle, qw, absmax, code, shape):
+    return oracle.dequantize_4bit_eager(qw.cpu(), absmax.cpu(), code.cpu(), 64, torch.bfloat16, shape).double()
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("shape", [(6144, 4096), (1024, 512), (28672, 4096), (128256, 4096), (304, 8192)])
+def test_rowscale_epilogue_against_float64(ta, F, glue, oracle, M, silu, shape):
+    """A producer's (xnext, sumsq) made by hand from a residual r: the consumer must give linear(rms_norm(r) * w)."""
+    N, K = shape
+    if N == 128256 and (silu or M == 2):
+        pytest.skip("the lm_head is checked once")
+    print(f"epilogue rowscale M={M} N={N} K={K} silu={silu}", flush=True)
+    qw, absmax, code = _quantized(ta, N, K, seed=N + K + 2)
+    r = _randn((M, K), seed=11 * N + M, std=3.0)
+    nw = (1.0 + _randn((K,), seed=K, std=0.1).float()).to(torch.bfloat16)
+    eps = 1e-5
+    xnext = (r.float() * nw.float()).to(torch.bfloat16)
+    parts = 37  # any split of the sum of squares into partial sums will do
+    sq = r.double().pow(2)
+    sumsq = torch.stack([c.sum(-1) for c in sq.chunk(parts, dim=-1)], dim=-1).float().contiguous()
+    out = F.matmul_nf4_epilogue(xnext.to(DEV), qw, None, absmax, code, 64, torch.bfloat16, (N, K), rowscale=(sumsq.to(DEV), eps))
+    torch.cuda.synchronize()
+    assert out is not None
+    h = r.double() * torch.rsqrt(sq.mean(-1, keepdim=True) + eps) * nw.double()
+    y = h @ _deq(oracle, qw, absmax, code, (N, K)).t()
+    torch.testing.assert_close(out.cpu().double(), y, **TOL)
+    if silu:  # SiLU * up on the scaled sums: the bits of the element-wise kernel on the scaled output above
+        both = F.matmul_nf4_epilogue(xnext.to(DEV), qw, None, absmax, code, 64, torch.bfloat16, (N, K), rowscale=(sumsq.to(DEV), eps),
+                                     silu_pairs=True)
+        assert both is not None and torch.equal(_bits(both), _bits(glue.silu_mul(out, pairs=True)))
+
+
+def test_chain_of_epilogues_is_a_decoder_layer_tail(ta, F, oracle):
+    """o_proj (residual add, next norm's input) -> gate-up (row scale, SiLU * up) -> down (residual add) against the same
+    arithmetic in float64 with bf16 roundings only where tensors are stored."""
+    d, dff, M = 1024, 2048, 2
+    print("epilogue chain", flush=True)
+    qo, ao, code = _quantized(ta, d, d, seed=1)
+    qg, ag, _ = _quantized(ta, 2 * dff, d, seed=2)
+    qd, ad, _ = _quantized(ta, d, dff, seed=3)
+    y = _randn((M, d), 4)
+    r0 = _randn((M, d), 5, 2.0)
+    w2 = (1.0 + _randn((d,), 6, 0.1).float()).to(torch.bfloat16)
+    w1 = (1.0 + _randn((d,), 7, 0.1).float()).to(torch.bfloat16)
+    eps = 1e-5
+    r1, xn, ss = F.matmul_nf4_epilogue(y.to(DEV), qo, None, ao, code, 64, torch.bfloat16, (d, d), resid_norm=(r0.to(DEV), w2.to(DEV)))
+    h = F.matmul_nf4_epilogue(xn, qg, None, ag, code, 64, torch.bfloat16, (2 * dff, d), rowscale=(ss, eps), silu_pairs=True)
+    r2, xn2, ss2 = F.matmul_nf4_epilogue(h, qd, None, ad, code, 64, torch.bfloat16, (d, dff), resid_norm=(r1, w1.to(DEV)))
+    torch.cuda.synchronize()
+
+    Wo, Wg, Wd = _deq(oracle, qo, ao, code, (d, d)), _deq(oracle, qg, ag, code, (2 * dff, d)), _deq(oracle, qd, ad, code, (d, dff))
+    bf = lambda t: t.to(torch.bfloat16).double()
+    r1_ref = bf(r0.double() + bf(y.double() @ Wo.t()))
+    hn = r1_ref * torch.rsqrt(r1_ref.pow(2).mean(-1, keepdim=True) + eps) * w2.double()
+    gu = hn @ Wg.t()
+    h_ref = bf(torch.nn.functional.silu(gu[:, 0::2]) * gu[:, 1::2])
+    r2_ref = bf(r1_ref + bf(h_ref @ Wd.t()))
+    torch.testing.assert_close(r1.cpu().double(), r1_ref, **TOL)
+    torch.testing.assert_close(h.cpu().double(), h_ref, rtol=4e-2, atol=4e-2)  # a product of two linear outputs
+    torch.testing.assert_close(r2.cpu().double(), r2_ref, rtol=4e-2, atol=4e-2)  # two linears deep
+    torch.testing.assert_close(ss2.double().sum(-1), r2.double().pow(2).sum(-1), rtol=1e-5, atol=0)
+    assert torch.equal(_bits(xn2), _bits((r2.float() * w1.to(DEV).float()).to(torch.bfloat16)))
+
+
+@pytest.mark.parametrize("M,shape", [(3, (512, 1024)), (1, (64, 20480)), (16, (256, 4096))])
+def test_cases_the_kernels_do_not_serve_return_none(ta, F, M, shape):
+    """More than two rows of x, or a K that one workgroup does not hold: the library answers NF4HIP_E_SHAPE before it
+    launches anything, and the host function hands None to its caller, which takes the two-step route."""
+    N, K = shape
+    qw, absmax, code = _quantized(ta, N, K, seed=N + K + 3)
+    x = _randn((M, K), seed=1).to(DEV)
+    resid = _randn((M, N), seed=2).to(DEV)
+    nw = torch.ones(N, dtype=torch.bfloat16, device=DEV)
+    assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw)) is None
+    assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), silu_pairs=True) is None
+    ss = torch.ones(M, 8, device=DEV)
+    assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), rowscale=(ss, 1e-5)) is None
+
+
+@pytest.mark.parametrize("batch", [1, 2, 8])
+def test_decode_step_with_linear_epilogues(ta, glue, monkeypatch, batch):
+    """The single-token step with the epilogues (five launches per layer) against the step with the glue kernels of
+    their own and against the plain-PyTorch step of the same quantized model; graph replay equals the eager loop."""
+    D = importlib.import_module("lightning-thunder_amd.decode")
+    print(f"decode with linear epilogues batch={batch}", flush=True)
+    dev = torch.device(DEV)
+    cfg = D.LlamaConfig.tiny(fused_projections=True, gate_up_interleaved=True, hip_glue=True)
+    model = D.build_llama(cfg, device=dev, seed=5)
+    jm = ta.jit(model, transforms=[ta.BitsAndBytesLinearQuant4bit()])
+    g = torch.Generator(device=dev).manual_seed(2)
+    prompt = torch.randint(0, cfg.vocab, (batch, 16), generator=g, device=dev)
+    eager, s0 = D.greedy_decode(jm, cfg, prompt, n_new=12, use_graph=False)
+    graph, s1 = D.greedy_decode(jm, cfg, prompt, n_new=12, use_graph=True)
+    assert s1["graph"] and torch.equal(eager, graph)
+
+    caches = [D.new_caches(cfg, batch, dev) for _ in range(3)]
+    pos = torch.arange(16, device=dev)
+    first = jm(prompt, pos, *caches[0]).argmax(-1, keepdim=True)
+    for kc, vc in caches[1:]:
+        jm(prompt, pos, kc, vc)
+    p1 = torch.full((1,), 16, device=dev, dtype=torch.long)
+    calls = {"silu": 0}
+    real = glue.silu_mul
+    monkeypatch.setattr(glue, "silu_mul", lambda *a, **k: (calls.__setitem__("silu", calls["silu"] + 1), real(*a, **k))[1])
+    a = jm(first, p1, *caches[0]).float()
+    # up to two rows of x the gate-up kernel applies SiLU * up itself; beyond, the step falls back to the glue kernels
+    assert calls["silu"] == (0 if batch <= 2 else cfg.n_layer)
+    cfg.linear_epilogues = False
+    b = jm(first, p1, *caches[1]).float()
+    cfg.hip_glue = False
+    c = jm(first, p1, *caches[2]).float()
+    torch.testing.assert_close(a, b, rtol=3e-2, atol=3e-2)
+    torch.testing.assert_close(a, c, rtol=3e-2, atol=3e-2)
+    for kc, vc in caches[1:]:
+        torch.testing.assert_close(caches[0][0][:, :, :, :17].float(), kc[:, :, :, :17].float(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(caches[0][1][:, :, :, :17].float(), vc[:, :, :, :17].float(), rtol=2e-2, atol=2e-2)

@@ -87,7 +87,8 @@ def test_nf4_executor_is_a_singleton_with_the_reference_signature(ta):
     assert ex.name == "quant_hip_nf4" and ta.extend.get_executor("quant_hip_nf4") is ex
     op = ex.opmap["hip_matmul_nf4"]
     assert op.executor is ex and set(ex.opmap) == {"hip_matmul_nf4", "hip_quantize_nf4", "hip_dequantize_nf4",
-                                                   "hip_matmul_nf4_dq", "hip_quantize_nf4_dq", "hip_dequantize_nf4_dq"}
+                                                   "hip_matmul_nf4_dq", "hip_quantize_nf4_dq", "hip_dequantize_nf4_dq",
+                                                   "hip_matmul_nf4_epilogue"}
     x = ta.TensorProxy("x", shape=(2, 3, 64), dtype=torch.bfloat16, device="cpu")
     out = op(x, None, None, None, None, 64, torch.bfloat16, (128, 64))
     assert out.shape == (2, 3, 128) and out.dtype == torch.bfloat16 and out.device == x.device

@@ -451,7 +451,7 @@ def llama_decode(torch, ta, n_new: int) -> dict:
     out = {
         "model": "Llama-3-8B architecture (32 layers, d 4096, 32q/8kv heads, FFN 14336, vocab 128256), random init, "
                  "all 161 linears NF4 (QKV and gate/up fused, gate and up rows interleaved), prompt 512, greedy, HIP-graph decode step; "
-                 "decode_tok_per_s: residual add + RMSNorm + SiLU*up in the epilogues of the NF4 decode kernels (up to two rows of x), "
+                 "decode_tok_per_s: residual add + RMSNorm + SiLU*up in the epilogues of the NF4 decode kernels (up to sixteen rows of x), "
                  "rotary + cache + attention and sampling as HIP glue kernels; _separate_glue: all of that work as HIP glue kernels "
                  "between the linears; _torch_glue: as PyTorch ops",
         "new_tokens": n_new,
@@ -464,11 +464,11 @@ def llama_decode(torch, ta, n_new: int) -> dict:
         D.greedy_decode(jm, cfg, prompt, n_new=1, use_graph=False)  # untimed: library start-up, GEMM heuristics
         res = {}
         # the single-token step with residual add / RMSNorm / SiLU * up done by the epilogues of the NF4 decode kernels
-        # where those take them (up to two rows of x; rotary + cache + attention and sampling as HIP glue kernels), with
+        # where those take them (up to sixteen rows of x; rotary + cache + attention and sampling as HIP glue kernels), with
         # all of that work as HIP glue kernels of its own, and with plain PyTorch ops in its place
         for key, glue, epi in (("", True, True), ("_separate_glue", True, False), ("_torch_glue", False, False)):
-            if (B > 8 and not glue) or (B > 2 and glue and not epi):
-                continue  # beyond two rows of x the first variant already is the second
+            if (B > 8 and not glue) or (B > 16 and glue and not epi):
+                continue  # beyond sixteen rows of x the linears run as GEMMs, without epilogues: the first variant is the second
             cfg.hip_glue, cfg.linear_epilogues = glue, epi
             _, st = D.greedy_decode(jm, cfg, prompt, n_new=n_new, use_graph=True)
             res[f"decode_tok_per_s{key}"] = round(st["decode_tok_per_s"], 1)

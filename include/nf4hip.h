@@ -153,6 +153,9 @@ typedef struct nf4hip_epilogue {
 } nf4hip_epilogue;
 /* partial sums per row of x that a RESID_NORM call on the current device writes (0: the shape is not served) */
 int nf4hip_gemv_norm_parts(int64_t M, int64_t N, int64_t K);
+/* 1 if nf4hip_gemv_epilogue takes this shape with these flags (in_parts: what a ROWSCALE call would pass, else 0),
+ * 0 if it would answer NF4HIP_E_SHAPE: for callers that must know before they launch the first kernel of a chain. */
+int nf4hip_gemv_epilogue_served(int64_t M, int64_t N, int64_t K, int blocksize, int flags, int in_parts);
 int nf4hip_gemv_epilogue(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
                          const float* lut16, const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out,
                          void* workspace, size_t workspace_bytes, const nf4hip_epilogue* epilogue, void* stream);

@@ -59,6 +59,7 @@ SYMBOLS = {
     "nf4hip_gemv_dq": (_i32, _MATMUL_DQ),
     "nf4hip_gemv_epilogue": (_i32, _MATMUL[:-1] + [ctypes.POINTER(Epilogue), _vp]),
     "nf4hip_gemv_norm_parts": (_i32, [_i64, _i64, _i64]),
+    "nf4hip_gemv_epilogue_served": (_i32, [_i64, _i64, _i64, _i32, _i32, _i32]),
     "nf4hip_gemv_static": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp]),
     "nf4hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "nf4hip_gemm": (_i32, _MATMUL),

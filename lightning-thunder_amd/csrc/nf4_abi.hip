@@ -303,6 +303,23 @@ int nf4hip_gemv_epilogue(const void* x, int x_dtype, int64_t M, const uint8_t* p
                          workspace, workspace_bytes, stream, false, epilogue);
 }
 
+int nf4hip_gemv_epilogue_served(int64_t M, int64_t N, int64_t K, int blocksize, int flags, int in_parts) {
+    const int bl = block_log2(blocksize);
+    if (bl < 0 || M <= 0 || M > 16 || N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX) return 0;
+    if ((M <= 4 ? K % 32 : K % 512) || (M > 4 && (K > (1 << 24) || K % blocksize))) return 0;
+    if (flags <= 0 || (flags & ~(NF4HIP_EPI_ROWSCALE | NF4HIP_EPI_SILU_PAIRS | NF4HIP_EPI_RESID_NORM)) ||
+        ((flags & NF4HIP_EPI_RESID_NORM) && flags != NF4HIP_EPI_RESID_NORM))
+        return 0;
+    nf4::MatmulArgs a{};
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.block_log2 = bl;
+    a.epi.flags = flags;
+    a.epi.in_parts = in_parts;
+    return nf4::gemv_epilogue_possible(a) ? 1 : 0;
+}
+
 int nf4hip_gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || M > 16) return 0;
     return nf4::gemv_norm_parts(M, N, K);

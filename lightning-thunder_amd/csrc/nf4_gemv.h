@@ -157,10 +157,14 @@ hipError_t gemv_quad_setup();
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream);
 bool gemv_quad_halves_possible(int64_t N, int64_t K);
 hipError_t launch_gemv_quad_halves(const MatmulArgs& a, int cus, hipStream_t stream);
+bool gemv_quad_epilogue_possible(const MatmulArgs& a);
+int gemv_quad_norm_parts(int64_t M, int64_t N, int64_t K, int cus, bool halves);
 
 // MFMA tile kernel, 5 <= M <= 16 (nf4_gemv_tiles.hip)
 size_t gemv_tiles_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t gemv_tiles_setup();
 hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream);
+bool gemv_tiles_epilogue_possible(const MatmulArgs& a);
+int gemv_tiles_norm_parts(int64_t N);
 
 }  // namespace nf4

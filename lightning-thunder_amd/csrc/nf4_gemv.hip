@@ -57,7 +57,8 @@ size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 bool gemv_epilogue_possible(const MatmulArgs& a) {
     if (a.epi.flags == EPI_NONE) return true;
     if (a.M <= 2) return gemv_rows_epilogue_possible(a);
-    return false;
+    if (quad_halves_serve(a.M, a.N, a.K) || quad_serves(a.M, a.N, a.K)) return gemv_quad_epilogue_possible(a);
+    return gemv_tiles_epilogue_possible(a);
 }
 
 // The number of partial sums is the number of bands of the launch plan, which depends on the device's CU count: the
@@ -66,7 +67,9 @@ int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     int cus = 256;
     if (device_setup(&cus) != hipSuccess) cus = 256;
     if (M <= 2) return gemv_rows_norm_parts(M, N, K, cus);
-    return 0;
+    if (quad_halves_serve(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, true);
+    if (quad_serves(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, false);
+    return gemv_tiles_norm_parts(N);
 }
 
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {

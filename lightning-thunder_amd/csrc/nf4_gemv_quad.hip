@@ -32,6 +32,7 @@
 //    by the last workgroup to arrive.
 #include <type_traits>
 
+#include "decode_math.h"
 #include "nf4_gemv.h"
 
 namespace nf4 {
@@ -49,6 +50,9 @@ constexpr int LOAD_K = 512;            // k covered by one wave-wide 16-byte loa
 constexpr int FLAG_OFFSET = GEMV_TABLE_BYTES + PART_BYTES - 16;
 constexpr int MAP_BYTES = 1024;         // nested absmax only: the 256-entry map, taken from the end of the partial sums
 constexpr int MAP_OFFSET = FLAG_OFFSET - MAP_BYTES;
+// kernels with an epilogue (fp32 absmax only): sums of squares per (row of x, wave), below the flag
+constexpr int SUMSQ_BYTES = 8 * GEMV_WAVES * 4;
+constexpr int SUMSQ_OFFSET = FLAG_OFFSET - 16 - SUMSQ_BYTES;
 
 struct QuadPlan {
     int waves_k;          // waves of a workgroup along K
@@ -92,8 +96,13 @@ __device__ __forceinline__ float reduce_rows(const float t[4], int lane) {
     return y;
 }
 
-template <int CPW, int U, int XS, bool NESTED, int MODE>
+// EPI (Epilogue flags; fp32 absmax): what the thread that finishes an output does with it; with K split over
+// workgroups that thread belongs to the last workgroup to arrive.  For the sums of squares of EPI_RESID_NORM a thread
+// keeps to one row of x (m = tid % MP, MP the power of two that holds M), lanes of equal m are added by a butterfly
+// and the waves in order.
+template <int CPW, int U, int XS, bool NESTED, int MODE, int EPI = EPI_NONE>
 __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a, QuadPlan p) {
+    static_assert(EPI == EPI_NONE || !NESTED, "epilogues come with fp32 absmax only");
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -117,10 +126,20 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
     if (gridDim.y > 1) {
         const int mb = 8 * (int)blockIdx.y;
         a.x += (int64_t)mb * a.K;
-        a.out += (int64_t)mb * a.N;
+        a.out += (int64_t)mb * ((EPI & EPI_SILU_PAIRS) ? a.N / 2 : a.N);
         a.M = min(a.M - mb, 8);
+        if (EPI & EPI_ROWSCALE) a.epi.in_sumsq += (int64_t)mb * a.epi.in_parts;
+        if (EPI & EPI_RESID_NORM) {
+            a.epi.resid_in += (int64_t)mb * a.N;
+            a.epi.resid_out += (int64_t)mb * a.N;
+            a.epi.xnext_out += (int64_t)mb * a.N;
+            a.epi.out_sumsq += (int64_t)mb * p.nbands;
+        }
     }
-    const int cw = wave % p.waves_k;
+    float* sumsq_s = reinterpret_cast<float*>(smem + SUMSQ_OFFSET);
+    // which K chunk a wave takes rotates with the workgroup: every workgroup reads all of x, and workgroups that start
+    // together would otherwise ask the same L2 channel for the same piece at the same time ([4096, 4096], 8 rows: 8.2 -> 7.8 us)
+    const int cw = (wave + (int)blockIdx.x) % p.waves_k;
     const int rg = wave / p.waves_k;
     const int64_t K = a.K;
     const int M = a.M;
@@ -207,6 +226,15 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
         for (int u = 0; u < U; ++u)
             if (u < cnt) issue(u, u);
 
+        // EPI_ROWSCALE: the producer's partial sums of squares, requested behind the first weights (they are wanted
+        // last: in front of x they would hold x back); wave w adds up row w of x -- in_parts <= 512 values, eight per
+        // lane -- once the task's rows are done
+        float ssp[8];
+        if constexpr (FIRST && (EPI & EPI_ROWSCALE) != 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                ssp[j] = (wave < M && lane + 64 * j < a.epi.in_parts) ? a.epi.in_sumsq[wave * a.epi.in_parts + lane + 64 * j] : 0.0f;
+        }
         // first task: the table is built while the loads are in flight
         if constexpr (FIRST) {
             if (EXACT)
@@ -337,6 +365,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
                 }
             }
         }
+        if constexpr (FIRST && (EPI & EPI_ROWSCALE) != 0) {
+            float ss = ((ssp[0] + ssp[1]) + (ssp[2] + ssp[3])) + ((ssp[4] + ssp[5]) + (ssp[6] + ssp[7]));
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lane == 0) sumsq_s[wave] = ss;  // rows of x beyond M: 0
+        }
         __syncthreads();
 
         // ---- band epilogue: add the waves of every row in a fixed order ----
@@ -345,15 +379,57 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
         // the last split may own fewer waves along K than the others
         const int wave_k = CPW * LOAD_K;
         const int nwk = min(p.waves_k, (int)((K + wave_k - 1) / wave_k) - ks * p.waves_k);
+        // What happens to the finished sums; `sum_of(r, m)`: the sum of output (row r of the band, row m of x) over K.
+        auto finish = [&](auto sum_of) {
+            auto finished = [&](int r, int m) {
+                float sum = sum_of(r, m);
+                // 1 / rms of row m of x, from the sum of squares the first task left in LDS
+                if (EPI & EPI_ROWSCALE) sum *= rsqrtf(sumsq_s[m] / (float)K + a.epi.eps);
+                if (a.bias) sum += bf16_bits_to_f32(a.bias[r_begin + r]);
+                return sum;
+            };
+            if (EPI & EPI_SILU_PAIRS) {
+                // rows 2j, 2j + 1 of the band: gate j, up j (a band is a whole number of four-row groups)
+                for (int idx = tid; idx < (nrows / 2) * M; idx += GEMV_THREADS) {
+                    const int j = idx / M, m = idx - j * M;
+                    const float g = nf4x::round_bf16(finished(2 * j, m)), u = nf4x::round_bf16(finished(2 * j + 1, m));
+                    a.out[(int64_t)m * (a.N / 2) + r_begin / 2 + j] = (uint16_t)nf4x::silu_mul_bf16(g, u);
+                }
+            } else if (EPI & EPI_RESID_NORM) {
+                const int MP = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : 8;  // thread = (m = tid % MP, rows tid / MP + i * 512 / MP)
+                const int m = tid % MP;
+                float ss = 0.0f;
+                if (m < M)
+                    for (int r = tid / MP; r < nrows; r += GEMV_THREADS / MP) {
+                        const int64_t at = (int64_t)m * a.N + r_begin + r;
+                        const float d = nf4x::round_bf16(finished(r, m));
+                        const float res = nf4x::resid_add(bf16_bits_to_f32(a.epi.resid_in[at]), d);
+                        a.epi.resid_out[at] = (uint16_t)f32_to_bf16_bits(res);
+                        a.epi.xnext_out[at] = (uint16_t)f32_to_bf16_bits(res * bf16_bits_to_f32(a.epi.norm_weight[r_begin + r]));
+                        ss = fmaf(res, res, ss);
+                    }
+                for (int o = 32; o >= MP; o >>= 1) ss += __shfl_xor(ss, o, 64);  // lanes of equal m
+                if (lane < MP) sumsq_s[lane * GEMV_WAVES + wave] = ss;
+                __syncthreads();
+                if (tid < M) {
+                    float tot = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < GEMV_WAVES; ++w) tot += sumsq_s[tid * GEMV_WAVES + w];
+                    a.epi.out_sumsq[tid * p.nbands + band] = tot;
+                }
+            } else {
+                for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
+                    const int r = idx / M, m = idx - r * M;
+                    a.out[(int64_t)m * a.N + r_begin + r] = (uint16_t)f32_to_bf16_bits(finished(r, m));
+                }
+            }
+        };
         if (p.splits == 1) {
-            for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
-                const int r = idx / M, m = idx - r * M;
+            finish([&](int r, int m) {
                 float sum = 0.0f;
                 for (int c = 0; c < nwk; ++c) sum += part[(r * p.waves_k + c) * M + m];
-                const int n = r_begin + r;
-                if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
-                a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
-            }
+                return sum;
+            });
         } else {
             for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
                 const int r = idx / M, m = idx - r * M;
@@ -372,16 +448,13 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
             __syncthreads();
             acquire_partials();
             if (*flag != 0) {
-                for (int idx = tid; idx < nrows * M; idx += GEMV_THREADS) {
-                    const int r = idx / M, m = idx - r * M;
-                    const int n = r_begin + r;
+                finish([&](int r, int m) {
                     float sum = 0.0f;
                     for (int k2 = 0; k2 < p.splits; ++k2)
-                        sum += __hip_atomic_load(&partial[((int64_t)k2 * M + m) * a.N + n], __ATOMIC_RELAXED,
+                        sum += __hip_atomic_load(&partial[((int64_t)k2 * M + m) * a.N + r_begin + r], __ATOMIC_RELAXED,
                                                  __HIP_MEMORY_SCOPE_AGENT);
-                    if (a.bias) sum += bf16_bits_to_f32(a.bias[n]);
-                    a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(sum);
-                }
+                    return sum;
+                });
                 if (tid == 0) __hip_atomic_store(&counters[band], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
@@ -405,7 +478,7 @@ int quad_splits(int64_t M, int64_t K) {
     return (int)((nwk + GEMV_WAVES - 1) / GEMV_WAVES);
 }
 
-QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested) {
+QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, bool nested, bool epi = false) {
     QuadPlan p;
     p.aligned = (K & (((int64_t)1 << block_log2) - 1)) == 0;
     const int64_t wave_k = (int64_t)pick_cpw(M, K) * LOAD_K;
@@ -414,7 +487,7 @@ QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
     p.waves_k = (nwk + p.splits - 1) / p.splits;
     p.row_groups = GEMV_WAVES / p.waves_k;
     const int groups = (int)((N + 3) / 4);
-    const int part_bytes = PART_BYTES - 64 - (nested ? MAP_BYTES : 0);
+    const int part_bytes = PART_BYTES - 64 - (nested ? MAP_BYTES : 0) - (epi ? SUMSQ_BYTES + 16 : 0);
     const int cap = (part_bytes / (4 * p.waves_k * M * 4)) / p.row_groups * p.row_groups;
     int bands_target = slots / p.splits;
     if (bands_target < 1) bands_target = 1;
@@ -435,46 +508,78 @@ QuadPlan make_quad_plan(int M, int64_t N, int64_t K, int block_log2, int slots, 
     return p;
 }
 
-template <int CPW, int U, int XS, bool NESTED>
+template <int CPW, int U, int XS, bool NESTED, int EPI>
 hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
     const int mode = gemv_arith_mode(a.K, true);
     const dim3 g((unsigned)grid, (unsigned)halves);
     if (mode == ARITH_EXACT)
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else if (mode == ARITH_F16)
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     else
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
 
 // U = row groups in flight per wave: U * CPW 16-byte loads per lane, at most 8 (4 with eight rows of x)
-template <int CPW, int XS, bool NESTED>
+template <int CPW, int XS, bool NESTED, int EPI>
 hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
     const int cnt = p.groups_per_band / p.row_groups;  // groups per wave and task
     constexpr int UMAX = 8 / (CPW * XS);
-    if constexpr (UMAX >= 8)
-        if (cnt >= 8) return launch_u<CPW, 8, XS, NESTED>(a, p, grid, stream, halves);
-    if constexpr (UMAX >= 4 && !(NESTED && CPW == 2))  // nested: one more register per load in flight
-        if (cnt >= 4) return launch_u<CPW, 4, XS, NESTED>(a, p, grid, stream, halves);
-    return launch_u<CPW, 2, XS, NESTED>(a, p, grid, stream, halves);
+    if constexpr (UMAX >= 8 && EPI == EPI_NONE)  // with an epilogue eight groups in flight would spill
+        if (cnt >= 8) return launch_u<CPW, 8, XS, NESTED, EPI>(a, p, grid, stream, halves);
+    // nested absmax: one more register per load in flight; the residual epilogue: its pointers -- either would spill
+    if constexpr (UMAX >= 4 && !((NESTED || EPI == EPI_RESID_NORM) && CPW == 2))
+        if (cnt >= 4) return launch_u<CPW, 4, XS, NESTED, EPI>(a, p, grid, stream, halves);
+    return launch_u<CPW, 2, XS, NESTED, EPI>(a, p, grid, stream, halves);
+}
+
+template <bool NESTED, int EPI>
+hipError_t launch_e(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
+    if (a.M > 4 || halves > 1) return launch_c<1, 2, NESTED, EPI>(a, p, grid, stream, halves);
+    return pick_cpw(a.M, a.K) == 1 ? launch_c<1, 1, NESTED, EPI>(a, p, grid, stream) : launch_c<2, 1, NESTED, EPI>(a, p, grid, stream);
 }
 
 template <bool NESTED>
-hipError_t launch_n(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream) {
-    if (a.M > 4) return launch_c<1, 2, NESTED>(a, p, grid, stream);
-    return pick_cpw(a.M, a.K) == 1 ? launch_c<1, 1, NESTED>(a, p, grid, stream) : launch_c<2, 1, NESTED>(a, p, grid, stream);
+hipError_t launch_n(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
+    if constexpr (!NESTED) {
+        switch (a.epi.flags) {
+            case EPI_ROWSCALE: return launch_e<false, EPI_ROWSCALE>(a, p, grid, stream, halves);
+            case EPI_ROWSCALE | EPI_SILU_PAIRS: return launch_e<false, EPI_ROWSCALE | EPI_SILU_PAIRS>(a, p, grid, stream, halves);
+            case EPI_SILU_PAIRS: return launch_e<false, EPI_SILU_PAIRS>(a, p, grid, stream, halves);
+            case EPI_RESID_NORM: return launch_e<false, EPI_RESID_NORM>(a, p, grid, stream, halves);
+        }
+    }
+    if (a.epi.flags != EPI_NONE) return hipErrorNotSupported;
+    return launch_e<NESTED, EPI_NONE>(a, p, grid, stream, halves);
+}
+
+template <int CPW, int U, int XS, int MODE>
+hipError_t allow_lds_epi() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_NONE>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, MODE, EPI_NONE>, SMEM_BYTES)) != hipSuccess) return e;
+    if constexpr (U <= 4) {
+        if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_ROWSCALE>, SMEM_BYTES)) != hipSuccess) return e;
+        if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_ROWSCALE | EPI_SILU_PAIRS>, SMEM_BYTES)) != hipSuccess) return e;
+        if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_SILU_PAIRS>, SMEM_BYTES)) != hipSuccess) return e;
+        if constexpr (!(CPW == 2 && U == 4))
+            if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_RESID_NORM>, SMEM_BYTES)) != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 template <int CPW, int U, int XS>
 hipError_t allow_lds_cu() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, ARITH_BF16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, ARITH_F16>, SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, ARITH_EXACT>, SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, ARITH_EXACT>, SMEM_BYTES);
+    if ((e = allow_lds_epi<CPW, U, XS, ARITH_BF16>()) != hipSuccess) return e;
+    if ((e = allow_lds_epi<CPW, U, XS, ARITH_F16>()) != hipSuccess) return e;
+    return allow_lds_epi<CPW, U, XS, ARITH_EXACT>();
+}
+
+int quad_slots(int cus) {
+    int slots = 2 * cus;
+    return slots > GEMV_COUNTER_BYTES / 4 ? GEMV_COUNTER_BYTES / 4 : slots;
 }
 
 }  // namespace
@@ -501,18 +606,34 @@ bool gemv_quad_halves_possible(int64_t N, int64_t K) { return K % LOAD_K == 0 &&
 
 hipError_t launch_gemv_quad_halves(const MatmulArgs& a, int cus, hipStream_t stream) {
     if (a.M <= 8 || a.M > 16 || !gemv_quad_halves_possible(a.N, a.K)) return hipErrorInvalidValue;
+    if (!gemv_quad_epilogue_possible(a)) return hipErrorNotSupported;
     // each half has the chip to itself in the plan: the two halves of a task then run side by side
     int slots = cus;
-    const QuadPlan p = make_quad_plan(8, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
+    const QuadPlan p = make_quad_plan(8, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr, a.epi.flags != EPI_NONE);
     if (p.splits != 1) return hipErrorInvalidValue;
     int grid = p.ntasks < slots ? p.ntasks : slots;
-    return a.nested.q ? launch_c<1, 2, true>(a, p, grid, stream, 2) : launch_c<1, 2, false>(a, p, grid, stream, 2);
+    return a.nested.q ? launch_n<true>(a, p, grid, stream, 2) : launch_n<false>(a, p, grid, stream, 2);
+}
+
+// epilogues of the quad kernel: fp32 absmax; (gate, up) pairs need an even N; the producer's partial sums one per thread
+bool gemv_quad_epilogue_possible(const MatmulArgs& a) {
+    if (a.epi.flags == EPI_NONE) return true;
+    if (a.nested.q) return false;
+    if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > GEMV_THREADS) return false;
+    return !(a.epi.flags & EPI_SILU_PAIRS) || a.N % 2 == 0;
+}
+
+// bands of the plan an EPI_RESID_NORM call runs with (`halves`: nine to sixteen rows of x as two halves of eight)
+int gemv_quad_norm_parts(int64_t M, int64_t N, int64_t K, int cus, bool halves) {
+    const QuadPlan p = halves ? make_quad_plan(8, N, K, 6, cus, false, true) : make_quad_plan((int)M, N, K, 6, quad_slots(cus), false, true);
+    if (p.splits > 1 && p.nbands > GEMV_COUNTER_BYTES / 4) return 0;
+    return p.nbands;
 }
 
 hipError_t launch_gemv_quad(const MatmulArgs& a, int cus, hipStream_t stream) {
-    int slots = 2 * cus;
-    if (slots > GEMV_COUNTER_BYTES / 4) slots = GEMV_COUNTER_BYTES / 4;
-    const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr);
+    if (!gemv_quad_epilogue_possible(a)) return hipErrorNotSupported;
+    const int slots = quad_slots(cus);
+    const QuadPlan p = make_quad_plan(a.M, a.N, a.K, a.block_log2, slots, a.nested.q != nullptr, a.epi.flags != EPI_NONE);
     // one arrival counter per band when K is split across workgroups
     if (p.splits > 1 && p.nbands > GEMV_COUNTER_BYTES / 4) return hipErrorInvalidValue;
     int grid = p.ntasks < slots ? p.ntasks : slots;

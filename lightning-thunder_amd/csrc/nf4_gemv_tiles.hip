@@ -33,6 +33,7 @@
 //  * K split.  Only when N alone cannot fill the chip is K also split over workgroups; partial
 //    sums then go to a workspace and the last WAVE to finish a tile (device-scope counter per
 //    tile) adds them in a fixed order, so the result does not depend on scheduling.
+#include "decode_math.h"
 #include "nf4_gemv.h"
 
 namespace nf4 {
@@ -50,7 +51,8 @@ constexpr int XBYTES_MAX = 80 * 1024;        // resident x operands
 constexpr int ITEMS_MAX = 512;               // longest work list of a workgroup (one entry per thread)
 constexpr int ITEMS_OFFSET = TABLE_BYTES + XBYTES_MAX;
 constexpr int UNSCALE_OFFSET = ITEMS_OFFSET + ITEMS_MAX * 16;  // fp16 mode: 16 floats, what undoes the scaling of each row of x
-constexpr int SMEM_BYTES = UNSCALE_OFFSET + 64;
+constexpr int SUMSQ_OFFSET = UNSCALE_OFFSET + 64;  // EPI_ROWSCALE: the sum of squares of each row of x, 16 floats
+constexpr int SMEM_BYTES = SUMSQ_OFFSET + 64;
 constexpr int COUNTER_BYTES = GEMV_COUNTER_BYTES;
 constexpr int SLOTS = 4;                     // ring slots = accumulator sets = largest batch
 
@@ -453,8 +455,14 @@ __device__ __forceinline__ void scale_x_slice_to_f16(uint4 (&v)[XUNITS], int n, 
 // everything in flight at the top of every group (loads under branches, and the stores of a batch
 // end, which complete out of order with loads).  The price is a drain when that loop is entered and
 // switched-off requests at the end of the list, which short lists cannot afford.
-template <bool B64, bool NESTED, int R, int MODE, bool STEADY>
+// EPI (Epilogue flags; fp32 absmax, blocksize 64): what the lane that finishes an output does with it -- at the end of
+// a batch, or in the wave that reduces a tile when K is split over workgroups.  A tile is 16 weight rows: the two
+// rows of a (gate, up) pair sit in neighbouring lanes, and EPI_RESID_NORM leaves one partial sum of squares per tile
+// (added over the tile's 16 lanes by a butterfly), so what a partial sum holds does not depend on which workgroup
+// finished the tile.
+template <bool B64, bool NESTED, int R, int MODE, bool STEADY, int EPI = EPI_NONE>
 __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Plan p) {
+    static_assert(EPI == EPI_NONE || (B64 && !NESTED), "epilogues: fp32 absmax, blocksize 64");
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int CAP = XBYTES_MAX / (R * 1024);  // phases of x that fit
@@ -507,7 +515,20 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
     ls.G = ls.tg0 < p.tile_groups ? (p.tile_groups - 1 - ls.tg0) / p.tg_step + 1 : 0;
     ls.nitems = list_length<CAP>(ls.G, ls.nsl, ls.last);
     const int cn = ls.nitems;  // <= ITEMS_MAX, guaranteed by the launcher
+    float* sumsq_s = reinterpret_cast<float*>(smem + SUMSQ_OFFSET);
     {
+        // EPI_ROWSCALE: this thread's share of the producer's partial sums of squares, the first requests of all
+        // (wave w adds up rows w and w + 8 of x: in_parts <= 512 values each, eight per lane)
+        float ssp[R / 8][8];
+        if (EPI & EPI_ROWSCALE) {
+#pragma unroll
+            for (int h = 0; h < R / 8; ++h)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int m = wave + 8 * h;
+                    ssp[h][j] = (m < a.M && lane + 64 * j < a.epi.in_parts) ? a.epi.in_sumsq[m * a.epi.in_parts + lane + 64 * j] : 0.0f;
+                }
+        }
         uint4 xv[XUNITS];
         const int nph0 = ls.nsl == 1 ? ls.last : CAP;
         load_x_slice<R>(a, xv, ls.r0 * PHASE_K, nph0, lane, wave);
@@ -534,8 +555,53 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
             build_pair_table<F16>(smem, lut_lane, lane, wave);
         if (F16) scale_x_slice_to_f16<R>(xv, nph0, smem + UNSCALE_OFFSET, lane, wave);
         store_x_slice<R>(a, xv, smem + TABLE_BYTES, nph0, lane, wave);
+        if (EPI & EPI_ROWSCALE) {
+#pragma unroll
+            for (int h = 0; h < R / 8; ++h) {
+                const float* v = ssp[h];
+                float ss = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                if (lane == 0) sumsq_s[wave + 8 * h] = ss;  // rows of x beyond M: 0
+            }
+        }
         __syncthreads();
     }
+    // 1 / rms of row m of x (EPI_ROWSCALE)
+    auto rstd_of = [&](int m) { return rsqrtf(sumsq_s[m] / (float)a.K + a.epi.eps); };
+    const int ntiles = (a.N + 15) / 16;  // EPI_RESID_NORM: partial sums per row of x
+    // The lane's finished sums of one tile: v[j] belongs to row m_of(j) of x and weight row n (valid: the lane owns a
+    // row of the matrix here).  Every lane of the wave takes part (the pair exchange and the butterfly need them all).
+    auto emit = [&](const float* v, int cnt, auto m_of, int n, bool valid, int tile) {
+        const float b = (a.bias && valid) ? bf16_bits_to_f32(a.bias[n]) : 0.0f;
+        for (int j = 0; j < cnt; ++j) {
+            const int m = m_of(j);
+            const bool on = valid && m < a.M;
+            float val = v[j];
+            if (EPI & EPI_ROWSCALE) val *= rstd_of(min(m, R - 1));
+            val += b;
+            if (EPI & EPI_SILU_PAIRS) {
+                // the lane of the odd row hands its value to the lane of the even row (N is even, tiles start on even rows)
+                const float mine = nf4x::round_bf16(val);
+                const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine), 0xB1, 0xf, 0xf, true));
+                if (on && !(n & 1)) a.out[(int64_t)m * (a.N / 2) + n / 2] = (uint16_t)nf4x::silu_mul_bf16(mine, other);
+            } else if (EPI & EPI_RESID_NORM) {
+                float sq = 0.0f;
+                if (on) {
+                    const int64_t at = (int64_t)m * a.N + n;
+                    const float res = nf4x::resid_add(bf16_bits_to_f32(a.epi.resid_in[at]), nf4x::round_bf16(val));
+                    a.epi.resid_out[at] = (uint16_t)f32_to_bf16_bits(res);
+                    a.epi.xnext_out[at] = (uint16_t)f32_to_bf16_bits(res * bf16_bits_to_f32(a.epi.norm_weight[n]));
+                    sq = res * res;
+                }
+#pragma unroll
+                for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);  // the 16 rows of the tile
+                if (col == 0 && m < a.M && tile < ntiles) a.epi.out_sumsq[m * ntiles + tile] = sq;
+            } else if (on) {
+                a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(val);
+            }
+        }
+    };
 
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + COUNTER_BYTES);
@@ -635,14 +701,8 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
                 const int n = max(min(n0, a.N - 16), 0) + col;  // the lane's row
                 const bool mine = n >= n0 && n < a.N;
                 if (p.splits == 1) {
-                    if (mine) {
-                        const float b = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.0f;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int m = 4 * g + i;
-                            if (m < a.M) a.out[(int64_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(acc[t][i] + b);
-                        }
-                    }
+                    const float v4[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+                    emit(v4, 4, [&](int i) { return 4 * g + i; }, n, mine, tile);
                 } else if (n0 < a.N) {
                     // Partial sums cross workgroups (and XCDs, whose L2s are not coherent with each
                     // other) through agent-scope relaxed atomics only: such stores write through
@@ -693,14 +753,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Pl
 #pragma unroll
                                 for (int o = 0; o < OUTS; ++o) sum[o] += k2 + j < p.splits ? v[o][j] : 0.0f;
                         }
-                        if (nn < a.N) {
-                            const float b = a.bias ? bf16_bits_to_f32(a.bias[nn]) : 0.0f;
-#pragma unroll
-                            for (int o = 0; o < OUTS; ++o) {
-                                const int m = g + 4 * o;
-                                if (m < a.M) a.out[(int64_t)m * a.N + nn] = (uint16_t)f32_to_bf16_bits(sum[o] + b);
-                            }
-                        }
+                        emit(sum, OUTS, [&](int o) { return g + 4 * o; }, min(nn, a.N - 1), nn < a.N, tile);
                         if (lane == 0)
                             __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
@@ -783,12 +836,29 @@ hipError_t allow_both() {
     return e != hipSuccess ? e : allow_rx<B64, NESTED, true>();
 }
 
+template <int EPI, bool STEADY>
+hipError_t allow_epi() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<true, false, 8, ARITH_BF16, STEADY, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<true, false, 16, ARITH_BF16, STEADY, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<true, false, 8, ARITH_F16, STEADY, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<true, false, 16, ARITH_F16, STEADY, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_tiles_kernel<true, false, 8, ARITH_EXACT, STEADY, EPI>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_tiles_kernel<true, false, 16, ARITH_EXACT, STEADY, EPI>, SMEM_BYTES);
+}
+
 hipError_t gemv_tiles_setup() {
     hipError_t e;
     if ((e = allow_both<false, false>()) != hipSuccess) return e;
     if ((e = allow_both<true, false>()) != hipSuccess) return e;
     if ((e = allow_both<false, true>()) != hipSuccess) return e;
-    return allow_both<true, true>();
+    if ((e = allow_both<true, true>()) != hipSuccess) return e;
+    if ((e = allow_epi<EPI_ROWSCALE, false>()) != hipSuccess || (e = allow_epi<EPI_ROWSCALE, true>()) != hipSuccess) return e;
+    if ((e = allow_epi<EPI_ROWSCALE | EPI_SILU_PAIRS, false>()) != hipSuccess) return e;
+    if ((e = allow_epi<EPI_ROWSCALE | EPI_SILU_PAIRS, true>()) != hipSuccess) return e;
+    if ((e = allow_epi<EPI_SILU_PAIRS, false>()) != hipSuccess || (e = allow_epi<EPI_SILU_PAIRS, true>()) != hipSuccess) return e;
+    if ((e = allow_epi<EPI_RESID_NORM, false>()) != hipSuccess) return e;
+    return allow_epi<EPI_RESID_NORM, true>();
 }
 
 template <int R, int MODE, bool STEADY>
@@ -798,6 +868,14 @@ hipError_t launch_rs(const MatmulArgs& a, const Plan& p, int grid, hipStream_t s
     auto kern = b64 ? (nested ? gemv_tiles_kernel<true, true, R, MODE, STEADY> : gemv_tiles_kernel<true, false, R, MODE, STEADY>)
                     : (nested ? gemv_tiles_kernel<false, true, R, MODE, STEADY>
                               : gemv_tiles_kernel<false, false, R, MODE, STEADY>);
+    switch (a.epi.flags) {  // epilogues: fp32 absmax and blocksize 64 (gemv_tiles_epilogue_possible)
+        case EPI_NONE: break;
+        case EPI_ROWSCALE: kern = gemv_tiles_kernel<true, false, R, MODE, STEADY, EPI_ROWSCALE>; break;
+        case EPI_ROWSCALE | EPI_SILU_PAIRS: kern = gemv_tiles_kernel<true, false, R, MODE, STEADY, EPI_ROWSCALE | EPI_SILU_PAIRS>; break;
+        case EPI_SILU_PAIRS: kern = gemv_tiles_kernel<true, false, R, MODE, STEADY, EPI_SILU_PAIRS>; break;
+        case EPI_RESID_NORM: kern = gemv_tiles_kernel<true, false, R, MODE, STEADY, EPI_RESID_NORM>; break;
+        default: return hipErrorNotSupported;
+    }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
     return hipGetLastError();
 }
@@ -812,7 +890,23 @@ hipError_t launch_m(const MatmulArgs& a, const Plan& p, int grid, bool steady, h
     return rows_held(a.M) == 8 ? launch_r<8, MODE>(a, p, grid, steady, stream) : launch_r<16, MODE>(a, p, grid, steady, stream);
 }
 
+// epilogues of the tile kernel: fp32 absmax, blocksize 64; (gate, up) pairs need an even N; the producer's partial
+// sums one per thread; a partial sum of squares per tile of 16 weight rows, at most one per thread of the consumer
+bool gemv_tiles_epilogue_possible(const MatmulArgs& a) {
+    if (a.epi.flags == EPI_NONE) return true;
+    if (a.nested.q || a.block_log2 != 6) return false;
+    if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > THREADS) return false;
+    if ((a.epi.flags & EPI_RESID_NORM) && gemv_tiles_norm_parts(a.N) == 0) return false;
+    return !(a.epi.flags & EPI_SILU_PAIRS) || a.N % 2 == 0;
+}
+
+int gemv_tiles_norm_parts(int64_t N) {
+    const int64_t tiles = (N + 15) / 16;
+    return tiles <= THREADS ? (int)tiles : 0;
+}
+
 hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream) {
+    if (!gemv_tiles_epilogue_possible(a)) return hipErrorNotSupported;
     Plan p = make_plan(a.M, a.N, a.K);
     const int grid = grid_for((int64_t)p.tile_groups * p.splits, p.splits, cus < 1024 ? cus : 1024);
     p.tg_step = grid / p.splits;

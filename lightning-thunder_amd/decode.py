@@ -171,7 +171,7 @@ class Llama(nn.Module):
         cfg = self.cfg
         H, Hkv, eps = cfg.n_head, cfg.n_kv_head, cfg.norm_eps
         x = self.wte(idx)[:, 0, :].contiguous()
-        if cfg.linear_epilogues and cfg.fused_projections and cfg.gate_up_interleaved and x.shape[0] <= 2:
+        if cfg.linear_epilogues and cfg.fused_projections and cfg.gate_up_interleaved and x.shape[0] <= 16:
             out = self._decode_step_epilogues(x, pos, kcache, vcache)
             if out is not None:
                 return out
@@ -204,9 +204,9 @@ class Llama(nn.Module):
         cfg = self.cfg
         H, Hkv, eps = cfg.n_head, cfg.n_kv_head, cfg.norm_eps
         lins = [l for blk in self.blocks for l in (blk.attn.qkv_proj, blk.attn.o_proj, blk.mlp.gate_up_proj, blk.mlp.down_proj)]
-        args = {id(l): _planned_nf4(l) for l in lins + [self.lm_head]}
-        if any(a is None for a in args.values()) or not _epilogues_served(x.shape[0], lins + [self.lm_head]):
+        if not _chain_served(x.shape[0], self):
             return None
+        args = {id(l): _planned_nf4(l) for l in lins + [self.lm_head]}
         ep = Q.hip_matmul_nf4_epilogue
         r = x
         xn = ss = None
@@ -247,13 +247,30 @@ def _planned_nf4(lin: nn.Linear):
     return (packed, lin.bias, *rest)
 
 
-def _epilogues_served(rows: int, linears) -> bool:
-    """Do the decode kernels take an epilogue at ``rows`` rows of x on every one of these weights?  (Asked of the
-    library through its own planning function, before the step launches anything.)"""
-    from . import _lib
+def _chain_served(rows: int, model: "Llama") -> bool:
+    """Do the decode kernels take, at ``rows`` rows of x, every epilogue that ``Llama._decode_step_epilogues`` asks of
+    the model's 4-bit linears?  (Asked before the step launches anything: a refusal half way would leave it nowhere.)"""
+    from . import _lib, functional
 
     lib = _lib.load()
-    return all(lib.nf4hip_gemv_norm_parts(rows, l.out_features, l.in_features) > 0 for l in linears)
+
+    def served(lin, producer=None, **kw):
+        args = _planned_nf4(lin)
+        if args is None:
+            return False
+        _, _, absmax, _, blocksize, dtype, shape = args
+        if producer is not None:  # row scale: as many partial sums as the producing linear leaves
+            kw["rowscale_parts"] = lib.nf4hip_gemv_norm_parts(rows, producer.out_features, producer.in_features)
+            if kw["rowscale_parts"] <= 0:
+                return False
+        return functional.epilogue_served(rows, shape, blocksize, dtype, isinstance(absmax, functional.NestedAbsmax), **kw)
+
+    for blk in model.blocks:
+        a, m = blk.attn, blk.mlp
+        if not (served(a.qkv_proj, m.down_proj) and served(a.o_proj, resid_norm=True)
+                and served(m.gate_up_proj, a.o_proj, silu_pairs=True) and served(m.down_proj, resid_norm=True)):
+            return False
+    return served(model.lm_head, model.blocks[-1].mlp.down_proj)
 
 
 def build_llama(cfg: LlamaConfig, device="cuda", dtype=torch.bfloat16, seed: int = 0) -> Llama:

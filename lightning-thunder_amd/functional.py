@@ -536,6 +536,18 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
 # ---- the decode kernels with an epilogue ---------------------------------------------------------------------
 
 
+def epilogue_served(rows: int, shape, blocksize: int = 64, dtype: torch.dtype = torch.bfloat16, nested: bool = False, *,
+                    rowscale_parts: int = 0, silu_pairs: bool = False, resid_norm: bool = False) -> bool:
+    """Will ``matmul_nf4_epilogue`` serve ``rows`` rows of bf16 x on an [N, K] weight with this epilogue
+    (``rowscale_parts``: the number of partial sums a row scale would be given, 0 for none)?  The library's own answer
+    for the current device; for callers that must know before they launch the first kernel of a chain."""
+    N, K = (int(s) for s in shape)
+    if nested or dtype != torch.bfloat16 or blocksize not in SUPPORTED_BLOCKSIZES:
+        return False
+    flags = (_lib.EPI_ROWSCALE if rowscale_parts else 0) | (_lib.EPI_SILU_PAIRS if silu_pairs else 0) | (_lib.EPI_RESID_NORM if resid_norm else 0)
+    return bool(_lib.load().nf4hip_gemv_epilogue_served(rows, N, K, blocksize, flags, rowscale_parts))
+
+
 def matmul_nf4_epilogue(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, *, rowscale=None, silu_pairs=False,
                         resid_norm=None):
     """``matmul_nf4`` at decode shapes with the step that follows (or precedes) the linear in a decoder layer done by

@@ -191,9 +191,13 @@ def test_epilogue_argument_errors(ta):
     assert call(L.Epilogue(L.EPI_ROWSCALE, 1e-5, A + 2, 8)) == L.E_ALIGN
     assert call(L.Epilogue(L.EPI_RESID_NORM, 0.0, None, 0, A, A, A, None, A)) == L.E_NULL and "xnext_out" in err()
     assert call(L.Epilogue(L.EPI_RESID_NORM, 0.0, None, 0, A, A, A + 1, A, A)) == L.E_ALIGN
-    args3 = (A, L.BF16, 3, A, A, A, None, 64, 4096, 64, A, A, 1 << 30)
-    assert call(L.Epilogue(L.EPI_SILU_PAIRS), args3) == L.E_SHAPE and "not served" in err()
+    tiles = (A, L.BF16, 16, A, A, A, None, 16384, 4096, 64, A, A, 1 << 30)  # tile kernel: 1024 tiles of 16 weight rows
+    assert call(L.Epilogue(L.EPI_RESID_NORM, 0.0, None, 0, A, A, A, A, A), tiles) == L.E_SHAPE and "not served" in err()
+    odd = (A, L.BF16, 3, A, A, A, None, 63, 4096, 64, A, A, 1 << 30)
+    assert call(L.Epilogue(L.EPI_SILU_PAIRS), odd) == L.E_SHAPE and "not served" in err()  # pairs need an even N
     long_k = (A, L.BF16, 1, A, A, A, None, 64, 20480, 64, A, A, 1 << 30)
     assert call(L.Epilogue(L.EPI_SILU_PAIRS), long_k) == L.E_SHAPE and "not served" in err()
     assert call(L.Epilogue(L.EPI_ROWSCALE, 1e-5, A, 513)) == L.E_SHAPE  # more partial sums than a workgroup has threads
-    assert lib.nf4hip_gemv_norm_parts(3, 64, 4096) == 0 and lib.nf4hip_gemv_norm_parts(1, 64, 20480) == 0
+    assert lib.nf4hip_gemv_norm_parts(16, 16384, 4096) == 0 and lib.nf4hip_gemv_norm_parts(1, 64, 20480) == 0
+    assert lib.nf4hip_gemv_norm_parts(16, 8192, 4096) == 512
+    assert lib.nf4hip_gemv_norm_parts(3, 64, 4096) > 0 and lib.nf4hip_gemv_norm_parts(8, 4096, 14336) > 0

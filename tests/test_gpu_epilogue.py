@@ -47,10 +47,19 @@ def _bits(t):
 PAIR_SHAPES = [(1024, 512), (28672, 4096), (2048, 14336), (272, 2080)]
 
 
-@pytest.mark.parametrize("M", [1, 2])
+def _served(F, M, N, K, **which):
+    """K % 32 == 0 up to four rows of x, K % 512 == 0 beyond, K within one workgroup's reach up to two; the residual
+    epilogue of the tile kernel (nine and more rows of x, or a large weight) leaves one partial sum per 16 weight rows,
+    at most 512 of them."""
+    return F.epilogue_served(M, (N, K), **which)
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 8, 16])
 @pytest.mark.parametrize("shape", PAIR_SHAPES)
 def test_silu_pairs_gives_the_two_step_bits(ta, F, glue, M, shape):
     N, K = shape
+    if not _served(F, M, N, K, silu_pairs=True):
+        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup up to two)")
     print(f"epilogue silu_pairs M={M} N={N} K={K}", flush=True)
     qw, absmax, code = _quantized(ta, N, K, seed=N + K)
     x = _randn((M, K), seed=3 * N + M).to(DEV)
@@ -63,13 +72,15 @@ def test_silu_pairs_gives_the_two_step_bits(ta, F, glue, M, shape):
 
 
 # (N, K): Llama-3-8B output and down projections, ragged, the longest K one workgroup holds
-RESID_SHAPES = [(4096, 4096), (4096, 14336), (517, 1056), (256, 16384)]
+RESID_SHAPES = [(4096, 4096), (4096, 14336), (517, 1056), (256, 16384), (8192, 8192), (1000, 28672)]
 
 
-@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16])
 @pytest.mark.parametrize("shape", RESID_SHAPES)
 def test_resid_norm_epilogue(ta, F, M, shape):
     N, K = shape
+    if not _served(F, M, N, K, resid_norm=True):
+        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup up to two)")
     print(f"epilogue resid_norm M={M} N={N} K={K}", flush=True)
     qw, absmax, code = _quantized(ta, N, K, seed=N + K + 1)
     x = _randn((M, K), seed=5 * N + M).to(DEV)
@@ -94,14 +105,16 @@ def _deq(oracle, qw, absmax, code, shape):
     return oracle.dequantize_4bit_eager(qw.cpu(), absmax.cpu(), code.cpu(), 64, torch.bfloat16, shape).double()
 
 
-@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 8, 16])
 @pytest.mark.parametrize("silu", [False, True])
 @pytest.mark.parametrize("shape", [(6144, 4096), (1024, 512), (28672, 4096), (128256, 4096), (304, 8192)])
 def test_rowscale_epilogue_against_float64(ta, F, glue, oracle, M, silu, shape):
     """A producer's (xnext, sumsq) made by hand from a residual r: the consumer must give linear(rms_norm(r) * w)."""
     N, K = shape
-    if N == 128256 and (silu or M == 2):
+    if N == 128256 and (silu or M != 1):
         pytest.skip("the lm_head is checked once")
+    if not _served(F, M, N, K, rowscale_parts=37, silu_pairs=silu):
+        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup up to two)")
     print(f"epilogue rowscale M={M} N={N} K={K} silu={silu}", flush=True)
     qw, absmax, code = _quantized(ta, N, K, seed=N + K + 2)
     r = _randn((M, K), seed=11 * N + M, std=3.0)
@@ -155,22 +168,39 @@ def test_chain_of_epilogues_is_a_decoder_layer_tail(ta, F, oracle):
     assert torch.equal(_bits(xn2), _bits((r2.float() * w1.to(DEV).float()).to(torch.bfloat16)))
 
 
-@pytest.mark.parametrize("M,shape", [(3, (512, 1024)), (1, (64, 20480)), (16, (256, 4096))])
+@pytest.mark.parametrize("M,shape", [(1, (64, 20480)), (2, (64, 32768))])
 def test_cases_the_kernels_do_not_serve_return_none(ta, F, M, shape):
-    """More than two rows of x, or a K that one workgroup does not hold: the library answers NF4HIP_E_SHAPE before it
-    launches anything, and the host function hands None to its caller, which takes the two-step route."""
+    """A K that one workgroup of the row kernel does not hold: the library answers NF4HIP_E_SHAPE before it launches
+    anything, and the host function hands None to its caller, which takes the two-step route."""
     N, K = shape
     qw, absmax, code = _quantized(ta, N, K, seed=N + K + 3)
     x = _randn((M, K), seed=1).to(DEV)
     resid = _randn((M, N), seed=2).to(DEV)
     nw = torch.ones(N, dtype=torch.bfloat16, device=DEV)
+    assert not F.epilogue_served(M, (N, K), resid_norm=True) and not F.epilogue_served(M, (N, K), silu_pairs=True)
     assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw)) is None
     assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), silu_pairs=True) is None
     ss = torch.ones(M, 8, device=DEV)
     assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), rowscale=(ss, 1e-5)) is None
 
 
-@pytest.mark.parametrize("batch", [1, 2, 8])
+def test_residual_epilogue_of_the_tile_kernel_needs_at_most_512_tiles(ta, F):
+    """Sixteen rows of x on [16384, 4096]: the tile kernel serves it, 1024 tiles of 16 weight rows are more partial
+    sums than a consumer's workgroup has threads -- refused for the residual epilogue, served for the others."""
+    N, K, M = 16384, 4096, 16
+    qw, absmax, code = _quantized(ta, N, K, seed=77)
+    x = _randn((M, K), seed=1).to(DEV)
+    assert not F.epilogue_served(M, (N, K), resid_norm=True) and F.epilogue_served(M, (N, K), silu_pairs=True)
+    resid = _randn((M, N), seed=2).to(DEV)
+    nw = torch.ones(N, dtype=torch.bfloat16, device=DEV)
+    assert F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw)) is None
+    out = F.matmul_nf4_epilogue(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K), silu_pairs=True)
+    two_step = importlib.import_module("lightning-thunder_amd.glue").silu_mul(
+        F.matmul_nf4(x, qw, None, absmax, code, 64, torch.bfloat16, (N, K)), pairs=True)
+    assert out is not None and torch.equal(_bits(out), _bits(two_step))
+
+
+@pytest.mark.parametrize("batch", [1, 2, 3, 8, 16])
 def test_decode_step_with_linear_epilogues(ta, glue, monkeypatch, batch):
     """The single-token step with the epilogues (five launches per layer) against the step with the glue kernels of
     their own and against the plain-PyTorch step of the same quantized model; graph replay equals the eager loop."""
@@ -196,8 +226,9 @@ def test_decode_step_with_linear_epilogues(ta, glue, monkeypatch, batch):
     real = glue.silu_mul
     monkeypatch.setattr(glue, "silu_mul", lambda *a, **k: (calls.__setitem__("silu", calls["silu"] + 1), real(*a, **k))[1])
     a = jm(first, p1, *caches[0]).float()
-    # up to two rows of x the gate-up kernel applies SiLU * up itself; beyond, the step falls back to the glue kernels
-    assert calls["silu"] == (0 if batch <= 2 else cfg.n_layer)
+    # every linear of this small model is served by a kernel with epilogues at these batch sizes: the gate-up kernel
+    # applies SiLU * up itself
+    assert calls["silu"] == 0
     cfg.linear_epilogues = False
     b = jm(first, p1, *caches[1]).float()
     cfg.hip_glue = False

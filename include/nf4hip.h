@@ -122,15 +122,19 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
  * of two.  In the reference these steps are fusions of its other executors around bnb_matmul_nf4
  * (thunder/transforms/quantization.py:34-39 has no epilogue); at one to sixteen rows of x each of them costs a launch
  * that takes as long as a small linear.  Every output is finished by exactly one thread, so nothing is computed twice.
- * fp32 absmax only; same rules as nf4hip_gemv otherwise.  A case the serving kernel does not take (rows of x beyond
- * two, K too long for one workgroup, odd N with pairs) returns NF4HIP_E_SHAPE: run nf4hip_gemv and the step by itself.
+ * fp32 absmax only; same rules as nf4hip_gemv otherwise.  What the serving kernel does not take returns
+ * NF4HIP_E_SHAPE (run nf4hip_gemv and the step by itself; nf4hip_gemv_epilogue_served answers beforehand):
+ * one or two rows of x with K > 16384 (the row kernel wants whole rows of x in one workgroup); a blocksize other than
+ * 64 where the MFMA tile kernel serves (nine and more rows of x beyond 2^24 weights, five and more beyond 2^26);
+ * RESID_NORM there with N > 8192; SILU_PAIRS with an odd N; ROWSCALE with in_parts > 512.
  *
  *   NF4HIP_EPI_SILU_PAIRS   weight rows 2j and 2j+1 are row j of the gate and of the up projection; out is [M, N/2]:
  *                           out[m][j] = bf16( bf16(silu(g)) * u ), g = bf16(sum[m][2j]), u = bf16(sum[m][2j+1])
  *                           -- what SiLU(gate) * up on the bf16 output of nf4hip_gemv gives, bit for bit.
  *   NF4HIP_EPI_RESID_NORM   d = bf16(sum[m][n] + bias[n]); r = bf16(resid_in[m][n] + d) -> resid_out[m][n];
  *                           bf16(r * norm_weight[n]) -> xnext_out[m][n]; the sum of r^2 over the outputs of one
- *                           workgroup -> out_sumsq[m * parts + workgroup], parts = nf4hip_gemv_norm_parts(M, N, K).
+ *                           workgroup (of one 16-row tile in the tile kernel) -> out_sumsq[m * parts + i], i < parts =
+ *                           nf4hip_gemv_norm_parts(M, N, K); what slot i holds does not depend on timing.
  *                           `out` is not written (NULL accepted).  resid_out may be resid_in.
  *   NF4HIP_EPI_ROWSCALE     x is the xnext_out of a RESID_NORM call and in_sumsq / in_parts its out_sumsq / parts:
  *                           sum[m][n] is multiplied by 1 / sqrt(sum_p in_sumsq[m][p] / K + eps) before the bias, i.e.

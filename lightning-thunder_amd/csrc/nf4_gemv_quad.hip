@@ -521,17 +521,14 @@ hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_
     return hipGetLastError();
 }
 
-// U = row groups in flight per wave: U * CPW 16-byte loads per lane, at most 8 (4 with eight rows of x)
+// U = row groups in flight per wave besides the one being worked on (a slot is refilled as soon as its codes are
+// copied out).  ONE is the fastest: measured against two, four and eight, four rows of x: [4096, 4096] 7.5-7.8 vs
+// 8.3-8.8 us, [14336, 4096] 12.3 vs 13.4-14.3, [28672, 4096] 17.1-17.5 vs 18.5-21.0, [4096, 14336] 13.8 vs 14.3-15.6,
+// lm_head the same; eight rows of x: [14336, 4096] 12.9-13.3 vs 14.2-15.1, the others the same.  More requests in
+// flight per wave only queue up behind each other (32 KB per CU are under way as it is) and cost registers.
 template <int CPW, int XS, bool NESTED, int EPI>
 hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
-    const int cnt = p.groups_per_band / p.row_groups;  // groups per wave and task
-    constexpr int UMAX = 8 / (CPW * XS);
-    if constexpr (UMAX >= 8 && EPI == EPI_NONE)  // with an epilogue eight groups in flight would spill
-        if (cnt >= 8) return launch_u<CPW, 8, XS, NESTED, EPI>(a, p, grid, stream, halves);
-    // nested absmax: one more register per load in flight; the residual epilogue: its pointers -- either would spill
-    if constexpr (UMAX >= 4 && !((NESTED || EPI == EPI_RESID_NORM) && CPW == 2))
-        if (cnt >= 4) return launch_u<CPW, 4, XS, NESTED, EPI>(a, p, grid, stream, halves);
-    return launch_u<CPW, 2, XS, NESTED, EPI>(a, p, grid, stream, halves);
+    return launch_u<CPW, 1, XS, NESTED, EPI>(a, p, grid, stream, halves);
 }
 
 template <bool NESTED, int EPI>
@@ -559,14 +556,10 @@ hipError_t allow_lds_epi() {
     hipError_t e;
     if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_NONE>, SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, true, MODE, EPI_NONE>, SMEM_BYTES)) != hipSuccess) return e;
-    if constexpr (U <= 4) {
-        if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_ROWSCALE>, SMEM_BYTES)) != hipSuccess) return e;
-        if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_ROWSCALE | EPI_SILU_PAIRS>, SMEM_BYTES)) != hipSuccess) return e;
-        if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_SILU_PAIRS>, SMEM_BYTES)) != hipSuccess) return e;
-        if constexpr (!(CPW == 2 && U == 4))
-            if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_RESID_NORM>, SMEM_BYTES)) != hipSuccess) return e;
-    }
-    return hipSuccess;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_ROWSCALE>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_ROWSCALE | EPI_SILU_PAIRS>, SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_SILU_PAIRS>, SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_quad_kernel<CPW, U, XS, false, MODE, EPI_RESID_NORM>, SMEM_BYTES);
 }
 
 template <int CPW, int U, int XS>
@@ -591,13 +584,9 @@ size_t gemv_quad_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 hipError_t gemv_quad_setup() {
     hipError_t e;
-    if ((e = allow_lds_cu<1, 8, 1>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<1, 4, 1>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<1, 2, 1>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<2, 4, 1>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<2, 2, 1>()) != hipSuccess) return e;
-    if ((e = allow_lds_cu<1, 4, 2>()) != hipSuccess) return e;
-    return allow_lds_cu<1, 2, 2>();
+    if ((e = allow_lds_cu<1, 1, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<2, 1, 1>()) != hipSuccess) return e;
+    return allow_lds_cu<1, 1, 2>();
 }
 
 // Nine to sixteen rows of x as two halves of up to eight, one workgroup each per task (the weight is read twice, the

@@ -488,17 +488,15 @@ hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_
     return launch_p<M, U, NESTED, false, EPI>(a, p, grid, stream);
 }
 
-// U = rows in flight per wave: as many as the wave has to do, within the register budget
-// (8 only for M = 1).
+// U = rows in flight per wave.  Four KB per wave, 64 KB per CU, cover the memory system's latency; eight rows in
+// flight (every one of the 128 registers in use, any further live value spilt) measured 0.3-0.5 us slower on the
+// 33-117 MB weights and 2.5 us slower on [28672, 8192].  Two rows of x: two rows in flight are faster up to 2^27
+// weights ([28672, 4096] 16.7-17.2 vs 17.9-18.6 us, [4096, 14336] 12.7 vs 13.4), four beyond (lm_head 55.4-56.2 vs 58.7-60.2).
 template <int M, bool NESTED, int EPI>
 hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int cnt = p.rows_per_band / p.row_lanes;  // rows per wave and task
-    // eight rows in flight fill the register file to the last register: one more live value (nested absmax: a register
-    // per slot; an epilogue: its pointers and flags) spills, and a kernel that uses scratch memory starts 2-3 us later
-    if constexpr (M == 1 && !NESTED && EPI == EPI_NONE)
-        if (cnt >= 8) return launch_u<1, 8, NESTED, EPI>(a, p, grid, stream);
-    if constexpr (M <= 2)
-        if (cnt >= 4) return launch_u<M, 4, NESTED, EPI>(a, p, grid, stream);
+    const bool four = M == 1 || (int64_t)a.N * a.K > ((int64_t)1 << 27);
+    if (cnt >= 4 && four) return launch_u<M, 4, NESTED, EPI>(a, p, grid, stream);
     return launch_u<M, 2, NESTED, EPI>(a, p, grid, stream);
 }
 
@@ -521,12 +519,10 @@ template <int M, int U, int MODE>
 hipError_t allow_lds_mode() {
     hipError_t e;
     if ((e = allow_lds_epi<M, U, MODE, EPI_NONE>()) != hipSuccess) return e;
-    if constexpr (U <= 4) {
-        if ((e = allow_lds_epi<M, U, MODE, EPI_ROWSCALE>()) != hipSuccess) return e;
-        if ((e = allow_lds_epi<M, U, MODE, EPI_ROWSCALE | EPI_SILU_PAIRS>()) != hipSuccess) return e;
-        if ((e = allow_lds_epi<M, U, MODE, EPI_SILU_PAIRS>()) != hipSuccess) return e;
-        if ((e = allow_lds_epi<M, U, MODE, EPI_RESID_NORM>()) != hipSuccess) return e;
-    }
+    if ((e = allow_lds_epi<M, U, MODE, EPI_ROWSCALE>()) != hipSuccess) return e;
+    if ((e = allow_lds_epi<M, U, MODE, EPI_ROWSCALE | EPI_SILU_PAIRS>()) != hipSuccess) return e;
+    if ((e = allow_lds_epi<M, U, MODE, EPI_SILU_PAIRS>()) != hipSuccess) return e;
+    if ((e = allow_lds_epi<M, U, MODE, EPI_RESID_NORM>()) != hipSuccess) return e;
     return gemv_allow_lds(gemv_rows_kernel<M, U, true, MODE, false>, SMEM_BYTES);
 }
 
@@ -556,7 +552,6 @@ size_t gemv_rows_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 hipError_t gemv_rows_setup() {
     hipError_t e;
-    if ((e = allow_lds_mu<1, 8>()) != hipSuccess) return e;
     if ((e = allow_lds_m<1>()) != hipSuccess) return e;
     return allow_lds_m<2>();
 }

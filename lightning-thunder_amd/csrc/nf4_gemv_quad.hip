@@ -17,7 +17,7 @@
 //    a workgroup keeps one K split for all its tasks, so x is read once per kernel, in contiguous
 //    1 KB requests, and put into that layout by a 4x4 transpose inside every quad.
 //    M = 5..8 (XS = 2): lane j also keeps x row j + 4, and every dequantised weight fragment feeds a
-//    second MFMA; a wave then covers 512 k instead of 1024 to stay within 128 registers.
+//    second MFMA (a wave then takes one or two loads per row group like the others: pick_cpw).
 //  * Code -> bf16: 256-entry LDS table indexed by a whole packed byte, both code values as one
 //    dword, replicated per lane with a 256-byte stride: address (byte << 8) | lane*4 is one
 //    v_perm_b32 and bank-conflict free.
@@ -467,10 +467,16 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a
     }
 }
 
-// k per wave = 512 * CPW.  Two loads per lane and row group keep x in 32 registers; one workgroup
-// (8 waves) then covers K <= 8192, larger K is split over workgroups.
-// Five to eight rows of x take twice the registers per load, so a wave then keeps one load's worth.
-int pick_cpw(int64_t M, int64_t K) { return (M > 4 || K <= 2 * LOAD_K) ? 1 : 2; }
+// k per wave = 512 * CPW: the fewest loads per wave with which the workgroup's 8 waves cover K, i.e. without splitting K
+// over workgroups -- one up to K = 4096, two up to 8192 (four rows of x, CPW 1 vs 2: [6144, 4096] 7.2 vs 9.2 us,
+// [4096, 4096] 6.2 vs 7.1; eight rows at [8192, 8192], 2 vs 1: 14.7 vs 16.4).  Longer K is split either way: two loads
+// with up to four rows of x ([8192, 8192]-like shapes measured 13 vs 15 us), one with eight (x then takes 64 of the
+// 128 registers at two loads; [4096, 14336]: 17.8 vs 19.0 us).
+int pick_cpw(int64_t M, int64_t K) {
+    if (K <= GEMV_WAVES * LOAD_K) return 1;
+    if (K <= 2 * GEMV_WAVES * LOAD_K) return 2;
+    return M > 4 ? 1 : 2;
+}
 
 int quad_splits(int64_t M, int64_t K) {
     const int64_t wave_k = (int64_t)pick_cpw(M, K) * LOAD_K;
@@ -533,7 +539,9 @@ hipError_t launch_c(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_
 
 template <bool NESTED, int EPI>
 hipError_t launch_e(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_t stream, int halves = 1) {
-    if (a.M > 4 || halves > 1) return launch_c<1, 2, NESTED, EPI>(a, p, grid, stream, halves);
+    if (a.M > 4 || halves > 1)  // (a half is planned as eight rows of x)
+        return pick_cpw(8, a.K) == 1 ? launch_c<1, 2, NESTED, EPI>(a, p, grid, stream, halves)
+                                     : launch_c<2, 2, NESTED, EPI>(a, p, grid, stream, halves);
     return pick_cpw(a.M, a.K) == 1 ? launch_c<1, 1, NESTED, EPI>(a, p, grid, stream) : launch_c<2, 1, NESTED, EPI>(a, p, grid, stream);
 }
 
@@ -586,6 +594,7 @@ hipError_t gemv_quad_setup() {
     hipError_t e;
     if ((e = allow_lds_cu<1, 1, 1>()) != hipSuccess) return e;
     if ((e = allow_lds_cu<2, 1, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds_cu<2, 1, 2>()) != hipSuccess) return e;
     return allow_lds_cu<1, 1, 2>();
 }
 

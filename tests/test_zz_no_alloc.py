@@ -49,7 +49,7 @@ PAIRS = [
     ((16, 6144, 4096), (16, 2048, 4096 + 512)),
     ((16, 4096, 14336), (9, 1000, 4096)),
     ((4, 8192, 28672), (2, 512, 28672)),
-    ((8, 8192, 8192), (1, 4096, 4096)),
+    ((8, 4096, 14336), (1, 4096, 4096)),
 ]
 
 

@@ -1,7 +1,7 @@
 // Dispatch of the decode-shape fused NF4 dequant-matmul (M <= 16) between its three kernels:
 // row-streaming (M = 1, 2, nf4_gemv_rows.hip), four weight rows per lane quad (M = 3, 4, and
-// M = 5..8 on weights of at most 2^26 elements, and M = 9..16 as two halves of x on weights of at most 2^24,
-// nf4_gemv_quad.hip) and MFMA tiles (the rest up to M = 16, nf4_gemv_tiles.hip).
+// M = 5..8 on weights of at most 2^26 elements -- 2^28 with 4096 < K <= 8192 -- and M = 9..16 as two halves of x on
+// weights of at most 2^24, nf4_gemv_quad.hip) and MFMA tiles (the rest up to M = 16, nf4_gemv_tiles.hip).
 //
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
@@ -33,9 +33,15 @@ hipError_t device_setup(int* cus_out) {
     return hipSuccess;
 }
 
-// Five to eight rows of x: the quad kernel starts faster (no x staging, no global split of K below
-// 8192), the tile kernel streams faster once the weights are large; they cross near 2^26 weights.
-bool quad_serves(int64_t M, int64_t N, int64_t K) { return M <= 4 || (M <= 8 && N * K <= ((int64_t)1 << 26)); }
+// Five to eight rows of x: the quad kernel starts faster (no x staging), the tile kernel streams faster once the weights
+// are large; with K = 4096 they cross near 2^26-2^27 weights ([28672, 4096]: 21.9 vs 22.2 us, lm_head 80 vs 64-71).
+// With 4096 < K <= 8192 the quad kernel's waves take two loads each and cover K without a split, and it stays ahead
+// much longer ([8192, 8192] 14.6 vs 18.8 us, [28672, 8192] 32.3 vs 36.4-38.4).
+bool quad_serves(int64_t M, int64_t N, int64_t K) {
+    if (M <= 4) return true;
+    if (M > 8) return false;
+    return N * K <= ((int64_t)1 << 26) || (K > 4096 && K <= 8192 && N * K <= ((int64_t)1 << 28));
+}
 
 // Nine to sixteen rows of x on a small weight (up to 2^24 elements): the quad kernel on two halves of x, whose
 // start-up is shorter than the tile kernel's (measured, 16 rows: [1024, 4096] 7.6 vs 10.5 us, [4096, 4096] 10.6 vs 11.5;

@@ -155,10 +155,10 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
         const bool lane_on = wave_on && kchunk + klane < K;
         const int cnt = wave_on ? (r_end - r_begin - rl + step - 1) / step : 0;  // rows of this wave
 
-        // What the epilogue needs from memory is requested first and parked in LDS before the first barrier (the
-        // oldest requests of the wave: waiting for them waits for nothing else), so that no register holds it while
-        // the weights stream.  EPI_ROWSCALE (first task): this thread's share of the producer's partial sums of
-        // squares.  EPI_RESID_NORM: residual and norm weight of the thread's first output (it rarely has a second).
+        // What the epilogue needs from memory is requested first, ahead of x and the weights.  EPI_ROWSCALE (first
+        // task): this thread's share of the producer's partial sums of squares, added up once the task's rows are
+        // done.  EPI_RESID_NORM: residual and norm weight of the thread's first output (it rarely has a second), parked
+        // in LDS before the first barrier (the wave's oldest requests: waiting for them waits for nothing else).
         const bool first_task = !table_built;
         float ssp[M];
         uint32_t pre_res = 0, pre_w = 0;
@@ -229,15 +229,6 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                 build_pair_table<F16>(smem, lut_mine, lane, wave);
             if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
             table_built = true;
-        }
-        if ((EPI & EPI_ROWSCALE) && first_task) {
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-                float ss = ssp[m];
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-                if (lane == 0) sumsq_s[m * GEMV_WAVES + wave] = ss;
-            }
         }
         if (EPI & EPI_RESID_NORM) pre_s[tid] = pre_res | (pre_w << 16);  // a slot per thread, read back by the same thread
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
@@ -336,6 +327,16 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a
                     if (lane < 8 && id < U * M && i < cnt)
                         part[((rl + i * step) * p.chunks + cw) * M + m] = total;
                 }
+            }
+        }
+        // EPI_ROWSCALE: the partial sums requested at the top have long arrived; nothing has looked at them so far
+        if ((EPI & EPI_ROWSCALE) && first_task) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float ss = ssp[m];
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                if (lane == 0) sumsq_s[m * GEMV_WAVES + wave] = ss;
             }
         }
         __syncthreads();

@@ -124,7 +124,7 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
  * that takes as long as a small linear.  Every output is finished by exactly one thread, so nothing is computed twice.
  * fp32 absmax only; same rules as nf4hip_gemv otherwise.  What the serving kernel does not take returns
  * NF4HIP_E_SHAPE (run nf4hip_gemv and the step by itself; nf4hip_gemv_epilogue_served answers beforehand):
- * one or two rows of x with K > 16384 (the row kernel wants whole rows of x in one workgroup); a blocksize other than
+ * one row of x with K > 16384 (the row kernel wants whole rows of x in one workgroup); a blocksize other than
  * 64 where the MFMA tile kernel serves (nine and more rows of x beyond 2^24 weights, five and more beyond 2^26);
  * RESID_NORM there with N > 8192; SILU_PAIRS with an odd N; ROWSCALE with in_parts > 512.
  *

@@ -1,5 +1,5 @@
 // Dispatch of the decode-shape fused NF4 dequant-matmul (M <= 16) between its three kernels:
-// row-streaming (M = 1, 2, nf4_gemv_rows.hip), four weight rows per lane quad (M = 3, 4, and
+// row-streaming (M = 1, and M = 2 where rows_serve says so, nf4_gemv_rows.hip), four weight rows per lane quad (M = 2..4, and
 // M = 5..8 on weights of at most 2^26 elements -- 2^28 with 4096 < K <= 8192 -- and M = 9..16 as two halves of x on
 // weights of at most 2^24, nf4_gemv_quad.hip) and MFMA tiles (the rest up to M = 16, nf4_gemv_tiles.hip).
 //
@@ -33,12 +33,23 @@ hipError_t device_setup(int* cus_out) {
     return hipSuccess;
 }
 
+// One row of x: the row kernel.  Two rows: the row kernel where it holds whole rows of x in one workgroup and the
+// quad kernel would split K (8192 < K <= 16384: [4096, 14336] 13.5 vs 14.9 us), and on small weights with K <= 4096
+// ([4096, 4096] 6.0 vs 6.2); elsewhere the quad kernel, which does two rows of x for the price of four:
+// [14336, 4096] 11.3 vs 13.1 us, [28672, 4096] 18.0 vs 19.5, [8192, 8192] 12.1 vs 14.3, [28672, 8192] 27 vs 32.5,
+// [8192, 28672] 37 vs 42, lm_head 60-68 vs 67-71.
+bool rows_serve(int64_t M, int64_t N, int64_t K) {
+    if (M == 1) return true;
+    if (M > 2) return false;
+    return (K > 8192 && K <= 16384) || (K <= 4096 && N * K <= ((int64_t)1 << 24));
+}
+
 // Five to eight rows of x: the quad kernel starts faster (no x staging), the tile kernel streams faster once the weights
 // are large; with K = 4096 they cross near 2^26-2^27 weights ([28672, 4096]: 21.9 vs 22.2 us, lm_head 80 vs 64-71).
 // With 4096 < K <= 8192 the quad kernel's waves take two loads each and cover K without a split, and it stays ahead
 // much longer ([8192, 8192] 14.6 vs 18.8 us, [28672, 8192] 32.3 vs 36.4-38.4).
 bool quad_serves(int64_t M, int64_t N, int64_t K) {
-    if (M <= 4) return true;
+    if (M <= 4) return true;  // (what is left of one and two rows of x included)
     if (M > 8) return false;
     return N * K <= ((int64_t)1 << 26) || (K > 4096 && K <= 8192 && N * K <= ((int64_t)1 << 28));
 }
@@ -55,14 +66,14 @@ bool quad_halves_serve(int64_t M, int64_t N, int64_t K) {
 // ---- dispatch -------------------------------------------------------------------------------
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (M <= 2) return gemv_rows_workspace_bytes(M, N, K);
+    if (rows_serve(M, N, K)) return gemv_rows_workspace_bytes(M, N, K);
     if (quad_halves_serve(M, N, K)) return gemv_quad_workspace_bytes(8, N, K);
     return quad_serves(M, N, K) ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
 }
 
 bool gemv_epilogue_possible(const MatmulArgs& a) {
     if (a.epi.flags == EPI_NONE) return true;
-    if (a.M <= 2) return gemv_rows_epilogue_possible(a);
+    if (rows_serve(a.M, a.N, a.K)) return gemv_rows_epilogue_possible(a);
     if (quad_halves_serve(a.M, a.N, a.K) || quad_serves(a.M, a.N, a.K)) return gemv_quad_epilogue_possible(a);
     return gemv_tiles_epilogue_possible(a);
 }
@@ -72,7 +83,7 @@ bool gemv_epilogue_possible(const MatmulArgs& a) {
 int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     int cus = 256;
     if (device_setup(&cus) != hipSuccess) cus = 256;
-    if (M <= 2) return gemv_rows_norm_parts(M, N, K, cus);
+    if (rows_serve(M, N, K)) return gemv_rows_norm_parts(M, N, K, cus);
     if (quad_halves_serve(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, true);
     if (quad_serves(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, false);
     return gemv_tiles_norm_parts(N);
@@ -83,7 +94,7 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     int cus = 0;
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;
-    if (a.M <= 2) return launch_gemv_rows(a, cus, stream);
+    if (rows_serve(a.M, a.N, a.K)) return launch_gemv_rows(a, cus, stream);
     if (quad_halves_serve(a.M, a.N, a.K)) return launch_gemv_quad_halves(a, cus, stream);
     return quad_serves(a.M, a.N, a.K) ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);
 }

@@ -560,7 +560,7 @@ def matmul_nf4_epilogue(x, qweight, bias, absmax, quant_map, blocksize, dtype, s
     * ``silu_pairs``: weight rows 2j / 2j+1 are gate row j / up row j; returns ``silu(gate) * up`` [rows, N/2].
 
     Returns None where the library does not serve the case (more than sixteen rows of x, nested absmax, other dtypes,
-    one or two rows of x with K > 16384, ...; ``epilogue_served`` answers beforehand): the caller then runs
+    one row of x with K > 16384, ...; ``epilogue_served`` answers beforehand): the caller then runs
     ``matmul_nf4`` and the step by itself."""
     N, K = (int(s) for s in shape)
     x2 = x.reshape(-1, K)

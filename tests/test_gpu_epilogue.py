@@ -48,7 +48,7 @@ PAIR_SHAPES = [(1024, 512), (28672, 4096), (2048, 14336), (272, 2080)]
 
 
 def _served(F, M, N, K, **which):
-    """K % 32 == 0 up to four rows of x, K % 512 == 0 beyond, K within one workgroup's reach up to two; the residual
+    """K % 32 == 0 up to four rows of x, K % 512 == 0 beyond, K within one workgroup's reach with one row of x; the residual
     epilogue of the tile kernel (nine and more rows of x, or a large weight) leaves one partial sum per 16 weight rows,
     at most 512 of them."""
     return F.epilogue_served(M, (N, K), **which)
@@ -59,7 +59,7 @@ def _served(F, M, N, K, **which):
 def test_silu_pairs_gives_the_two_step_bits(ta, F, glue, M, shape):
     N, K = shape
     if not _served(F, M, N, K, silu_pairs=True):
-        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup up to two)")
+        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup with one row of x)")
     print(f"epilogue silu_pairs M={M} N={N} K={K}", flush=True)
     qw, absmax, code = _quantized(ta, N, K, seed=N + K)
     x = _randn((M, K), seed=3 * N + M).to(DEV)
@@ -80,7 +80,7 @@ RESID_SHAPES = [(4096, 4096), (4096, 14336), (517, 1056), (256, 16384), (8192, 8
 def test_resid_norm_epilogue(ta, F, M, shape):
     N, K = shape
     if not _served(F, M, N, K, resid_norm=True):
-        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup up to two)")
+        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup with one row of x)")
     print(f"epilogue resid_norm M={M} N={N} K={K}", flush=True)
     qw, absmax, code = _quantized(ta, N, K, seed=N + K + 1)
     x = _randn((M, K), seed=5 * N + M).to(DEV)
@@ -114,7 +114,7 @@ def test_rowscale_epilogue_against_float64(ta, F, glue, oracle, M, silu, shape):
     if N == 128256 and (silu or M != 1):
         pytest.skip("the lm_head is checked once")
     if not _served(F, M, N, K, rowscale_parts=37, silu_pairs=silu):
-        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup up to two)")
+        pytest.skip("not a shape the kernels take with an epilogue (K % 512 beyond four rows of x, K within one workgroup with one row of x)")
     print(f"epilogue rowscale M={M} N={N} K={K} silu={silu}", flush=True)
     qw, absmax, code = _quantized(ta, N, K, seed=N + K + 2)
     r = _randn((M, K), seed=11 * N + M, std=3.0)
@@ -168,7 +168,7 @@ def test_chain_of_epilogues_is_a_decoder_layer_tail(ta, F, oracle):
     assert torch.equal(_bits(xn2), _bits((r2.float() * w1.to(DEV).float()).to(torch.bfloat16)))
 
 
-@pytest.mark.parametrize("M,shape", [(1, (64, 20480)), (2, (64, 32768))])
+@pytest.mark.parametrize("M,shape", [(1, (64, 20480)), (1, (64, 32768))])
 def test_cases_the_kernels_do_not_serve_return_none(ta, F, M, shape):
     """A K that one workgroup of the row kernel does not hold: the library answers NF4HIP_E_SHAPE before it launches
     anything, and the host function hands None to its caller, which takes the two-step route."""

@@ -238,3 +238,36 @@ def test_decode_step_with_linear_epilogues(ta, glue, monkeypatch, batch):
     for kc, vc in caches[1:]:
         torch.testing.assert_close(caches[0][0][:, :, :, :17].float(), kc[:, :, :, :17].float(), rtol=2e-2, atol=2e-2)
         torch.testing.assert_close(caches[0][1][:, :, :, :17].float(), vc[:, :, :, :17].float(), rtol=2e-2, atol=2e-2)
+
+
+def test_epilogues_hold_over_many_launches_with_k_split_over_workgroups(ta, F):
+    """A producer / consumer pair whose kernels split K over workgroups (eight rows of x on [4096, 14336]: the quad
+    kernel's last-arriving workgroup runs the residual epilogue; sixteen rows on [6144, 4096]: the tile kernel's
+    reducing wave applies the row scale), 600 times on the stream's one workspace: every result must equal the first
+    bit for bit, whichever workgroup arrived last.  The comparison runs on the device; the host looks every 100."""
+    print("epilogues with split K, 600 launches", flush=True)
+    lib = ta._lib.load()
+    M8, M16 = 8, 16
+    qd, ad, code = _quantized(ta, 4096, 14336, seed=21)
+    qq, aq, _ = _quantized(ta, 6144, 4096, seed=22)
+    assert lib.nf4hip_gemv_workspace_bytes(M8, 4096, 14336) > 65536 * 4 and lib.nf4hip_gemv_workspace_bytes(M16, 6144, 4096) > 65536 * 4
+    x8 = _randn((M8, 14336), seed=23).to(DEV)
+    r8 = _randn((M8, 4096), seed=24, std=2.0).to(DEV)
+    nw = (1.0 + _randn((4096,), seed=25, std=0.1).float()).to(torch.bfloat16).to(DEV)
+    xn16 = _randn((M16, 4096), seed=26, std=2.0).to(DEV)
+    ss16 = (torch.rand(M16, 256, device=DEV) * 100.0).contiguous()
+
+    def once():
+        r, xn, ss = F.matmul_nf4_epilogue(x8, qd, None, ad, code, 64, torch.bfloat16, (4096, 14336), resid_norm=(r8, nw))
+        q = F.matmul_nf4_epilogue(xn16, qq, None, aq, code, 64, torch.bfloat16, (6144, 4096), rowscale=(ss16, 1e-5))
+        return r, xn, ss, q
+
+    first = once()
+    bad = torch.zeros((), dtype=torch.bool, device=DEV)
+    for it in range(600):
+        got = once()
+        for a, b in zip(got, first):
+            bad |= (a.view(torch.int32 if a.dtype == torch.float32 else torch.int16) !=
+                    b.view(torch.int32 if b.dtype == torch.float32 else torch.int16)).any()
+        if it % 100 == 99:
+            assert not bool(bad), f"a result changed between launches {it - 99} and {it}"

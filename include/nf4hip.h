@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define NF4HIP_ABI_VERSION 2
+#define NF4HIP_ABI_VERSION 3
 
 #define NF4HIP_BF16 0
 #define NF4HIP_F16 1

@@ -11,7 +11,7 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 BF16, F16, F32 = 0, 1, 2
 

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(ta):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/nf4hip.h but not exported"
     assert sorted(ta._lib.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
-    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 2
+    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 3
 
 
 def test_missing_library_fails_loudly(ta, tmp_path):

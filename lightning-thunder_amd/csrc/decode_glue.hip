@@ -117,8 +117,12 @@ __global__ __launch_bounds__(NORM_THREADS) void add_rmsnorm_kernel(uint16_t* x, 
 }
 
 constexpr int ATTN_THREADS = 256;
+constexpr int ATTN_XCDS = 8;  // workgroup id % 8 is the XCD a workgroup runs on
 
-// One workgroup per (query head, sequence, split of the cached keys).  qkv holds this step's q, k, v
+// One workgroup per (query head, sequence, split of the cached keys).  The query heads of one kv group read the same
+// cached rows: the 1-D grid is laid out so that they are neighbours in dispatch order AND land on one XCD (workgroups go
+// to the 8 XCDs round robin, id % 8), i.e. behind one L2 -- the cached rows then come from HBM once instead of once per
+// query head.  qkv holds this step's q, k, v
 // rows of the sequence; position p = *pos.  The new k (rotated) and v are written to the caches by
 // one workgroup of each kv group and used from LDS by all of them, so no workgroup depends on
 // another's write.  With more than one split every workgroup leaves (max, sum, unnormalised output)
@@ -127,8 +131,8 @@ constexpr int ATTN_THREADS = 256;
 template <int HD>
 __global__ __launch_bounds__(ATTN_THREADS) void attention_decode_kernel(const uint16_t* qkv, const int64_t* pos,
                                                                         const float* cos_t, const float* sin_t,
-                                                                        uint16_t* kcache, uint16_t* vcache, int H,
-                                                                        int Hkv, int max_seq, uint16_t* out,
+                                                                        uint16_t* kcache, uint16_t* vcache, int batch,
+                                                                        int H, int Hkv, int max_seq, uint16_t* out,
                                                                         int splits, uint32_t* counters, float* partials) {
     constexpr int LPK = HD / 16;            // lanes per key: 16 elements each
     constexpr int KPI = ATTN_THREADS / LPK;  // keys per iteration of the score loop
@@ -143,9 +147,13 @@ __global__ __launch_bounds__(ATTN_THREADS) void attention_decode_kernel(const ui
     float* p_s = acc_s + SG * HD;     // [max_seq] scores, then probabilities
 
     const int tid = threadIdx.x;
-    const int h = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
+    // a stream = (sequence, split, kv head): XCD slot stream_id % 8; its `rep` query heads are 8 workgroup ids apart
     const int rep = H / Hkv;
-    const int hk = h / rep;
+    const int slot = (int)blockIdx.x & (ATTN_XCDS - 1), outer = (int)blockIdx.x / ATTN_XCDS;
+    const int stream_id = (outer / rep) * ATTN_XCDS + slot;
+    if (stream_id >= batch * splits * Hkv) return;  // uniform: padding of the last group of eight streams
+    const int hk = stream_id % Hkv, split = (stream_id / Hkv) % splits, b = stream_id / (Hkv * splits);
+    const int h = hk * rep + outer % rep;
     const int p = (int)*pos;
     if (p < 0 || p >= max_seq) return;  // uniform: a position outside the cache touches nothing
     // this workgroup's cached keys [lo, hi) of 0 .. p-1; the last split also takes the new key p
@@ -483,7 +491,8 @@ __attribute__((visibility("default"))) int nf4hip_decode_attention(const void* q
     float* partials = need ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + ATTN_COUNTER_BYTES) : nullptr;
     const int sg = ATTN_THREADS / (head_dim / 8);
     const size_t lds = sizeof(float) * (size_t)(3 * head_dim + 8 + sg * head_dim + max_seq);
-    const dim3 grid((unsigned)n_head, (unsigned)batch, (unsigned)splits);
+    const int64_t streams = batch * splits * n_kv_head;
+    const dim3 grid((unsigned)((streams + ATTN_XCDS - 1) / ATTN_XCDS * ATTN_XCDS * (n_head / n_kv_head)));
     // allow the whole 160 KB of LDS once per device (what a launch takes is its own `lds`)
     static bool ready[64] = {};
     int dev = 0;
@@ -497,7 +506,7 @@ __attribute__((visibility("default"))) int nf4hip_decode_attention(const void* q
     auto launch = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, dim3(ATTN_THREADS), lds, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(qkv), pos, cos_t, sin_t, static_cast<uint16_t*>(kcache),
-                           static_cast<uint16_t*>(vcache), n_head, n_kv_head, (int)max_seq, static_cast<uint16_t*>(out),
+                           static_cast<uint16_t*>(vcache), (int)batch, n_head, n_kv_head, (int)max_seq, static_cast<uint16_t*>(out),
                            splits, counters, partials);
     };
     if (head_dim == 128)

@@ -7,6 +7,36 @@ namespace nf4 {
 
 constexpr int GEMV_THREADS = 512;  // 8 waves; two workgroups per CU
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
+
+// What a wave's first requests depend on -- code book, x, codes, absmax, N, K, M -- travels ahead of the argument
+// structs as scalars.  This library is built with -mllvm -amdgpu-kernarg-preload-count: the leading scalar arguments of
+// a kernel (up to 14 dwords; structs are passed by reference and never qualify) then arrive in SGPRs with the wave, and
+// the kernel requests its code-book entry, x and first weights without first waiting for a load from the argument
+// block.  Measured on the row kernel, one row of x: [6144, 4096] 7.1 -> 6.8 us, [14336, 4096] 11.2 -> 10.7,
+// [4096, 14336] 11.5 -> 11.1, [28672, 4096] 17.0 -> 16.6; a 161-linear decode step 1.764 -> 1.715 ms.
+// 11 dwords here; a kernel adds up to three of its launch plan.
+#define NF4_HOT_PARAMS                                                                                          \
+    const float *hot_lut, const uint16_t *hot_x, const uint8_t *hot_packed, const float *hot_absmax, int hot_N, \
+        int hot_K, int hot_M_log2
+// (with nested absmax the slot of the absmax pointer carries the pointer to their 8-bit codes)
+#define NF4_HOT_VALUES(a)                                                                                              \
+    (a).lut16, (a).x, (a).packed, ((a).nested.q ? reinterpret_cast<const float*>((a).nested.q) : (a).absmax), (a).N, (a).K, \
+        ((a).M | ((a).block_log2 << 8))
+#define NF4_HOT_NAMES hot_lut, hot_x, hot_packed, hot_absmax, hot_N, hot_K, hot_M_log2
+
+template <bool NESTED>
+__device__ __forceinline__ MatmulArgs with_hot_args(const MatmulArgs& in, NF4_HOT_PARAMS) {
+    MatmulArgs a = in;
+    a.lut16 = hot_lut; a.x = hot_x; a.packed = hot_packed;
+    if (NESTED) {
+        a.nested.q = reinterpret_cast<const uint8_t*>(hot_absmax);
+        a.absmax = nullptr;
+    } else {
+        a.absmax = hot_absmax;
+    }
+    a.N = hot_N; a.K = hot_K; a.M = hot_M_log2 & 0xff; a.block_log2 = hot_M_log2 >> 8;
+    return a;
+}
 constexpr int GEMV_TABLE_BYTES = 256 * 256;     // 256 byte values x 64 lanes x 4 B
 constexpr int GEMV_COUNTER_BYTES = (int)GEMV_COUNTER_REGION_BYTES;  // split-K arrival counters at the head of the workspace
 

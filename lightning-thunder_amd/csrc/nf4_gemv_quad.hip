@@ -101,7 +101,13 @@ __device__ __forceinline__ float reduce_rows(const float t[4], int lane) {
 // keeps to one row of x (m = tid % MP, MP the power of two that holds M), lanes of equal m are added by a butterfly
 // and the waves in order.
 template <int CPW, int U, int XS, bool NESTED, int MODE, int EPI = EPI_NONE>
-__global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(MatmulArgs a, QuadPlan p) {
+__global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(NF4_HOT_PARAMS, int hot_plan, int hot_groups_per_band, int hot_ntasks,
+                                                                     MatmulArgs a_rest, QuadPlan p_rest) {
+    // (arguments in SGPRs at wave start; the structs supply what is wanted later)
+    MatmulArgs a = with_hot_args<NESTED>(a_rest, NF4_HOT_NAMES);
+    QuadPlan p = p_rest;
+    p.waves_k = hot_plan & 0xf; p.row_groups = (hot_plan >> 4) & 0xf; p.aligned = (hot_plan >> 8) & 1; p.splits = hot_plan >> 9;
+    p.groups_per_band = hot_groups_per_band; p.ntasks = hot_ntasks;
     static_assert(EPI == EPI_NONE || !NESTED, "epilogues come with fp32 absmax only");
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -519,11 +525,14 @@ hipError_t launch_u(const MatmulArgs& a, const QuadPlan& p, int grid, hipStream_
     const int mode = gemv_arith_mode(a.K, true);
     const dim3 g((unsigned)grid, (unsigned)halves);
     if (mode == ARITH_EXACT)
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_EXACT, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a),
+                           p.waves_k | (p.row_groups << 4) | (p.aligned << 8) | (p.splits << 9), p.groups_per_band, p.ntasks, a, p);
     else if (mode == ARITH_F16)
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_F16, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a),
+                           p.waves_k | (p.row_groups << 4) | (p.aligned << 8) | (p.splits << 9), p.groups_per_band, p.ntasks, a, p);
     else
-        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_quad_kernel<CPW, U, XS, NESTED, ARITH_BF16, EPI>), g, dim3(GEMV_THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a),
+                           p.waves_k | (p.row_groups << 4) | (p.aligned << 8) | (p.splits << 9), p.groups_per_band, p.ntasks, a, p);
     return hipGetLastError();
 }
 

@@ -118,7 +118,13 @@ __device__ __forceinline__ int reduce8_id(int lane) { return (lane & 1) | ((lane
 //                EPI_RESID_NORM: a thread's outputs all belong to one row of x (M divides the workgroup size), so its
 //                squares add up in a register; lanes of equal m are added by a butterfly, waves in order.
 template <int M, int U, bool NESTED, int MODE, bool PAIRED, int EPI = EPI_NONE>
-__global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(MatmulArgs a, RowsPlan p) {
+__global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(NF4_HOT_PARAMS, int hot_plan, int hot_rows_per_band, int hot_ntasks,
+                                                                     MatmulArgs a_rest, RowsPlan p_rest) {
+    // (arguments in SGPRs at wave start; the structs supply what is wanted later)
+    const MatmulArgs a = with_hot_args<NESTED>(a_rest, NF4_HOT_NAMES);
+    RowsPlan p = p_rest;
+    p.chunks = hot_plan & 0xf; p.row_lanes = (hot_plan >> 4) & 0xf; p.aligned = (hot_plan >> 8) & 1; p.splits = hot_plan >> 9;
+    p.rows_per_band = hot_rows_per_band; p.ntasks = hot_ntasks;
     static_assert(EPI == EPI_NONE || (!NESTED && GEMV_THREADS % M == 0 && M <= 2), "epilogues: fp32 absmax, M = 1, 2");
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -474,11 +480,14 @@ template <int M, int U, bool NESTED, bool PAIRED, int EPI>
 hipError_t launch_p(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int mode = gemv_arith_mode(a.K, true);
     if (mode == ARITH_EXACT)
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_EXACT, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a),
+                           p.chunks | (p.row_lanes << 4) | (p.aligned << 8) | (p.splits << 9), p.rows_per_band, p.ntasks, a, p);
     else if (mode == ARITH_F16)
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_F16, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a),
+                           p.chunks | (p.row_lanes << 4) | (p.aligned << 8) | (p.splits << 9), p.rows_per_band, p.ntasks, a, p);
     else
-        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, a, p);
+        hipLaunchKernelGGL((gemv_rows_kernel<M, U, NESTED, ARITH_BF16, PAIRED, EPI>), dim3(grid), dim3(GEMV_THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a),
+                           p.chunks | (p.row_lanes << 4) | (p.aligned << 8) | (p.splits << 9), p.rows_per_band, p.ntasks, a, p);
     return hipGetLastError();
 }
 

@@ -461,7 +461,14 @@ __device__ __forceinline__ void scale_x_slice_to_f16(uint4 (&v)[XUNITS], int n, 
 // (added over the tile's 16 lanes by a butterfly), so what a partial sum holds does not depend on which workgroup
 // finished the tile.
 template <bool B64, bool NESTED, int R, int MODE, bool STEADY, int EPI = EPI_NONE>
-__global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(MatmulArgs a, Plan p) {
+__global__ __launch_bounds__(THREADS, 2) void gemv_tiles_kernel(NF4_HOT_PARAMS, int hot_splits, int hot_range_phases, int hot_tg_step,
+                                                                MatmulArgs a_rest) {
+    // (arguments in SGPRs at wave start; the struct supplies what is wanted later)
+    const MatmulArgs a = with_hot_args<NESTED>(a_rest, NF4_HOT_NAMES);
+    Plan p;
+    p.tile_groups = (a.N + 16 * WAVES - 1) / (16 * WAVES);
+    p.total_phases = a.K / PHASE_K;
+    p.splits = hot_splits; p.range_phases = hot_range_phases; p.tg_step = hot_tg_step;
     static_assert(EPI == EPI_NONE || (B64 && !NESTED), "epilogues: fp32 absmax, blocksize 64");
     constexpr bool EXACT = MODE == ARITH_EXACT, F16 = MODE == ARITH_F16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -876,7 +883,7 @@ hipError_t launch_rs(const MatmulArgs& a, const Plan& p, int grid, hipStream_t s
         case EPI_RESID_NORM: kern = gemv_tiles_kernel<true, false, R, MODE, STEADY, EPI_RESID_NORM>; break;
         default: return hipErrorNotSupported;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, a, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), SMEM_BYTES, stream, NF4_HOT_VALUES(a), p.splits, p.range_phases, p.tg_step, a);
     return hipGetLastError();
 }
 

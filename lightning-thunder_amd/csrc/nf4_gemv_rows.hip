@@ -500,13 +500,14 @@ hipError_t launch_u(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_
 
 // U = rows in flight per wave.  Four KB per wave, 64 KB per CU, cover the memory system's latency; eight rows in
 // flight (every one of the 128 registers in use, any further live value spilt) measured 0.3-0.5 us slower on the
-// 33-117 MB weights and 2.5 us slower on [28672, 8192].  Two rows of x: two rows in flight are faster up to 2^27
-// weights ([28672, 4096] 16.7-17.2 vs 17.9-18.6 us, [4096, 14336] 12.7 vs 13.4), four beyond (lm_head 55.4-56.2 vs 58.7-60.2).
+// 33-117 MB weights and 2.5 us slower on [28672, 8192].  Two rows of x: two rows in flight ([28672, 4096] 16.7-17.2 vs
+// 17.9-18.6 us, [4096, 14336] 12.7 vs 13.4; four rows in flight and two rows of x leave no register free).
 template <int M, bool NESTED, int EPI>
 hipError_t launch_m(const MatmulArgs& a, const RowsPlan& p, int grid, hipStream_t stream) {
     const int cnt = p.rows_per_band / p.row_lanes;  // rows per wave and task
-    const bool four = M == 1 || (int64_t)a.N * a.K > ((int64_t)1 << 27);
-    if (cnt >= 4 && four) return launch_u<M, 4, NESTED, EPI>(a, p, grid, stream);
+    if constexpr (M == 1) {
+        if (cnt >= 4) return launch_u<1, 4, NESTED, EPI>(a, p, grid, stream);
+    }
     return launch_u<M, 2, NESTED, EPI>(a, p, grid, stream);
 }
 
@@ -546,7 +547,7 @@ hipError_t allow_lds_mu() {
 
 template <int M>
 hipError_t allow_lds_m() {
-    if constexpr (M <= 2) {
+    if constexpr (M == 1) {  // four rows in flight: one row of x only (launch_m)
         const hipError_t e = allow_lds_mu<M, 4>();
         if (e != hipSuccess) return e;
     }

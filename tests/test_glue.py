@@ -127,6 +127,8 @@ def _rope_ref(x, cos, sin):  # x [..., hd] fp32, cos/sin [hd]
 @pytest.mark.parametrize("B,H,Hkv,hd,max_seq,p", [
     (1, 32, 8, 128, 640, 512), (8, 32, 8, 128, 640, 639), (3, 8, 2, 64, 64, 0), (2, 8, 8, 64, 64, 17),
     (2, 4, 1, 128, 300, 299), (1, 32, 8, 128, 640, 1), (40, 32, 8, 128, 96, 70), (16, 32, 8, 128, 640, 300),
+    # (sequence, split, kv head) streams that do not fill the last group of eight: 201 and 126 of them
+    (67, 4, 1, 64, 48, 40), (9, 16, 2, 64, 80, 79),
 ])
 def test_attention_decode(glue, B, H, Hkv, hd, max_seq, p):
     print(f"attention_decode B={B} H={H} Hkv={Hkv} hd={hd} max_seq={max_seq} p={p}", flush=True)

@@ -208,7 +208,7 @@ def test_gemv_rows(ta, oracle, M):
 @pytest.mark.parametrize(
     "N,K",
     [(16, 512), (48, 512), (100, 1024), (130, 2048), (1024, 4096), (4096, 4096), (1000, 14336), (2048 + 16, 8192),
-     (300, 28672), (77, 32768 + 512)],
+     (300, 28672), (77, 32768 + 512), (8, 1 << 20)],  # the last: K split over 64 to 256 workgroups
 )
 @pytest.mark.parametrize("M", [1, 2, 4, 5, 16])
 def test_gemv_shapes(ta, oracle, N, K, M):

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define NF4HIP_ABI_VERSION 3
+#define NF4HIP_ABI_VERSION 4
 
 #define NF4HIP_BF16 0
 #define NF4HIP_F16 1
@@ -178,7 +178,8 @@ int nf4hip_gemv_epilogue(const void* x, int x_dtype, int64_t M, const uint8_t* p
  *     (different streams, or a graph replayed beside eager calls) race.  The array keeps the last
  *     call's partial sums; the counters at its head are back at zero whenever a call has completed.
  *   - The first call on a GPU resolves the array's address and clears its counters with a small
- *     kernel on `stream`; make that call outside a capture.
+ *     kernel on `stream`; make that call outside a capture (under capture it fails with NF4HIP_E_HIP
+ *     and records nothing).
  */
 #define NF4HIP_STATIC_SCRATCH_BYTES (4u << 20)
 int nf4hip_gemv_static(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
@@ -196,6 +197,14 @@ int nf4hip_gemv_static(const void* x, int x_dtype, int64_t M, const uint8_t* pac
  * matters, one stream at a time; the two kernels may share one workspace.
  */
 size_t nf4hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+/*
+ * The launch plan nf4hip_gemm would use for a shape (no GPU needed): plan[0] rows of x per tile (64, 128 or 256),
+ * plan[1] tiles (tiles of x rows x tiles of 256 weight rows), plan[2] pieces a tile is cut into along K (they meet in
+ * the workspace), plan[3] workgroups launched.  For host code that chooses between this kernel and dequantize +
+ * dense GEMM (the choice bitsandbytes.matmul_4bit makes at thunder/transforms/quantization.py:39) without keeping
+ * a copy of the launcher's rules.  K must be a multiple of 64.
+ */
+int nf4hip_gemm_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]);
 int nf4hip_gemm(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
                 const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
                 size_t workspace_bytes, void* stream);

@@ -369,7 +369,8 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_kernel(const uint16_t* 
     const int tid = threadIdx.x;
     const uint16_t* row = logits + (int64_t)blockIdx.x * vocab;
     auto key_of = [](uint32_t bf, int64_t idx) -> unsigned long long {
-        const uint32_t bits = bf << 16;
+        uint32_t bits = bf << 16;
+        if ((bits << 1) == 0) bits = 0;  // -0.0 and +0.0 compare equal: one key for both, the lower index wins
         uint32_t ord = (bits & 0x80000000u) ? ~bits : bits | 0x80000000u;
         if ((bits & 0x7fffffffu) > 0x7f800000u) ord = 0xffffffffu;  // NaN
         return ((unsigned long long)ord << 32) | (uint32_t)(0xffffffffu - (uint32_t)idx);

@@ -35,6 +35,10 @@ hipError_t static_scratch(void** out, hipStream_t stream) {
     if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
     void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (!p) {
+        // the set-up below must run, not be recorded: refuse a first call made under stream capture
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+            return hipErrorStreamCaptureUnsupported;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return e;
         if (!p) return hipErrorInvalidSymbol;
@@ -278,6 +282,16 @@ int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const f
 
 size_t nf4hip_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) { return nf4::gemv_workspace_bytes(M, N, K); }
 size_t nf4hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return nf4::gemm_workspace_bytes(M, N, K); }
+
+int nf4hip_gemm_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]) {
+    if (!plan) return fail(NF4HIP_E_NULL, "nf4hip_gemm_plan: plan is null");
+    if (M <= 0 || N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX || M > INT32_MAX || K % 64)
+        return fail(NF4HIP_E_SHAPE, "nf4hip_gemm_plan: M, N, K must be positive and K a multiple of 64");
+    int p[4];
+    nf4::gemm_plan(M, N, K, p);
+    for (int i = 0; i < 4; ++i) plan[i] = p[i];
+    return NF4HIP_OK;
+}
 
 int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
                 const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,

@@ -77,6 +77,11 @@ hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream);
 int gemm_wide_tile_rows(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemm_wide(const MatmulArgs& a, hipStream_t stream);
 size_t gemm_wide_workspace_bytes(int64_t M, int64_t N, int64_t K);
+// The launch plan of the fused GEMM for a shape, as the launchers compute it: plan[0] rows of x per tile (64, 128,
+// 256), plan[1] tiles (tiles of x rows times tiles of 256 weight rows), plan[2] pieces a tile is cut into along K,
+// plan[3] workgroups launched.
+void gemm_wide_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
+void gemm_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
 
 // ---------------------------------------------------------------------------------------------
 // device helpers
@@ -95,6 +100,14 @@ __device__ __forceinline__ uint4 load16_stream(const void* p) {
 __device__ __forceinline__ uint4 load16(const void* p) {
     const u32x4_t v = *reinterpret_cast<const u32x4_t*>(p);
     return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// 4-byte and 16-byte streaming loads of fp32 absmax values: like the codes they are read exactly once.
+__device__ __forceinline__ float load_f32_stream(const float* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ float4 load_f32x4_stream(const float* p) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
 }
 
 // 16-byte store, ordinary or streaming (non-temporal: the data is not meant to stay in the caches).
@@ -117,20 +130,27 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// Hand-off of split-K partial sums between workgroups: the producer stores its partials with
-// agent-scope relaxed atomic stores (write-through to L2, the level all CUs of the device share),
-// calls publish_partials(), then counts its arrival with an agent-scope relaxed RMW; the last arriver
-// calls acquire_partials() and reads every producer's partials with agent-scope relaxed atomic loads
-// (which bypass its CU's L1).
-//   * For the compiler the two fences are ordering points: no store may sink below the release
-//     fence, no load may be hoisted above the acquire fence, and neither may be moved across the
-//     counter RMW between them.
-//   * For the hardware the release fence at workgroup scope costs nothing on this target (a CU keeps
-//     a workgroup's vector memory operations in order), so the explicit s_waitcnt(0) behind it is
-//     what makes the wave wait until L2 has acknowledged every store before the arrival is counted.
-//   * An agent-scope fence would also be correct, but it writes back and invalidates the whole L2
-//     (measured at 45 us per launch); nothing here needs that, because every access to the shared
-//     data is itself an agent-scope atomic.
+// Hand-off of split-K partial sums between workgroups, which may run on different XCDs (eight on this part, each with
+// an L2 of its own; what they share is the memory-side Infinity Cache and HBM).  The producer stores its partials with
+// agent-scope relaxed atomic stores, calls publish_partials(), then counts its arrival with an agent-scope relaxed
+// RMW on the band's counter; the last arriver calls acquire_partials() and reads every producer's partials with
+// agent-scope relaxed atomic loads.  What is relied on:
+//   * EVERY access to the shared words -- partials and counters, writes and reads -- is itself an agent-scope atomic.
+//     On this target such an access carries the cache-policy bits that make it coherent across the agent: the store
+//     is written through the issuing XCD's L2 to memory, the load and the RMW are served from there and not from a
+//     stale line of the reader's L1 or L2.  No plain load or store ever touches these words, so no cache holds a copy
+//     that a fence would have to write back or invalidate.
+//   * The producer's s_waitcnt(0) makes the wave wait until every one of its stores has been acknowledged, i.e. has
+//     reached the level at which agent-scope accesses of other XCDs see it, BEFORE the arrival is counted (where one thread
+//     counts for a whole workgroup, a workgroup barrier stands between the waves' waits and that RMW; where a wave
+//     counts for itself, the RMW follows its own wait).  The last arriver's loads are issued after its RMW has returned -- a data dependence through the flag --
+//     so they are served after every producer's acknowledged stores.
+//   * The two fences are there for the COMPILER: no store may sink below the release fence, no load may be hoisted
+//     above the acquire fence, and neither may move across the counter RMW between them.  At workgroup scope they
+//     order nothing at agent scope in the language's memory model and emit no cache maintenance; the ordering across
+//     XCDs comes from the two points above.
+//   * An agent-scope fence pair would be the model-blessed spelling, but on this target it writes back and
+//     invalidates the whole L2 (measured at 45 us per launch), which nothing here needs.
 __device__ __forceinline__ void publish_partials() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);

@@ -385,6 +385,16 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return GEMM_COUNTER_BYTES + (size_t)((N + BN - 1) / BN) * splits * bm * BN * sizeof(float);
 }
 
+void gemm_plan(int64_t M, int64_t N, int64_t K, int plan[4]) {
+    if (M > 128 && M * K * 2 < ((int64_t)1 << 32)) return gemm_wide_plan(M, N, K, plan);
+    const int bm = M <= 64 ? 64 : M <= 128 ? 128 : 256;
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + BN - 1) / BN);
+    plan[0] = bm;
+    plan[1] = (int)tiles;
+    plan[2] = gemm_splits(M, N, K);
+    plan[3] = (int)tiles * plan[2];
+}
+
 hipError_t launch_gemm(const MatmulArgs& a, hipStream_t stream) {
     // the smallest tile height that covers x with one tile: the weight tile is expanded once per tile of x rows
     if (a.M <= 64) return a.nested.q ? launch_tile<true, 64>(a, stream) : launch_tile<false, 64>(a, stream);

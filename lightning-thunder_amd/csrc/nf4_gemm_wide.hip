@@ -629,6 +629,15 @@ size_t gemm_wide_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return s.pieces > 1 ? wide_tail_bytes(s.tail_tiles, s.pieces, bm) : 0;
 }
 
+void gemm_wide_plan(int64_t M, int64_t N, int64_t K, int plan[4]) {
+    const int bm = gemm_wide_tile_rows(M, N, K);
+    const WideSchedule s = wide_schedule(M, N, K, bm, ~(size_t)0);
+    plan[0] = bm;
+    plan[1] = s.m_tiles * s.n_tiles;
+    plan[2] = s.pieces;
+    plan[3] = s.full + s.tail_tiles * s.pieces;
+}
+
 hipError_t launch_gemm_wide(const MatmulArgs& a, hipStream_t stream) {
     const bool nested = a.nested.q != nullptr;
     if (gemm_wide_tile_rows(a.M, a.N, a.K) == 128)

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_quad_kernel(NF4_HOT_PARA
                         sq[u][c] = __uint_as_float((uint32_t)a.nested.q[blk]);
                         s2[u][c] = a.nested.absmax2[blk >> a.nested.nested_log2];
                     } else {
-                        sq[u][c] = a.absmax[blk];
+                        sq[u][c] = load_f32_stream(a.absmax + blk);
                     }
                 }
         };

@@ -214,12 +214,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(NF4_HOT_PARA
                         sq[u] = __uint_as_float((uint32_t)a.nested.q[blk]);
                         s2[u] = a.nested.absmax2[blk >> a.nested.nested_log2];
                     } else if (!PAIRED) {
-                        sq[u] = a.absmax[blk];
+                        sq[u] = load_f32_stream(a.absmax + blk);
                     } else if ((u & 1) == 0) {
                         // even lanes: this row; odd lanes: the row of slot u + 1 (the wave's next row, if it has one)
                         const int row2 = r_begin + rl + min(i + 1, cnt - 1) * step;
                         const int64_t blk2 = (((int64_t)row2 * K + kchunk) >> a.block_log2) + (klane >> a.block_log2);
-                        sq[u] = a.absmax[(lane & 1) ? blk2 : blk];
+                        sq[u] = load_f32_stream(a.absmax + ((lane & 1) ? blk2 : blk));
                     }
                 }
             };

@@ -237,6 +237,7 @@ __device__ __forceinline__ void load_phase(const MatmulArgs& a, PhaseRegs& r, co
         }
     } else if (B64) {
         const float* sp = a.absmax + (e0 >> 6) + s_off;
+        // (ordinary loads: a phase takes 32 bytes of a row's absmax line, the next phases the rest of it from the caches)
         r.s[0] = *reinterpret_cast<const float4*>(sp);
         r.s[1] = *reinterpret_cast<const float4*>(sp + 4);
     } else {

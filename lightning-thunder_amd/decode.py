@@ -204,9 +204,20 @@ class Llama(nn.Module):
         cfg = self.cfg
         H, Hkv, eps = cfg.n_head, cfg.n_kv_head, cfg.norm_eps
         lins = [l for blk in self.blocks for l in (blk.attn.qkv_proj, blk.attn.o_proj, blk.mlp.gate_up_proj, blk.mlp.down_proj)]
-        if not _chain_served(x.shape[0], self):
+        # The library's verdict and the operator arguments of every linear depend on (rows of x, device, what the
+        # compiled module planned for each weight) only: asked once and kept on the model, so that an eager step does not
+        # repeat a few hundred host-side queries per token.  The plan objects are part of the key (and kept alive by it):
+        # a module that is re-planned -- its override tables changed -- gets a fresh answer.
+        plans = tuple(getattr(l.weight, "_planned_operator", None) for l in lins + [self.lm_head])
+        key = (x.shape[0], x.device, tuple(id(p) for p in plans))
+        cached = self.__dict__.get("_epilogue_chain")
+        if cached is None or cached[0] != key:
+            served = _chain_served(x.shape[0], self)
+            cached = (key, plans, served, {id(l): _planned_nf4(l) for l in lins + [self.lm_head]} if served else None)
+            self.__dict__["_epilogue_chain"] = cached
+        if not cached[2]:
             return None
-        args = {id(l): _planned_nf4(l) for l in lins + [self.lm_head]}
+        args = cached[3]
         ep = Q.hip_matmul_nf4_epilogue
         r = x
         xn = ss = None

@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 from dataclasses import dataclass
 
 import torch
@@ -244,21 +245,24 @@ def reconstruct_absmax(nq: NestedAbsmax) -> torch.Tensor:
 # Nested state as plain tensors (what a state dict can hold): absmax_q uint8 [nblocks], nested_absmax fp32
 # [ceil(nblocks / nested_blocksize)], nested_quant_map fp32 [256], nested_offset fp32 [1].  The C ABI takes the
 # offset by value; reading it back from the device costs a synchronisation, so it is read once per tensor and
-# again only after the tensor was written to (torch bumps ``_version`` on every in-place write).
-_offset_cache: dict[int, tuple[int, int, float]] = {}
+# again only after the tensor was written to (torch bumps ``_version`` on every in-place write) or rebound to other
+# storage.  The value is kept ON the tensor object: it dies with it, so a new tensor that happens to get a dead one's
+# id and address (CPython reuses ids, the caching allocator reuses addresses) can never see a stale value.
+_OFFSET_ATTR = "_nf4hip_offset_value"
+
+
+def _remember_offset(nested_offset: torch.Tensor, value: float) -> None:
+    setattr(nested_offset, _OFFSET_ATTR, (nested_offset.data_ptr(), nested_offset._version, value))
 
 
 def _offset_value(nested_offset) -> float:
     if not isinstance(nested_offset, torch.Tensor):
         return float(nested_offset)
-    key = id(nested_offset)
-    hit = _offset_cache.get(key)
+    hit = getattr(nested_offset, _OFFSET_ATTR, None)
     if hit is not None and hit[0] == nested_offset.data_ptr() and hit[1] == nested_offset._version:
         return hit[2]
-    if len(_offset_cache) > 4096:
-        _offset_cache.clear()
     value = float(nested_offset.reshape(-1)[0].item())
-    _offset_cache[key] = (nested_offset.data_ptr(), nested_offset._version, value)
+    _remember_offset(nested_offset, value)
     return value
 
 
@@ -273,7 +277,7 @@ def quantize_nf4_dq(w: torch.Tensor, blocksize: int = 64, nested_blocksize: int 
     qw, absmax, code = quantize_nf4(w, blocksize)
     nq = compress_absmax(absmax, nested_blocksize)
     offset = torch.tensor([nq.offset], dtype=torch.float32, device=qw.device)
-    _offset_cache[id(offset)] = (offset.data_ptr(), offset._version, float(nq.offset))
+    _remember_offset(offset, float(nq.offset))
     return qw, nq.q, nq.absmax2, nq.map256, offset, code
 
 
@@ -314,18 +318,17 @@ def reserve_workspace(device=None, nbytes: int | None = None) -> int:
         return _workspace_pool.reserve(dev, nbytes)
 
 
+def _gemm_plan(M: int, N: int, K: int) -> tuple[int, int, int, int]:
+    """``(rows of x per tile, tiles, pieces per tile along K, workgroups)`` of the fused GEMM for this shape: the
+    library's own answer (``nf4hip_gemm_plan``), so that the time models below never restate a launcher's rules."""
+    plan = (ctypes.c_int * 4)()
+    _lib.check(_lib.load().nf4hip_gemm_plan(M, N, K, ctypes.byref(plan)))
+    return plan[0], plan[1], plan[2], plan[3]
+
+
 def _gemm_splits(M: int, N: int, K: int) -> int:
-    """K splits the fused GEMM kernel uses (gemm_splits in csrc/nf4_gemm.hip): up to 128 rows of x,
-    as many workgroups as fit the chip's 256 CUs in one round when the weight has few 256-row tiles; the
-    k steps divide evenly and every split keeps at least 4."""
-    if M > 128:
-        return 1
-    tiles, ksteps = (N + 255) // 256, K // 64
-    best = 1
-    for s in range(2, 9):
-        if tiles * s <= 256 and ksteps % s == 0 and ksteps // s >= 4:
-            best = s
-    return best
+    """K splits of the fused GEMM kernel for up to 128 rows of x (1 beyond)."""
+    return _gemm_plan(M, N, K)[2] if M <= 128 else 1
 
 
 def _fused_gemm_us(M: int, N: int, K: int) -> float:
@@ -352,18 +355,10 @@ def _dense_route_us(N: int, K: int) -> float:
 
 
 def _wide_schedule(M: int, N: int, K: int) -> tuple[int, int, int]:
-    """(rows of x per tile, tiles, pieces per tile) of the fused GEMM kernel for more than 128 rows of x; mirrors
-    gemm_wide_tile_rows and wide_schedule in csrc/nf4_gemm_wide.hip: the 256-row tile from 160 tiles on or when
-    tiles x k steps >= 28672, else the 128-row tile; a call with fewer tiles than the 256 CUs cuts every tile into
-    up to 8 equal pieces along k (at most 256 pieces in all, 16 k steps or more each) that meet in the workspace."""
-    n_tiles, ksteps = (N + 255) // 256, K // 64
-    tiles256 = ((M + 255) // 256) * n_tiles
-    bm = 256 if tiles256 >= 160 or tiles256 * ksteps >= 28672 else 128
-    tiles = ((M + bm - 1) // bm) * n_tiles
-    pieces = 1
-    if tiles < 256 and ksteps >= 32:
-        gran = 4 if ksteps % 4 == 0 else 2 if ksteps % 2 == 0 else 1
-        pieces = max(1, min(256 // tiles, 8, ksteps // 16, ksteps // gran))
+    """(rows of x per tile, tiles, pieces per tile) of the fused GEMM kernel for more than 128 rows of x: the 256-row
+    tile from 160 tiles on or when tiles x k steps >= 28672, else the 128-row tile; a call with fewer tiles than the 256
+    CUs cuts every tile into up to 8 equal pieces along k that meet in the workspace."""
+    bm, tiles, pieces, _ = _gemm_plan(M, N, K)
     return bm, tiles, pieces
 
 
@@ -438,6 +433,45 @@ def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
     return t < 0.8 * _dense_route_us(N, K)
 
 
+# Many rows of x: the fused GEMM and dequantize + dense GEMM are within a few per cent of each other over a wide range
+# of shapes, and which one leads moves with the board (clocks under a power limit, the library's GEMM heuristics).  The
+# time models above are the answer where nothing can be measured (on the CPU, under stream capture); otherwise the
+# first call of a shape on a device times both routes once -- a few launches each -- and every later call takes the
+# faster one.  NF4HIP_CALIBRATE=0 switches the measurement off.
+CALIBRATE_MIN_M = 129
+_route_measured: dict[tuple, str] = {}
+
+
+def _route_key(device: torch.device, M: int, N: int, K: int, blocksize: int, nested: bool, has_bias: bool) -> tuple:
+    index = device.index if device.index is not None else (torch.cuda.current_device() if device.type == "cuda" else -1)
+    return (device.type, index, M, N, K, blocksize, nested, has_bias)
+
+
+def _calibration_enabled() -> bool:
+    return os.environ.get("NF4HIP_CALIBRATE", "1") != "0"
+
+
+def _measure_route(key: tuple, candidates: dict, launches: int = 3) -> str:
+    """Time every candidate (a callable per route name) on the current stream: one untimed call, then ``launches``
+    calls between two events; remember and return the fastest.  A candidate within 2 % of the best that needs no
+    transient bf16 weight ("gemm") is preferred."""
+    times = {}
+    for name, fn in candidates.items():
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        e1.synchronize()
+        times[name] = e0.elapsed_time(e1)
+    best = min(times, key=times.get)
+    if "gemm" in times and times["gemm"] <= 1.02 * times[best]:
+        best = "gemm"
+    _route_measured[key] = best
+    return best
+
+
 def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape, nested: bool = False) -> str:
     """Which kernel serves this call: ``"gemv"``, ``"gemv-chunks"`` (the decode kernel once per 16
     rows of x), ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP
@@ -468,6 +502,9 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
     if K % 512 == 0 and _chunked_gemv_wins(M, N, K):
         return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
+    measured = _route_measured.get(_route_key(x.device, M, N, K, blocksize, nested, bias is not None))
+    if measured is not None:
+        return measured  # both routes were timed on this device for this shape (_measure_route)
     if _fused_gemm_wins(M, N, K, nested):
         return "gemm"  # expanding the weight tiles in registers beats writing the bf16 weight out
     # the fused GEMM kernel streams K sequentially per tile: beyond LONG_K even a few rows of x are
@@ -484,7 +521,24 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
     N, K = shape
     assert x.shape[-1] == K, f"{x.shape=}, rhs {shape=}"
     _require_gpu(x, qweight, quant_map, bias)
-    route = fused_route(x, bias, blocksize, dtype, shape, isinstance(absmax, NestedAbsmax))
+    nested = isinstance(absmax, NestedAbsmax)
+    route = fused_route(x, bias, blocksize, dtype, shape, nested)
+    M = x.numel() // K
+    if (route in ("gemm", "dequant+gemm") and M >= CALIBRATE_MIN_M and _calibration_enabled()
+            and not torch.cuda.is_current_stream_capturing()):
+        key = _route_key(x.device, M, N, K, blocksize, nested, bias is not None)
+        if key not in _route_measured:
+            with _on_device(x.device):
+                route = _measure_route(key, {
+                    "gemm": lambda: _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, "gemm"),
+                    "dequant+gemm": lambda: _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, "dequant+gemm"),
+                })
+    return _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, route)
+
+
+def _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, route: str) -> torch.Tensor:
+    """:func:`matmul_nf4` on a given route (one of ``fused_route``'s answers)."""
+    N, K = shape
     if route in ("dequant+linear", "dequant+gemm"):
         w = dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape).to(x.dtype)
         return torch.nn.functional.linear(x, w, bias)

@@ -85,6 +85,16 @@ def hip_matmul_nf4_dq_impl(x, qweight, bias, absmax_q, nested_absmax, nested_qua
                                     blocksize, nested_blocksize, dtype, shape)
 
 
+def _norm_parts(rows: int, shape) -> int:
+    """Partial sums of squares per row of x that the residual epilogue leaves for this shape on the current device (the
+    band or tile count of the serving kernel's launch plan, asked of the library); 1 where the kernels do not serve the
+    case and the operator computes the step itself."""
+    from .. import _lib
+
+    parts = _lib.load().nf4hip_gemv_norm_parts(rows, int(shape[0]), int(shape[1])) if 0 < rows <= 16 else 0
+    return parts if parts > 0 else 1
+
+
 def hip_matmul_nf4_epilogue_meta(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=None, silu_pairs=False,
                                  resid_norm=None):
     _check_matmul_shapes(x, shape)
@@ -93,15 +103,38 @@ def hip_matmul_nf4_epilogue_meta(x, qweight, bias, absmax, quant_map, blocksize,
     if resid_norm is None:
         return out
     rows = _numel(x.shape[:-1])
-    return out, TensorProxy(like=x, shape=(*x.shape[:-1], n)), _plain(x, (rows, 512), torch.float32)
+    return out, TensorProxy(like=x, shape=(*x.shape[:-1], n)), _plain(x, (rows, _norm_parts(rows, shape)), torch.float32)
 
 
 def hip_matmul_nf4_epilogue_impl(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=None, silu_pairs=False,
                                  resid_norm=None):
     """``hip_matmul_nf4`` with the decoder layer's neighbouring step done in the kernel's epilogue
-    (``functional.matmul_nf4_epilogue``); None where the kernels do not serve the case."""
-    return functional.matmul_nf4_epilogue(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=rowscale,
-                                          silu_pairs=silu_pairs, resid_norm=resid_norm)
+    (``functional.matmul_nf4_epilogue``).  Where the kernels do not serve the case (more than sixteen rows of x, nested
+    absmax, a shape outside their rules) the operator runs ``hip_matmul_nf4`` and the step by itself, with the same
+    roundings of stored tensors, so that it always returns what its meta function describes."""
+    got = functional.matmul_nf4_epilogue(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, rowscale=rowscale,
+                                         silu_pairs=silu_pairs, resid_norm=resid_norm)
+    if got is not None:
+        return got
+    N, K = (int(v) for v in shape)
+    if rowscale is not None:
+        sumsq, eps = rowscale
+        rstd = torch.rsqrt(sumsq.float().sum(-1, keepdim=True) / K + eps)
+        sums = functional.matmul_nf4(x, qweight, None, absmax, quant_map, blocksize, dtype, shape).float() * rstd.reshape(*x.shape[:-1], 1)
+        if bias is not None:
+            sums = sums + bias.float()
+        y = sums.to(x.dtype)
+    else:
+        y = functional.matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape)
+    if silu_pairs:
+        gate, up = y[..., 0::2].float(), y[..., 1::2].float()
+        return (torch.nn.functional.silu(gate).to(x.dtype).float() * up).to(x.dtype)
+    if resid_norm is not None:
+        resid, norm_weight = resid_norm
+        r = (resid.float() + y.float()).to(x.dtype)
+        xnext = (r.float() * norm_weight.float()).to(x.dtype)
+        return r, xnext, r.float().pow(2).sum(-1, keepdim=True).reshape(-1, 1)
+    return y
 
 
 def hip_quantize_nf4_impl(w, blocksize=64):

@@ -4,6 +4,10 @@ import sys
 
 import pytest
 
+# Tests name the route they mean to exercise: the one-time timing of both routes for many rows of x
+# (functional._measure_route) stays off unless a test switches it on.
+os.environ.setdefault("NF4HIP_CALIBRATE", "0")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TESTS = os.path.dirname(os.path.abspath(__file__))
 if TESTS not in sys.path:

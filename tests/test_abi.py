@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(ta):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/nf4hip.h but not exported"
     assert sorted(ta._lib.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
-    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 3
+    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 4
 
 
 def test_missing_library_fails_loudly(ta, tmp_path):
@@ -201,3 +201,39 @@ def test_epilogue_argument_errors(ta):
     assert lib.nf4hip_gemv_norm_parts(16, 16384, 4096) == 0 and lib.nf4hip_gemv_norm_parts(1, 64, 20480) == 0
     assert lib.nf4hip_gemv_norm_parts(16, 8192, 4096) == 512
     assert lib.nf4hip_gemv_norm_parts(3, 64, 4096) > 0 and lib.nf4hip_gemv_norm_parts(8, 4096, 14336) > 0
+
+
+def test_gemm_plan_is_the_launchers_and_agrees_with_the_workspace(ta):
+    """nf4hip_gemm_plan is what the host-side time models read instead of restating the launchers' rules: over a sweep of
+    shapes its answer must account for nf4hip_gemm_workspace_bytes exactly (counter region + one fp32 partial tile of
+    `rows x 256` per piece wherever tiles are cut along K, nothing otherwise), and the Python helpers must pass it on."""
+    import torch  # noqa: F401
+
+    F, L = ta.functional, ta._lib
+    lib = L.load()
+    counter_region = 65536 * 4
+    seen_cut = seen_whole = 0
+    for M in (17, 64, 65, 128, 129, 256, 512, 1000, 2048, 4096, 8192):
+        for N in (64, 1000, 1024, 4096, 6144, 14336, 28672, 128256):
+            for K in (64, 1344, 4096, 8192, 14336, 28672):
+                rows, tiles, pieces, wgs = F._gemm_plan(M, N, K)
+                n_tiles = (N + 255) // 256
+                assert rows in (64, 128, 256) and tiles == ((M + rows - 1) // rows) * n_tiles
+                assert 1 <= pieces <= 8 and wgs <= max(256, tiles)
+                need = lib.nf4hip_gemm_workspace_bytes(M, N, K)
+                if pieces == 1:
+                    assert need == 0 and wgs == tiles
+                    seen_whole += 1
+                else:
+                    cut = tiles if M <= 128 else tiles % 256  # beyond 128 rows of x only a call without a full round is cut
+                    assert wgs == (tiles - cut) + cut * pieces and (K // 64) >= pieces
+                    assert need == counter_region + cut * pieces * rows * 256 * 4
+                    seen_cut += 1
+                assert F._gemm_splits(M, N, K) == (pieces if M <= 128 else 1)
+                if M > 128:
+                    assert F._wide_schedule(M, N, K) == (rows, tiles, pieces)
+    assert seen_cut > 50 and seen_whole > 50
+    plan = (ctypes.c_int * 4)()
+    assert lib.nf4hip_gemm_plan(0, 64, 64, ctypes.byref(plan)) == L.E_SHAPE
+    assert lib.nf4hip_gemm_plan(64, 64, 100, ctypes.byref(plan)) == L.E_SHAPE
+    assert lib.nf4hip_gemm_plan(64, 64, 64, None) == L.E_NULL

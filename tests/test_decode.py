@@ -85,9 +85,13 @@ def test_quantized_decode_graph_equals_eager(D, ta, fused, batch):
 
 @pytest.mark.gpu
 def test_llama3_8b_full_size_decode(D, ta):
-    """The benchmark's model at full size: 32 layers, d = 4096, 32 / 8 heads, FFN 14336, vocab 128256, every
-    linear NF4-quantized through the transform, prompts of 512 random token ids, batch 1 and 8.  The HIP-graph
-    replay of the decode step must give the tokens of the eager loop, token for token.
+    """The benchmark's model at full size, as the benchmark builds it: 32 layers, d = 4096, 32 / 8 heads, FFN 14336,
+    vocab 128256, Q/K/V and gate/up as one linear each with gate and up rows interleaved, every linear NF4-quantized
+    through the transform, prompts of 512 random token ids, batch 1 and 8.  Both single-token steps are run: the one
+    whose tok/s the benchmark reports (``linear_epilogues``: residual add, RMSNorm and SiLU * up in the epilogues of the
+    decode kernels, five launches per layer) and the one with that work as glue kernels of their own.  For each, the
+    HIP-graph replay of the step must give the tokens of the eager loop, token for token; the two steps must give each
+    other's tokens unless the logits they disagree on are a tie within the matmul's tolerance.
 
     Logits (prefill, then one decode step on the caches the prefill wrote) are judged against the SAME model in
     fp32 -- dequantized weights, fp32 activations, plain PyTorch -- next to a plain PyTorch bf16 model on the same
@@ -98,14 +102,14 @@ def test_llama3_8b_full_size_decode(D, ta):
     """
     print("llama-3-8b full size", flush=True)
     dev = torch.device("cuda:0")
-    cfg = D.LlamaConfig.llama3_8b(fused_projections=True, hip_glue=True)
+    cfg = D.LlamaConfig.llama3_8b(fused_projections=True, gate_up_interleaved=True, hip_glue=True)
     model = D.build_llama(cfg, device=dev, seed=4000)
     jm = ta.jit(model, transforms=[ta.BitsAndBytesLinearQuant4bit()])
     n_linear = sum(1 for k in jm.state_dict() if k.endswith(".absmax"))
     assert n_linear == 32 * 4 + 1  # fused qkv, o, fused gate/up, down per layer, and the lm_head
 
     # references: same architecture and seed, weights replaced by their NF4 round trip, plain PyTorch ops
-    ref_cfg = D.LlamaConfig.llama3_8b(fused_projections=True, hip_glue=False)
+    ref_cfg = D.LlamaConfig.llama3_8b(fused_projections=True, gate_up_interleaved=True, hip_glue=False)
     ref = D.build_llama(ref_cfg, device=dev, seed=4000)
     for name, mod in ref.named_modules():
         if isinstance(mod, torch.nn.Linear):
@@ -128,23 +132,70 @@ def test_llama3_8b_full_size_decode(D, ta):
         assert rms_a <= 1.5 * rms_b + 1e-3, f"{what}: rms error {rms_a:.4f} vs PyTorch bf16 {rms_b:.4f}"
         assert max_a <= 1.5 * max_b + 1e-2, f"{what}: max error {max_a:.4f} vs PyTorch bf16 {max_b:.4f}"
 
+    def launches_of_a_step(batch):
+        """How many times the step calls the epilogue operator (counted on one eager step)."""
+        from importlib import import_module
+
+        Q = import_module("lightning-thunder_amd.transforms.quantization")
+        real, n = Q.hip_matmul_nf4_epilogue, [0]
+
+        def counting(*a, **k):
+            n[0] += 1
+            return real(*a, **k)
+
+        Q.hip_matmul_nf4_epilogue = counting
+        try:
+            kc, vc = D.new_caches(cfg, batch, dev)
+            jm(torch.zeros(batch, 1, dtype=torch.long, device=dev), torch.zeros(1, dtype=torch.long, device=dev), kc, vc)
+        finally:
+            Q.hip_matmul_nf4_epilogue = real
+        return n[0]
+
     g = torch.Generator().manual_seed(4001)
     for batch in (1, 8):
-        print(f"  batch {batch}", flush=True)
         prompt = torch.randint(0, cfg.vocab, (batch, 512), generator=g).to(dev)
-        eager, s0 = D.greedy_decode(jm, cfg, prompt, n_new=8, use_graph=False)
-        graph, s1 = D.greedy_decode(jm, cfg, prompt, n_new=8, use_graph=True)
-        assert s1["graph"] and not s0["graph"]
-        assert torch.equal(eager, graph), "graph replay and eager decode disagree"
-        assert int(eager.min()) >= 0 and int(eager.max()) < cfg.vocab
-        kc, vc = D.new_caches(cfg, batch, dev)
         kr, vr = D.new_caches(cfg, batch, dev)
         k32, v32 = D.new_caches(cfg, batch, dev, torch.float32)
         pos = torch.arange(512, device=dev)
-        a = jm(prompt, pos, kc, vc)
+        pos1 = torch.full((1,), 512, device=dev, dtype=torch.long)
         b = ref(prompt, pos, kr, vr)
         c = ref32(prompt, pos, k32, v32)
-        judge(a, b, c, f"prefill, batch {batch}")
         tok = c.argmax(-1, keepdim=True)
-        pos1 = torch.full((1,), 512, device=dev, dtype=torch.long)
-        judge(jm(tok, pos1, kc, vc), ref(tok, pos1, kr, vr), ref32(tok, pos1, k32, v32), f"decode step, batch {batch}")
+        b1, c1 = ref(tok, pos1, kr, vr), ref32(tok, pos1, k32, v32)
+        tokens, step_logits = {}, {}
+        for epilogues in (True, False):
+            cfg.linear_epilogues = epilogues
+            what = "epilogues" if epilogues else "separate glue kernels"
+            print(f"  batch {batch}, {what}", flush=True)
+            # the step under test is the one it claims to be: 4 x 32 + 1 epilogue calls, less the first QKV, or none
+            assert launches_of_a_step(batch) == (32 * 4 if epilogues else 0)
+            eager, s0 = D.greedy_decode(jm, cfg, prompt, n_new=8, use_graph=False)
+            graph, s1 = D.greedy_decode(jm, cfg, prompt, n_new=8, use_graph=True)
+            assert s1["graph"] and not s0["graph"]
+            assert torch.equal(eager, graph), f"{what}: graph replay and eager decode disagree"
+            assert int(eager.min()) >= 0 and int(eager.max()) < cfg.vocab
+            tokens[epilogues] = eager
+            kc, vc = D.new_caches(cfg, batch, dev)
+            a = jm(prompt, pos, kc, vc)
+            if epilogues:
+                judge(a, b, c, f"prefill, batch {batch}")
+            step_logits[epilogues] = jm(tok, pos1, kc, vc)
+            judge(step_logits[epilogues], b1, c1, f"decode step ({what}), batch {batch}")
+        cfg.linear_epilogues = True
+        # the two steps against each other: the same tokens, except where a sequence's two best logits are closer
+        # than the two evaluations are to each other (from there on the sequences differ and are not compared)
+        torch.testing.assert_close(step_logits[True].float(), step_logits[False].float(), rtol=3e-2, atol=3e-2)
+        for s in range(batch):
+            ta_, tb_ = tokens[True][s], tokens[False][s]
+            if torch.equal(ta_, tb_):
+                continue
+            i = int((ta_ != tb_).nonzero()[0])
+            assert i >= 1, "the first token comes from the prefill, which the two steps share"
+            # replay both variants on the common prefix and look at the logits of the two candidates
+            seq = torch.cat([prompt[s:s + 1], ta_[None, :i]], dim=1)
+            kc, vc = D.new_caches(cfg, 1, dev)
+            jm(seq[:, :-1], torch.arange(seq.shape[1] - 1, device=dev), kc, vc)
+            lg = jm(seq[:, -1:], torch.full((1,), seq.shape[1] - 1, device=dev, dtype=torch.long), kc, vc).float()[0]
+            gap = abs(float(lg[ta_[i]] - lg[tb_[i]]))
+            print(f"  batch {batch} sequence {s}: the two steps part at token {i}, logit gap {gap:.4f}", flush=True)
+            assert gap <= 6e-2, f"sequence {s}: the two steps disagree at token {i} with a logit gap of {gap:.4f}"

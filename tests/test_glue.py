@@ -116,6 +116,12 @@ def test_argmax(glue, rows, vocab):
     assert int(pos) == 42
     glue.argmax_into(xd, out)  # without the counter
     assert int(pos) == 42 and torch.equal(out.cpu(), x.float().argmax(-1))
+    # a row whose maximum is zero, -0.0 ahead of +0.0: the two are equal, the first index wins
+    z = -_randn((rows, vocab), 10, 3.0).abs() - 1.0
+    z[:, 3], z[:, vocab - 2] = -0.0, 0.0
+    zd = z.to(DEV)
+    glue.argmax_into(zd, out)
+    assert torch.equal(out.cpu(), torch.full((rows,), 3)) and torch.equal(out, zd.argmax(-1))
 
 
 def _rope_ref(x, cos, sin):  # x [..., hd] fp32, cos/sin [hd]

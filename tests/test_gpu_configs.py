@@ -70,7 +70,8 @@ class QuantizedWeight:
         L, lib = ta._lib, ta._lib.load()
         self.N, self.K = N, K
         n = N * K
-        w = _cpu_weight(N, K, seed).to(DEV)
+        w_cpu = _cpu_weight(N, K, seed)
+        w = w_cpu.to(DEV)
         self.packed_g = Guarded(n // 2)
         self.absmax_g = Guarded(n // 64 * 4)
         L.check(lib.nf4hip_quantize(w.data_ptr(), L.BF16, n, 64, self.packed_g.ptr(), self.absmax_g.ptr(),
@@ -90,6 +91,8 @@ class QuantizedWeight:
         tiles = sorted({0, (N // 256) // 2 * 256, max(N - 256, 0)})
         rows = torch.cat([torch.arange(t, min(t + 256, N)) for t in tiles] + [torch.randint(0, N, (64,), generator=g)])
         self.rows = torch.unique(rows)
+        self.w_rows = w_cpu[self.rows].clone()  # the sampled rows of the bf16 weight, for the oracle's own quantisation
+        del w_cpu
 
     def oracle_rows(self, oracle):
         """fp64 [len(rows), K] on the GPU: the sampled weight rows dequantised by the CPU oracle."""
@@ -115,6 +118,22 @@ def weights(ta):
 
     yield get
     cache.clear()
+
+
+@pytest.mark.parametrize("shape,seed", [(s, 2000 + i) for i, s in enumerate(LLAMA_8B)] + [(s, 5000 + i) for i, s in enumerate(LLAMA_70B)])
+def test_full_size_quantize_equals_the_oracle_on_sampled_rows(ta, oracle, weights, shape, seed):
+    """nf4hip_quantize ran over the whole benchmark weight; its codes and absmax of three complete 256-row tiles (first,
+    middle, last) and 64 scattered rows must be the CPU oracle's for the same bf16 rows, bit for bit (K is a multiple of
+    the blocksize, so a row's blocks depend on that row alone)."""
+    N, K = shape
+    print(f"full-size quantize vs oracle [{N},{K}]", flush=True)
+    qw = weights(N, K, seed, nested=shape in LLAMA_70B)
+    rows = qw.rows.to(DEV)
+    packed = qw.packed.view(N, K // 2)[rows].cpu()
+    absmax = qw.absmax.view(N, K // 64)[rows].cpu()
+    packed_o, absmax_o = oracle.C().quantize(qw.w_rows, 64)
+    assert torch.equal(packed.reshape(-1, 1), packed_o), "packed codes differ from the oracle's"
+    assert torch.equal(absmax.reshape(-1).view(torch.int32), absmax_o.view(torch.int32)), "absmax differs from the oracle's"
 
 
 def _check_against_oracle(out, x, qw, oracle, what):

@@ -517,3 +517,35 @@ def test_thunder_adapter_is_import_guarded():
     else:
         cls = adapter.install()
         assert cls.executor.name == adapter.EXECUTOR_NAME
+
+
+def test_nested_offset_is_remembered_per_tensor_object(ta):
+    """The double-quant offset is read from its one-element tensor once and kept ON that tensor: a tensor that is
+    written to or rebound is read again, and a new tensor never inherits a dead one's value, even when CPython hands
+    it the same id and the allocator the same address."""
+    F = ta.functional
+    t = torch.tensor([0.25])
+    assert F._offset_value(t) == 0.25
+    reads = []
+    real_item = torch.Tensor.item
+    try:
+        torch.Tensor.item = lambda self: (reads.append(1), real_item(self))[1]
+        assert F._offset_value(t) == 0.25 and not reads  # remembered: no second read
+        t.fill_(0.5)  # in-place write bumps the version
+        assert F._offset_value(t) == 0.5 and len(reads) == 1
+        t.data = torch.tensor([0.75])  # rebound to other storage
+        assert F._offset_value(t) == 0.75 and len(reads) == 2
+        # a dead tensor's id and address taken by a new one with another value
+        for _ in range(64):
+            a = torch.tensor([1.5])
+            assert F._offset_value(a) == 1.5
+            ident, ptr = id(a), a.data_ptr()
+            del a
+            b = torch.tensor([2.5])
+            same_slot = id(b) == ident and b.data_ptr() == ptr
+            assert F._offset_value(b) == 2.5
+            if same_slot:
+                break
+        assert F._offset_value(3.0) == 3.0
+    finally:
+        torch.Tensor.item = real_item

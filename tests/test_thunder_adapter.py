@@ -89,3 +89,45 @@ def test_install_on_a_stand_in_thunder(ta, fake_thunder):
     with pytest.raises(RuntimeError, match="trace rewrite failed"):
         t.transform_traces_pre_prologue("p", "c", "e", fail=True)
     assert ref.bnb_matmul_nf4 == "theirs"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 16, 512])
+def test_installed_operator_runs_the_hip_kernels(ta, oracle, fake_thunder, M):
+    """``install()`` on the stand-in ``thunder`` with the real libnf4hip.so behind it (no CPU stand-in installed): the
+    subclass's ``quantize_weight`` on a GPU tensor gives the oracle's codes and absmax bit for bit, keeps the
+    reference's device policy for CPU and meta weights (thunder/transforms/quantization.py:53-63), and the operator
+    registered on the executor (thunder/extend/__init__.py:146-198) multiplies GPU tensors within rtol = atol = 2e-2
+    of the oracle's float64 dequantize-then-matmul -- one row of x (row kernel), sixteen (tile kernel), 512 (GEMM)."""
+    print(f"thunder adapter on the HIP kernels M={M}", flush=True)
+    adapter = importlib.import_module("lightning-thunder_amd.thunder_adapter")
+    T = adapter.install()
+    ex = fake_thunder.extend.get_executor("quant_hip_nf4")
+    sym = ex.opmap["hip_matmul_nf4"]
+    assert ex is T.executor
+    N, K = 1536, 4096
+    dev = torch.device("cuda:0")
+    w = (torch.randn(N, K, generator=torch.Generator().manual_seed(11)) * 0.02).to(torch.bfloat16)
+    t = T()
+    qw, state = t.quantize_weight(w.to(dev))
+    qw_o, absmax_o = oracle.C().quantize(w, 64)
+    assert qw.is_cuda and state.absmax.is_cuda and state.code.is_cuda
+    assert torch.equal(qw.cpu(), qw_o) and torch.equal(state.absmax.cpu().view(torch.int32), absmax_o.view(torch.int32))
+    assert torch.equal(state.code.cpu(), oracle.nf4_lut()) and state.shape == (N, K) and state.dtype == torch.bfloat16
+    # a CPU weight is quantised on the GPU (the reference moves it there), a meta weight stands for zeros
+    qc, sc = t.quantize_weight(w)
+    assert qc.is_cuda and torch.equal(qc.cpu(), qw_o)
+    qz, sz = t.quantize_weight(torch.empty(N, K, dtype=torch.bfloat16, device="meta"))
+    assert qz.is_cuda and not bool(sz.absmax.any())
+
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(12 + M)).to(torch.bfloat16)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(13)) * 0.5).to(torch.bfloat16)
+    for b in (None, bias):
+        y = sym(x.to(dev), qw, None if b is None else b.to(dev), state.absmax, state.code, 64, torch.bfloat16, (N, K))
+        assert y.is_cuda and y.shape == (M, N) and y.dtype == torch.bfloat16
+        ref = oracle.matmul_4bit_f64(x, qw_o, b, absmax_o, oracle.nf4_lut(), 64, torch.bfloat16, (N, K))
+        torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
+    # leading dimensions pass through, as the meta function promises
+    y3 = sym(x.to(dev).reshape(1, M, K), qw, None, state.absmax, state.code, 64, torch.bfloat16, (N, K))
+    assert y3.shape == sym.meta(types.SimpleNamespace(shape=(1, M, K), dtype=torch.bfloat16, device="cuda"), None, None, None, None,
+                                64, torch.bfloat16, (N, K)).shape

@@ -22,7 +22,7 @@ def _case(ta, M, N, K, seed):
     return x, qw, absmax, code, bias
 
 
-def _both(ta, M, N, K, seed, with_bias):
+def _both(ta, M, N, K, seed, with_bias, check_memory=False):
     L, lib = ta._lib, ta._lib.load()
     x, qw, absmax, code, bias = _case(ta, M, N, K, seed)
     bptr = bias.data_ptr() if with_bias else None
@@ -34,9 +34,13 @@ def _both(ta, M, N, K, seed, with_bias):
     out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
     L.check(lib.nf4hip_gemv(x.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(), bptr, N, K, 64,
                             ref.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0] if check_memory else None
     L.check(lib.nf4hip_gemv_static(x.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(), bptr, N, K,
                                    64, out.data_ptr(), stream))
     torch.cuda.synchronize()
+    if check_memory:  # what the entry point exists for: the device's free memory is the same after the call
+        assert torch.cuda.mem_get_info()[0] == free_before, "nf4hip_gemv_static changed the device's free memory"
     assert not torch.isnan(ref.float()).any()
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"M={M} N={N} K={K}: static scratch differs"
     return need
@@ -57,7 +61,7 @@ PAIRS = [
 def test_static_scratch_matches_workspace_entry(ta, first, second):
     print(f"gemv_static {first} then {second}", flush=True)
     n1 = _both(ta, *first, seed=11, with_bias=False)
-    n2 = _both(ta, *second, seed=12, with_bias=True)
+    n2 = _both(ta, *second, seed=12, with_bias=True, check_memory=True)  # (the first call on a device sets the array up)
     assert max(n1, n2) > 65536 * 4, "neither call of the pair used partial sums"
 
 
@@ -70,3 +74,37 @@ def test_static_scratch_refuses_oversized_shape(ta):
     assert rc == L.E_WORKSPACE
     with pytest.raises(L.NF4HipError, match="scratch"):
         L.check(rc)
+
+
+def test_static_scratch_under_graph_capture(ta):
+    """After one eager call on the device (which resolves the array), the entry point may be recorded into a HIP graph:
+    every replay, with eager calls of other shapes on the same array in between, gives the bits of nf4hip_gemv."""
+    print("gemv_static in a graph", flush=True)
+    L, lib = ta._lib, ta._lib.load()
+    M, N, K = 16, 6144, 4096  # K split over workgroups: counters and partial sums in use
+    x, qw, absmax, code, _ = _case(ta, M, N, K, seed=21)
+    need = lib.nf4hip_gemv_workspace_bytes(M, N, K)
+    assert 65536 * 4 < need <= L.STATIC_SCRATCH_BYTES
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    ref = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    L.check(lib.nf4hip_gemv(x.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(), None, N, K, 64,
+                            ref.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    L.check(lib.nf4hip_gemv_static(x.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(), None, N, K,
+                                   64, out.data_ptr(), stream))  # warm-up: outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            L.check(lib.nf4hip_gemv_static(x.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(), None,
+                                           N, K, 64, out.data_ptr(), side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"replay {rep} differs"
+        _both(ta, 8, 4096, 14336, seed=30 + rep, with_bias=False)  # eager work on the same array between the replays

@@ -108,6 +108,14 @@ int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const f
  * streams) need different workspaces.
  */
 size_t nf4hip_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
+/*
+ * Process-wide choice among the decode kernels behind nf4hip_gemv (all give results within the same tolerance of the
+ * reference; they differ in how the weight stream reaches the matrix pipe): 1 = the kernel that stages codes and absmax
+ * through LDS wherever it applies (fp32 absmax, blocksize 64, K a multiple of 256 up to 8192), 0 = never that kernel,
+ * -1 = the library's own rule (the default; the environment variable NF4HIP_STAGE presets it).  For measurements and
+ * tests; nf4hip_gemv_workspace_bytes covers every choice.
+ */
+int nf4hip_gemv_prefer_staged(int mode);
 int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
                 const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
                 size_t workspace_bytes, void* stream);

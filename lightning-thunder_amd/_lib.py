@@ -55,6 +55,7 @@ SYMBOLS = {
     "nf4hip_dq_reconstruct": (_i32, [_vp, _vp, _vp, _f32, _i64, _i32, _vp, _vp]),
     "nf4hip_dequantize_dq": (_i32, [_vp, _vp, _vp, _vp, _f32, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
     "nf4hip_gemv_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "nf4hip_gemv_prefer_staged": (_i32, [_i32]),
     "nf4hip_gemv": (_i32, _MATMUL),
     "nf4hip_gemv_dq": (_i32, _MATMUL_DQ),
     "nf4hip_gemv_epilogue": (_i32, _MATMUL[:-1] + [ctypes.POINTER(Epilogue), _vp]),

@@ -281,6 +281,12 @@ int nf4hip_dequantize_dq(const uint8_t* packed, const uint8_t* absmax_q, const f
 }
 
 size_t nf4hip_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) { return nf4::gemv_workspace_bytes(M, N, K); }
+
+int nf4hip_gemv_prefer_staged(int mode) {
+    if (mode < -1 || mode > 1) return fail(NF4HIP_E_SHAPE, "nf4hip_gemv_prefer_staged: mode %d is not -1, 0 or 1", mode);
+    nf4::gemv_set_staged(mode);
+    return NF4HIP_OK;
+}
 size_t nf4hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return nf4::gemm_workspace_bytes(M, N, K); }
 
 int nf4hip_gemm_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]) {

@@ -69,6 +69,7 @@ constexpr size_t GEMV_COUNTER_REGION_BYTES = 65536 * 4;
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream);
+void gemv_set_staged(int mode);  // -1 the dispatcher's rule, 0 never, 1 wherever the LDS-staged decode kernel applies
 bool gemv_epilogue_possible(const MatmulArgs& a);  // does the kernel that serves (M, N, K) take a.epi?
 int gemv_norm_parts(int64_t M, int64_t N, int64_t K);  // partial sums per row of x an EPI_RESID_NORM call writes (0: not served)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);

@@ -197,4 +197,10 @@ hipError_t launch_gemv_tiles(const MatmulArgs& a, int cus, hipStream_t stream);
 bool gemv_tiles_epilogue_possible(const MatmulArgs& a);
 int gemv_tiles_norm_parts(int64_t N);
 
+// codes and absmax staged through LDS, 1 <= M <= 16, fp32 absmax, blocksize 64, K % 256 == 0 (nf4_gemv_stage.hip)
+bool gemv_stage_possible(const MatmulArgs& a);
+size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K);
+hipError_t gemv_stage_setup();
+hipError_t launch_gemv_stage(const MatmulArgs& a, int cus, hipStream_t stream);
+
 }  // namespace nf4

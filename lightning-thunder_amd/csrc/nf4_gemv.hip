@@ -6,9 +6,14 @@
 // Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive), the kernel that
 // bitsandbytes.matmul_4bit picks for a single-row x; call site
 // thunder/transforms/quantization.py:39.
+#include <stdlib.h>
+
+#include <atomic>
+
 #include "nf4_gemv.h"
 
 namespace nf4 {
+size_t gemv_workspace_bytes_unstaged(int64_t M, int64_t N, int64_t K);
 namespace {
 
 constexpr int MAX_DEVICES = 64;
@@ -27,6 +32,7 @@ hipError_t device_setup(int* cus_out) {
         if ((e = gemv_tiles_setup()) != hipSuccess) return e;
         if ((e = gemv_rows_setup()) != hipSuccess) return e;
         if ((e = gemv_quad_setup()) != hipSuccess) return e;
+        if ((e = gemv_stage_setup()) != hipSuccess) return e;
         g_num_cus[dev] = cus > 0 ? cus : 256;
     }
     *cus_out = g_num_cus[dev];
@@ -61,11 +67,42 @@ bool quad_halves_serve(int64_t M, int64_t N, int64_t K) {
     return M > 8 && N * K <= ((int64_t)1 << 24) && gemv_quad_halves_possible(N, K);
 }
 
+// Which launches go to the kernel that stages codes and absmax through LDS (nf4_gemv_stage.hip): -1 the dispatcher's
+// own rule, 0 none, 1 every launch that kernel takes.  Preset by the environment variable NF4HIP_STAGE, changed by
+// gemv_set_staged (measurements and tests).
+std::atomic<int> g_stage_mode{-2};  // -2: not read from the environment yet
+
+int stage_mode() {
+    int m = g_stage_mode.load(std::memory_order_relaxed);
+    if (m == -2) {
+        const char* v = getenv("NF4HIP_STAGE");
+        m = v ? atoi(v) : -1;
+        if (m < -1 || m > 1) m = -1;
+        g_stage_mode.store(m, std::memory_order_relaxed);
+    }
+    return m;
+}
+
+bool stage_serves(const MatmulArgs& a) {
+    const int mode = stage_mode();
+    if (mode == 0 || !gemv_stage_possible(a)) return false;
+    if (mode == 1) return true;
+    return false;
+}
+
 }  // namespace
 
 // ---- dispatch -------------------------------------------------------------------------------
 
+void gemv_set_staged(int mode) { g_stage_mode.store(mode < -1 || mode > 1 ? -1 : mode, std::memory_order_relaxed); }
+
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const size_t staged = K % 256 == 0 && K <= 8192 ? gemv_stage_workspace_bytes(M, N, K) : 0;
+    const size_t other = gemv_workspace_bytes_unstaged(M, N, K);
+    return staged > other ? staged : other;
+}
+
+size_t gemv_workspace_bytes_unstaged(int64_t M, int64_t N, int64_t K) {
     if (rows_serve(M, N, K)) return gemv_rows_workspace_bytes(M, N, K);
     if (quad_halves_serve(M, N, K)) return gemv_quad_workspace_bytes(8, N, K);
     return quad_serves(M, N, K) ? gemv_quad_workspace_bytes(M, N, K) : gemv_tiles_workspace_bytes(M, N, K);
@@ -94,6 +131,7 @@ hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     int cus = 0;
     const hipError_t e = device_setup(&cus);
     if (e != hipSuccess) return e;
+    if (stage_serves(a)) return launch_gemv_stage(a, cus, stream);
     if (rows_serve(a.M, a.N, a.K)) return launch_gemv_rows(a, cus, stream);
     if (quad_halves_serve(a.M, a.N, a.K)) return launch_gemv_quad_halves(a, cus, stream);
     return quad_serves(a.M, a.N, a.K) ? launch_gemv_quad(a, cus, stream) : launch_gemv_tiles(a, cus, stream);

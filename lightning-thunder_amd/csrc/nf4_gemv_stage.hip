@@ -1,0 +1,389 @@
+// Decode-shape fused NF4 dequant-matmul for gfx950, 1 <= M <= 16 rows of x, blocksize 64, fp32 absmax, K a multiple
+// of 256: codes AND absmax are staged through LDS by LDS-direct loads, so that every byte of the weight stream is
+// requested in whole 128-byte lines, no register holds data in flight, and the layout the MFMA wants costs nothing.
+//
+// Replaces bitsandbytes' gemv_4bit (kgemm_4bit_inference_naive) / small-batch matmul_4bit, call site
+// thunder/transforms/quantization.py:39.
+//
+// HBM-bound: 0.5 byte of codes + 1/16 byte of absmax per weight, each read exactly once.
+//
+//  * One workgroup of 16 waves per CU.  Wave w owns k slice w of the workgroup's K range: 256 consecutive k =
+//    128 bytes of codes (one cache line) and 16 bytes of absmax (four blocks) of every weight row.  Its slice of x
+//    (16 rows x 256 k) sits in 32 registers as the A operands of eight v_mfma_f32_16x16x32_bf16 for the whole kernel.
+//    A workgroup streams a contiguous range of weight rows, 16 at a time (a tile).
+//  * Codes.  buffer_load_dwordx4 ... lds: one instruction moves 8 rows x 128 bytes (eight whole lines) from HBM into
+//    a wave-private ring of five 1 KB slots (two of them feed the tile being multiplied, three are in flight).  The
+//    16-byte pieces of a line are stored XOR-swizzled by row, so that the MFMA-order reads below are conflict-free.
+//  * absmax.  The 16 rows x 16 waves x 16 bytes a tile needs are contiguous per row (256 bytes); wave r fetches row r
+//    with one 16-lane LDS-direct load two tiles ahead, into one of three 4 KB buffers, pieces XOR-swizzled by row;
+//    every wave then reads its four block scales of a row with one conflict-free ds_read_b128.
+//  * Into MFMA order for free.  Lane (n = lane & 15, g = lane >> 4) supplies the B operand of weight row n.  For
+//    block b of the slice it reads 8 bytes -- half (g & 1) of 16-byte piece 2b + (g >> 1) -- whose two dwords feed the
+//    two MFMAs of the block; the A operands were loaded from x in the same k order, so no transposes are needed, and
+//    the two MFMAs of a block cover exactly its 64 k: the block sum is scaled by absmax afterwards (4 FMAs).
+//  * Code -> bf16.  256-entry byte -> (bf16, bf16) LDS table replicated for 32 lane columns with a 256-byte stride
+//    (address = (byte << 8) | column * 4: one v_perm_b32); the unused second half of every 256-byte row holds the
+//    buffers of the cross-wave reduction.
+//  * Reduction.  The sixteen waves hold sixteen partial 16 x 16 tiles (one per k slice).  They go to LDS (double
+//    buffered, one barrier per tile); wave m then adds the sixteen partials of row m of x in a fixed order, adds the
+//    bias, rounds and stores 16 consecutive outputs.
+//  * K > 4096 is split over workgroups (each keeps its slice of x): per-(tile, m) partial sums go to the workspace
+//    through agent-scope atomics, the last wave to arrive (counter per (tile, m)) adds them in split order.
+//
+// What keeps the waits exact: every wave issues the same sequence of vector memory operations per tile (one absmax
+// load, then two code loads at the end), also where a load is not needed (rows are clamped into the workgroup's
+// range), so the hand-counted s_waitcnt vmcnt(n) below always name the same operations.
+#include "nf4_gemv.h"
+
+namespace nf4 {
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+constexpr int ST_WAVES = 16;
+constexpr int ST_THREADS = ST_WAVES * 64;
+constexpr int SLICE_K = 256;                 // k per wave
+constexpr int SLOT_BYTES = 1024;             // one LDS-direct load: 8 rows x 128 B
+constexpr int RING_SLOTS = 5;
+constexpr int TABLE_SPAN = 256 * 256;        // table rows of 256 B: first half table, second half reduction buffers
+constexpr int RING_OFF = TABLE_SPAN;
+constexpr int ABS_OFF = RING_OFF + ST_WAVES * RING_SLOTS * SLOT_BYTES;
+constexpr int ABS_BYTES = 16 * ST_WAVES * 16;  // 16 rows x 16 waves x 16 B
+constexpr int ABS_BUFS = 3;
+constexpr int ST_SMEM_BYTES = ABS_OFF + ABS_BUFS * ABS_BYTES;  // 64 + 80 + 12 = 156 KB
+constexpr int RED_BUF_BYTES = ST_WAVES * 1024;                 // per buffer: 16 waves x 64 lanes x 16 B
+static_assert(2 * RED_BUF_BYTES <= TABLE_SPAN / 2, "reduction buffers live in the table's unused half rows");
+static_assert(ST_SMEM_BYTES <= 160 * 1024, "LDS of one CU");
+
+struct StagePlan {
+    int rows_per_wg;    // weight rows of one workgroup (a multiple of 8)
+    int wgs_per_split;  // workgroups that share one K range
+    int splits;         // K ranges
+    int slices_per_split;  // 256-k slices of one K range (<= 16); the last range may hold fewer
+};
+
+// byte offset in LDS of byte `o` of the reduction buffers: the second half of the table's 256-byte rows
+__device__ __forceinline__ uint32_t red_addr(uint32_t o) { return ((o >> 7) << 8) | 0x80u | (o & 127u); }
+
+__device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
+    typedef __attribute__((address_space(3))) const uint32_t* p_t;
+    return *reinterpret_cast<p_t>((uintptr_t)addr);
+}
+__device__ __forceinline__ float lds_read_f32(uint32_t addr) {
+    typedef __attribute__((address_space(3))) const float* p_t;
+    return *reinterpret_cast<p_t>((uintptr_t)addr);
+}
+__device__ __forceinline__ uint2 lds_read_u32x2(uint32_t addr) {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) const u32x2_t* p_t;
+    const u32x2_t v = *reinterpret_cast<p_t>((uintptr_t)addr);
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ float4 lds_read_f32x4(uint32_t addr) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) const f32x4_t* p_t;
+    const f32x4_t v = *reinterpret_cast<p_t>((uintptr_t)addr);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void lds_write_f32x4(uint32_t addr, f32x4 v) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) f32x4_t* p_t;
+    const f32x4_t w = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<p_t>((uintptr_t)addr) = w;
+}
+
+// wait until at most N of this wave's vector memory operations are outstanding (they complete in order)
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// 16 bytes per active lane from a buffer straight into LDS at lds_base + lane * 16 (nontemporal)
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t byte_offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(uintptr_t)lds_base, 16, byte_offset, 0, 0, 2 /* nt */);
+}
+
+template <int MGROUPS>  // lane groups of four rows of x that carry rows < M: ceil(M / 4)
+__global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAMS, int hot_rows_per_wg, int hot_wgs_per_split,
+                                                                     int hot_splits_slices, MatmulArgs a_rest) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const MatmulArgs a = with_hot_args<false>(a_rest, NF4_HOT_NAMES);
+    const int splits = hot_splits_slices & 0xffff, slices_per_split = hot_splits_slices >> 16;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4;
+    const int M = a.M, N = a.N, K = a.K;
+    const int row_bytes = K >> 1;
+
+    // this workgroup's K range and rows
+    const int split = (int)blockIdx.x % splits;
+    const int part = (int)blockIdx.x / splits;
+    const int r0 = part * hot_rows_per_wg;
+    const int r1 = min(N, r0 + hot_rows_per_wg);
+    const int rmax = r1 - 1;                       // rows beyond the range are clamped to its last row
+    const int halves = (r1 - r0 + 7) >> 3;         // 8-row loads
+    const int tiles = (halves + 1) >> 1;
+    const int total_slices = K / SLICE_K;
+    const int slice0 = split * slices_per_split;
+    const int nslices = min(slices_per_split, total_slices - slice0);  // k slices of this range
+    const bool wave_on = wave < nslices;
+    const int slice = slice0 + (wave_on ? wave : 0);  // (a wave without a slice runs on slice 0 and contributes zeros)
+
+    const __amdgpu_buffer_rsrc_t codes_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.packed), 0, (int)(uint32_t)((int64_t)N * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t abs_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(a.absmax), 0, (int)(uint32_t)((int64_t)N * (K >> 6) * 4), 0x00020000);
+
+    // the two code-book values of this thread's table entry (entry tid >> 2): requested first, so that waiting for them
+    // later waits for nothing that is requested after them
+    const float lut_hi = a.lut16[tid >> 6], lut_lo = a.lut16[(tid >> 2) & 15];
+    asm volatile("" ::: "memory");
+
+    // ---- x: the A operands of the wave's eight MFMAs, loaded once -------------------------------------------------
+    // MFMA (b, h) of block b covers k = slice * 256 + 64 b + 16 g' + 8 h + [0, 8) over the four lane groups g'
+    bf16x8 xa[4][2];
+    {
+        const uint16_t* xrow = a.x + (int64_t)min(n, M - 1) * K + slice * SLICE_K + 16 * g;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint4 v = load16(xrow + 64 * b + 8 * h);
+                xa[b][h] = __builtin_bit_cast(bf16x8, v);
+            }
+    }
+
+    // ---- load side: lane constants ----------------------------------------------------------------------------------
+    // code loads: lane i takes row (i >> 3) of the 8-row half tile and the 16-byte piece (i & 7) ^ f(row in tile),
+    // f(n) = n >> 1 (rows 0..7: the even half tile; rows 8..15: the odd one)
+    const int lrow = lane >> 3;
+    const uint32_t cpiece_even = (uint32_t)((lane & 7) ^ (lrow >> 1)) << 4;
+    const uint32_t cpiece_odd = (uint32_t)((lane & 7) ^ (4 + (lrow >> 1))) << 4;
+    const uint32_t ccol = (uint32_t)slice * 128u;
+    const uint32_t ring = RING_OFF + wave * (RING_SLOTS * SLOT_BYTES);
+    auto load_codes = [&](int h, int slot) {  // half tile h of this workgroup into ring slot `slot`
+        const int row = min(r0 + 8 * h + lrow, rmax);
+        const uint32_t off = (uint32_t)row * (uint32_t)row_bytes + ccol + ((h & 1) ? cpiece_odd : cpiece_even);
+        dma16(codes_rsrc, ring + slot * SLOT_BYTES, off);
+    };
+    // absmax loads: wave r fetches row r of a tile, lanes 0..15 the pieces of the range's k slices; lane q stores
+    // piece q ^ r at position q (readers of slice w look at position w ^ row)
+    const uint32_t abs_row_bytes = (uint32_t)(K >> 6) * 4u;
+    const int apiece = (lane & 15) ^ wave;
+    const bool abs_lane = lane < 16 && apiece < nslices;
+    auto load_absmax = [&](int t) {
+        const int row = min(r0 + 16 * t + wave, rmax);
+        const uint32_t off = (uint32_t)row * abs_row_bytes + (uint32_t)(slice0 + apiece) * 16u;
+        if (abs_lane) dma16(abs_rsrc, ABS_OFF + (t % ABS_BUFS) * ABS_BYTES + wave * 256, off);
+    };
+
+    // ---- get the stream going: absmax of tiles 0 and 1, the first five half tiles -----------------------------------
+    load_absmax(0);
+    load_absmax(1);
+#pragma unroll
+    for (int h = 0; h < RING_SLOTS; ++h) load_codes(h, h);
+
+    // ---- byte -> (bf16, bf16) table: entry e = tid >> 2, 32 bytes per thread -----------------------------------------
+    {
+        const uint32_t vb = f32_to_bf16_bits(lut_hi) | (f32_to_bf16_bits(lut_lo) << 16);
+        const float v = __uint_as_float(vb);
+        const uint32_t dst = (uint32_t)(tid >> 2) * 256u + (uint32_t)(tid & 3) * 32u;  // (the table starts at LDS address 0)
+        lds_write_f32x4(dst, f32x4{v, v, v, v});
+        lds_write_f32x4(dst + 16, f32x4{v, v, v, v});
+    }
+    wait_vm<RING_SLOTS>();  // everything older than the five code loads: x, code book, absmax of tiles 0 and 1
+    // (x is in its registers from here on: said once, so that the loop does not carry waits for it)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) asm volatile("" ::"v"(xa[b][0]), "v"(xa[b][1]));
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+
+    // ---- read side: lane constants ------------------------------------------------------------------------------------
+    const uint32_t col4 = (uint32_t)(lane & 31) * 4u;
+    const int f = n >> 1;
+    // codes of block b: 8 bytes at piece (2b + (g >> 1)) ^ f, half (g & 1), of row n & 7 of the even / odd half tile
+    const uint32_t cread0 = ring + (uint32_t)(n & 7) * 128u + ((uint32_t)((g >> 1) ^ f) << 4) + (uint32_t)(g & 1) * 8u;
+    const uint32_t aread = ABS_OFF + (uint32_t)(n * 16 + ((wave_on ? wave : 0) ^ n)) * 16u;
+    const uint32_t red_write = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
+    const bool reducer = wave < M;  // wave m finishes row m of x
+    unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
+
+    auto tile_body = [&](int t, auto s0_tag, auto s1_tag) {
+        constexpr int S0 = decltype(s0_tag)::value, S1 = decltype(s1_tag)::value;
+        // codes of this tile have landed: the four youngest loads (half tile 2t + 2, absmax t + 1, half tiles 2t + 3,
+        // 2t + 4) may still be under way -- three in the first tile.  (A wave that stored outputs since then has those
+        // stores among its youngest operations and so waits for a load or two more than it needs.)
+        if (t == 0)
+            wait_vm<3>();
+        else
+            wait_vm<4>();
+        load_absmax(t + 2);  // into the buffer tile t - 1 used: every wave is past the barrier that ended it
+
+        const uint32_t cread = cread0 + (n < 8 ? S0 * SLOT_BYTES : S1 * SLOT_BYTES);
+        uint2 cd[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) cd[b] = lds_read_u32x2(cread ^ (uint32_t)(b << 5));
+        const float4 am4 = lds_read_f32x4(aread + (t % ABS_BUFS) * ABS_BYTES);
+        const float am[4] = {am4.x, am4.y, am4.z, am4.w};
+
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int bp = 0; bp < 4; bp += 2) {  // two blocks at a time, their MFMAs interleaved (independent accumulators)
+            f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t d0 = h ? cd[bp].y : cd[bp].x, d1 = h ? cd[bp + 1].y : cd[bp + 1].x;
+                uint32_t w0[4], w1[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t sel = 0x0c0c0400u | ((uint32_t)j << 8);
+                    w0[j] = lds_read_u32(__builtin_amdgcn_perm(d0, col4, sel));
+                    w1[j] = lds_read_u32(__builtin_amdgcn_perm(d1, col4, sel));
+                }
+                const uint4 p0 = make_uint4(w0[0], w0[1], w0[2], w0[3]), p1 = make_uint4(w1[0], w1[1], w1[2], w1[3]);
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[bp][h], __builtin_bit_cast(bf16x8, p0), c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[bp + 1][h], __builtin_bit_cast(bf16x8, p1), c1, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(c0[i], am[bp], acc[i]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(c1[i], am[bp + 1], acc[i]);
+        }
+        if (!wave_on) acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (g < MGROUPS) lds_write_f32x4(red_addr((uint32_t)(t & 1) * RED_BUF_BYTES + red_write), acc);
+
+        // the two slots are free: the next half tiles but three (all reads of the slots have returned their data)
+        load_codes(2 * t + RING_SLOTS, S0);
+        load_codes(2 * t + RING_SLOTS + 1, S1);
+
+        // absmax of tile t + 1 (requested one tile ago) has landed in every wave before anyone reads it: younger are
+        // the two code loads of the previous tile's end, this tile's absmax request and its two code loads
+        wait_vm<5>();
+        wait_lds();
+        __builtin_amdgcn_s_barrier();
+
+        // ---- wave m finishes row m of x for this tile -------------------------------------------------------------------
+        if (reducer) {
+            const int m = wave;
+            // lane (n, G = g): partial sums of waves G, G + 4, G + 8, G + 12 in that order, then the four groups
+            const uint32_t src = (uint32_t)(t & 1) * RED_BUF_BYTES + (uint32_t)(16 * (m >> 2) + n) * 16u + (uint32_t)(m & 3) * 4u;
+            float sum = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) sum += lds_read_f32(red_addr(src + (uint32_t)(g + 4 * q) * 1024u));
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            const int row = r0 + 16 * t + n;
+            if (splits == 1) {
+                if (g == 0 && row < r1) {
+                    if (a.bias) sum += bf16_bits_to_f32(a.bias[row]);
+                    a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(sum);
+                }
+            } else {
+                // K split over workgroups: this wave's 16 sums of (tile, m) meet those of the other ranges in the workspace
+                const int tile_id = (r0 >> 4) + t;  // (with K split, a workgroup's rows start at a multiple of 16)
+                if (g == 0 && row < r1)
+                    __hip_atomic_store(&partial[((int64_t)split * M + m) * N + row], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                publish_partials();
+                unsigned prev = 0;
+                if (lane == 0)
+                    prev = __hip_atomic_fetch_add(&counters[tile_id * 16 + m], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                prev = __builtin_amdgcn_readfirstlane(prev);
+                acquire_partials();
+                if (prev == (unsigned)splits - 1u) {
+                    if (g == 0 && row < r1) {
+                        float tot = 0.0f;
+                        for (int s = 0; s < splits; ++s)
+                            tot += __hip_atomic_load(&partial[((int64_t)s * M + m) * N + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (a.bias) tot += bf16_bits_to_f32(a.bias[row]);
+                        a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(tot);
+                    }
+                    if (lane == 0) __hip_atomic_store(&counters[tile_id * 16 + m], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                wait_vm<0>();  // (this path's own loads and stores were not counted above: start the counting afresh)
+            }
+        }
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>;
+    for (int t = 0; t < tiles; t += RING_SLOTS) {
+        tile_body(t, I0{}, I1{});
+        if (t + 1 < tiles) tile_body(t + 1, I2{}, I3{});
+        if (t + 2 < tiles) tile_body(t + 2, I4{}, I0{});
+        if (t + 3 < tiles) tile_body(t + 3, I1{}, I2{});
+        if (t + 4 < tiles) tile_body(t + 4, I3{}, I4{});
+    }
+    wait_vm<0>();  // loads issued past the end of the range still target this workgroup's LDS
+#endif
+}
+
+int stage_splits(int64_t K) { return (int)((K / SLICE_K + ST_WAVES - 1) / ST_WAVES); }
+
+StagePlan make_stage_plan(int64_t N, int64_t K, int cus) {
+    StagePlan p;
+    p.splits = stage_splits(K);
+    const int total = (int)(K / SLICE_K);
+    p.slices_per_split = (total + p.splits - 1) / p.splits;
+    int wgs = cus / p.splits;
+    if (wgs < 1) wgs = 1;
+    // contiguous row ranges in units of 8 rows (one load); with K split, of 16 (one (tile, m) counter per tile)
+    const int unit = p.splits > 1 ? 16 : 8;
+    int64_t rows = (N + wgs - 1) / wgs;
+    rows = (rows + unit - 1) / unit * unit;
+    p.rows_per_wg = (int)rows;
+    p.wgs_per_split = (int)((N + rows - 1) / rows);
+    return p;
+}
+
+template <int MG>
+hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
+    hipLaunchKernelGGL((gemv_stage_kernel<MG>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
+                       NF4_HOT_VALUES(a), p.rows_per_wg, p.wgs_per_split, p.splits | (p.slices_per_split << 16), a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 8192 (beyond, the bf16 code book is not
+// accurate enough), no epilogue, offsets that fit 32 bits.
+bool gemv_stage_possible(const MatmulArgs& a) {
+    if (a.nested.q || a.block_log2 != 6 || a.epi.flags != EPI_NONE) return false;
+    if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 8192) return false;
+    if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
+    const int splits = stage_splits(a.K);
+    return splits == 1 || ((int64_t)((a.N + 15) / 16) * 16 <= GEMV_COUNTER_BYTES / 4);
+}
+
+size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int s = stage_splits(K);
+    return (size_t)GEMV_COUNTER_BYTES + (s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0);
+}
+
+hipError_t gemv_stage_setup() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<1>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<2>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<3>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_stage_kernel<4>, ST_SMEM_BYTES);
+}
+
+hipError_t launch_gemv_stage(const MatmulArgs& a, int cus, hipStream_t stream) {
+    if (!gemv_stage_possible(a)) return hipErrorNotSupported;
+    const StagePlan p = make_stage_plan(a.N, a.K, cus);
+    switch ((a.M + 3) / 4) {
+        case 1: return launch_mg<1>(a, p, stream);
+        case 2: return launch_mg<2>(a, p, stream);
+        case 3: return launch_mg<3>(a, p, stream);
+        default: return launch_mg<4>(a, p, stream);
+    }
+}
+
+}  // namespace nf4

@@ -1,0 +1,94 @@
+"""The decode kernel that stages codes and absmax through LDS (csrc/nf4_gemv_stage.hip), forced through the C ABI
+(``nf4hip_gemv_prefer_staged(1)``) on shapes chosen to hit its corners, against the CPU oracle's dequantised weights
+multiplied in float64 (rtol = atol = 2e-2, the matmul's bar), with guard bands around the output and the workspace,
+and bit for bit against itself over repeated launches."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+SENTINEL = 0xA5
+GUARD = 4096
+
+
+@pytest.fixture()
+def staged(ta):
+    lib = ta._lib.load()
+    assert lib.nf4hip_gemv_prefer_staged(1) == 0
+    yield lib
+    assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+
+
+def _guarded(nbytes, fill=None):
+    raw = torch.full((GUARD + nbytes + (-nbytes) % 256 + GUARD,), SENTINEL, dtype=torch.uint8, device=DEV)
+    body = raw[GUARD:GUARD + nbytes]
+    if fill is not None:
+        body.fill_(fill)
+    return raw, body
+
+
+def _intact(raw, nbytes):
+    return bool((raw[:GUARD] == SENTINEL).all()) and bool((raw[GUARD + nbytes:] == SENTINEL).all())
+
+
+def _run(ta, lib, oracle, M, N, K, seed, bias=False, reps=1):
+    L = ta._lib
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    b = (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16) if bias else None
+    qw, absmax, code = ta.quantize_nf4(w.to(DEV))
+    xd = x.to(DEV)
+    bd = b.to(DEV) if bias else None
+    need = lib.nf4hip_gemv_workspace_bytes(M, N, K)
+    ws_raw, ws = _guarded(max(need, 256), fill=0)
+    out_raw, out = _guarded(M * N * 2)
+    stream = torch.cuda.current_stream().cuda_stream
+    results = []
+    for _ in range(reps):
+        out.fill_(0xFF)
+        L.check(lib.nf4hip_gemv(xd.data_ptr(), L.BF16, M, qw.data_ptr(), absmax.data_ptr(), code.data_ptr(),
+                                None if bd is None else bd.data_ptr(), N, K, 64, out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+        torch.cuda.synchronize()
+        results.append(out.view(torch.bfloat16).view(M, N).clone())
+    assert _intact(out_raw, M * N * 2), "bytes written outside the output"
+    assert _intact(ws_raw, max(need, 256)), "bytes written outside the workspace"
+    deq = oracle.C().dequantize(qw.cpu(), absmax.cpu(), oracle.nf4_lut(), 64, torch.bfloat16, (N, K)).double()
+    ref = x.double() @ deq.t()
+    if bias:
+        ref = ref + b.double()
+    torch.testing.assert_close(results[0].cpu().double(), ref, rtol=2e-2, atol=2e-2)
+    for r in results[1:]:
+        assert torch.equal(r.view(torch.int16), results[0].view(torch.int16)), "a repeated launch gave other bits"
+
+
+# K = 4096: sixteen slices, one K range.  N: one half tile, ragged rows (N % 8 != 0), more rows than one round of workgroups
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 8, 9, 13, 16])
+@pytest.mark.parametrize("N,K", [(8, 4096), (1000, 4096), (4096, 4096), (6152, 4096)])
+def test_staged_kernel_one_k_range(ta, oracle, staged, M, N, K):
+    print(f"staged gemv M={M} N={N} K={K}", flush=True)
+    _run(ta, staged, oracle, M, N, K, seed=M + N, bias=(N == 1000))
+
+
+# fewer than sixteen slices (waves without a slice), and K beyond 4096: two K ranges meeting in the workspace
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,K", [(520, 512), (2048, 1024), (1024, 2560), (4096, 8192), (1160, 6144), (304, 7168)])
+def test_staged_kernel_short_and_split_k(ta, oracle, staged, M, N, K):
+    print(f"staged gemv M={M} N={N} K={K}", flush=True)
+    _run(ta, staged, oracle, M, N, K, seed=3 * M + N + K, bias=(K == 6144), reps=3)
+
+
+def test_staged_kernel_many_launches_are_bit_stable(ta, oracle, staged):
+    """[4096, 8192], sixteen rows of x: K is split over two workgroups per tile, whichever arrives last adds the
+    partial sums in range order -- 200 launches on one workspace must give one result."""
+    print("staged gemv, 200 launches with K split", flush=True)
+    _run(ta, staged, oracle, 16, 4096, 8192, seed=99, reps=200)
+
+
+def test_staged_kernel_is_refused_where_it_does_not_apply(ta, oracle, staged):
+    """K not a multiple of 256, or beyond 8192: nf4hip_gemv falls back to its other kernels (same result contract)."""
+    print("staged gemv, shapes it leaves to the other kernels", flush=True)
+    _run(ta, staged, oracle, 4, 512, 4096 + 512 + 32, seed=5)
+    _run(ta, staged, oracle, 16, 512, 14336, seed=6)

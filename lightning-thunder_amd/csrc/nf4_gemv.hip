@@ -83,11 +83,21 @@ int stage_mode() {
     return m;
 }
 
+// The dispatcher's own rule, from interleaved timings of both sides (us, staged vs the other kernels, one to sixteen
+// rows of x): lm_head [128256, 4096] 47.8 / 49.7 / 53.4 / 60.2 vs 52.4 / 57.7 / 60.9 / 60.8 at M = 1 / 4 / 8 / 16;
+// [28672, 4096] 14.9 / 15.4 / 16.2 / 18.4 vs 15.5 / 15.8 / 20.4 / 23.5; [14336, 4096] 11.2 / 11.5 / 11.9 / 13.6 vs 10.2 /
+// 10.2 / 12.8 / 16.5; [6144, 4096] 8.0 / 8.3 / 8.7 / 10.1 vs 6.7 / 7.0 / 8.4 / 11.8; [4096, 4096] 6.7 / 7.1 / 7.6 / 8.4 vs
+// 5.1 / 6.3 / 7.5 / 9.3; [1024, 4096] 6.2 / 6.7 / 7.4 / 8.4 vs 4.1 / 4.5 / 5.1 / 6.5.  The staged kernel streams faster and
+// starts more slowly (a workgroup of sixteen waves, a barrier behind the table build): every weight of a hundred
+// million elements or more, from five rows of x on beyond forty million, from nine rows on beyond 2^24.
 bool stage_serves(const MatmulArgs& a) {
     const int mode = stage_mode();
     if (mode == 0 || !gemv_stage_possible(a)) return false;
     if (mode == 1) return true;
-    return false;
+    const int64_t weights = (int64_t)a.N * a.K;
+    if (weights >= 100000000) return true;
+    if (weights >= 40000000) return a.M >= 5;
+    return weights >= ((int64_t)1 << 24) && a.M >= 9;
 }
 
 }  // namespace
@@ -110,6 +120,7 @@ size_t gemv_workspace_bytes_unstaged(int64_t M, int64_t N, int64_t K) {
 
 bool gemv_epilogue_possible(const MatmulArgs& a) {
     if (a.epi.flags == EPI_NONE) return true;
+    if (stage_serves(a)) return true;
     if (rows_serve(a.M, a.N, a.K)) return gemv_rows_epilogue_possible(a);
     if (quad_halves_serve(a.M, a.N, a.K) || quad_serves(a.M, a.N, a.K)) return gemv_quad_epilogue_possible(a);
     return gemv_tiles_epilogue_possible(a);

@@ -25,14 +25,21 @@
 //    (address = (byte << 8) | column * 4: one v_perm_b32); the unused second half of every 256-byte row holds the
 //    buffers of the cross-wave reduction.
 //  * Reduction.  The sixteen waves hold sixteen partial 16 x 16 tiles (one per k slice).  They go to LDS (double
-//    buffered, one barrier per tile); wave m then adds the sixteen partials of row m of x in a fixed order, adds the
-//    bias, rounds and stores 16 consecutive outputs.
+//    buffered, one barrier per tile); wave m adds the sixteen partials of row m of x in a fixed order, adds the bias,
+//    rounds and stores 16 consecutive outputs -- one tile late: it asks for the partials of tile t - 1 at the top of
+//    tile t and adds them up at its end, so that the reads' latency hides behind the tile's own work.
 //  * K > 4096 is split over workgroups (each keeps its slice of x): per-(tile, m) partial sums go to the workspace
 //    through agent-scope atomics, the last wave to arrive (counter per (tile, m)) adds them in split order.
+//
+//  * Epilogues (K not split): wave m may scale its finished sums of row m by 1 / rms (EPI_ROWSCALE: the producer's
+//    partial sums of squares are added up once per workgroup, by wave m for its row, while the first weights are on their
+//    way) and merge (gate, up) pairs of outputs into SiLU(gate) * up (EPI_SILU_PAIRS: the odd row's lane hands its value
+//    to the even row's lane), with the roundings of the two-step route.
 //
 // What keeps the waits exact: every wave issues the same sequence of vector memory operations per tile (one absmax
 // load, then two code loads at the end), also where a load is not needed (rows are clamped into the workgroup's
 // range), so the hand-counted s_waitcnt vmcnt(n) below always name the same operations.
+#include "decode_math.h"
 #include "nf4_gemv.h"
 
 namespace nf4 {
@@ -141,6 +148,10 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     // the two code-book values of this thread's table entry (entry tid >> 2): requested first, so that waiting for them
     // later waits for nothing that is requested after them
     const float lut_hi = a.lut16[tid >> 6], lut_lo = a.lut16[(tid >> 2) & 15];
+    // EPI_ROWSCALE: wave m's share of the partial sums of squares of row m of x (at most 512: eight per lane)
+    float ssq = 0.0f;
+    if ((a.epi.flags & EPI_ROWSCALE) && wave < M)
+        for (int p = lane; p < a.epi.in_parts; p += 64) ssq += a.epi.in_sumsq[wave * a.epi.in_parts + p];
     asm volatile("" ::: "memory");
 
     // ---- x: the A operands of the wave's eight MFMAs, loaded once -------------------------------------------------
@@ -202,6 +213,13 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     wait_lds();
     __builtin_amdgcn_s_barrier();
 
+    float rstd = 1.0f;  // EPI_ROWSCALE: 1 / rms of row `wave` of the producer's residual stream
+    if (a.epi.flags & EPI_ROWSCALE) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o, 64);
+        rstd = rsqrtf(ssq / (float)K + a.epi.eps);
+    }
+
     // ---- read side: lane constants ------------------------------------------------------------------------------------
     const uint32_t col4 = (uint32_t)(lane & 31) * 4u;
     const int f = n >> 1;
@@ -213,100 +231,151 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
 
+    // splits == 1 without a bias: a finishing wave issues exactly one store per tile, which the counted waits below
+    // take into account; otherwise they assume none, which only makes them wait for a load or two more than needed
+    const bool counted_store = reducer && splits == 1 && !a.bias;
+
+    // Finishing tile t (wave m, row m of x): lane (n, G = g) reads the partial sums of waves G, G + 4, G + 8, G + 12 ...
+    struct Pending {
+        float p[4];
+    };
+    auto read_partials = [&](int t) {
+        const int m = wave;
+        const uint32_t src = (uint32_t)(t & 1) * RED_BUF_BYTES + (uint32_t)(16 * (m >> 2) + n) * 16u + (uint32_t)(m & 3) * 4u;
+        Pending pd;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) pd.p[q] = lds_read_f32(red_addr(src + (uint32_t)(g + 4 * q) * 1024u));
+        return pd;
+    };
+    // ... adds them in that order, then the four lane groups (two register swaps across the wave: no LDS round trip),
+    // and stores the 16 outputs
+    auto finish_tile = [&](int t, const Pending& pd) {
+        const int m = wave;
+        float sum = ((pd.p[0] + pd.p[1]) + pd.p[2]) + pd.p[3];
+        {
+            const uint32_t v = __float_as_uint(sum);
+            const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);  // rows 1, 3 of the first <-> rows 0, 2 of the second
+            sum = __uint_as_float(r[0]) + __uint_as_float(r[1]);               // lanes l and l ^ 16
+            const uint32_t w = __float_as_uint(sum);
+            const auto r2 = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+            sum = __uint_as_float(r2[0]) + __uint_as_float(r2[1]);             // lanes l and l ^ 32
+        }
+        const int row = r0 + 16 * t + n;
+        if (splits == 1) {
+            sum *= rstd;
+            if (a.epi.flags & EPI_SILU_PAIRS) {
+                // rows 2j, 2j + 1 = gate j, up j: the even row's lane takes the odd row's value (lane ^ 1)
+                if (a.bias && row < r1) sum += bf16_bits_to_f32(a.bias[row]);
+                const float mine = nf4x::round_bf16(sum);
+                const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine), 0xB1, 0xf, 0xf, true));
+                if (g == 0 && row < r1 && !(n & 1)) a.out[(int64_t)m * (N >> 1) + (row >> 1)] = (uint16_t)nf4x::silu_mul_bf16(mine, other);
+            } else if (g == 0 && row < r1) {
+                if (a.bias) sum += bf16_bits_to_f32(a.bias[row]);
+                a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(sum);
+            }
+        } else {
+            // K split over workgroups: this wave's 16 sums of (tile, m) meet those of the other ranges in the workspace
+            const int tile_id = (r0 >> 4) + t;  // (with K split, a workgroup's rows start at a multiple of 16)
+            if (g == 0 && row < r1)
+                __hip_atomic_store(&partial[((int64_t)split * M + m) * N + row], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            publish_partials();
+            unsigned prev = 0;
+            if (lane == 0)
+                prev = __hip_atomic_fetch_add(&counters[tile_id * 16 + m], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            prev = __builtin_amdgcn_readfirstlane(prev);
+            acquire_partials();
+            if (prev == (unsigned)splits - 1u) {
+                if (g == 0 && row < r1) {
+                    float tot = 0.0f;
+                    for (int s = 0; s < splits; ++s)
+                        tot += __hip_atomic_load(&partial[((int64_t)s * M + m) * N + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (a.bias) tot += bf16_bits_to_f32(a.bias[row]);
+                    a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(tot);
+                }
+                if (lane == 0) __hip_atomic_store(&counters[tile_id * 16 + m], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            wait_vm<0>();  // (this path's own loads and stores are not counted below: start the counting afresh)
+        }
+    };
+
+    // two blocks of the slice, their MFMAs interleaved (independent accumulators), scaled into acc
+    auto two_blocks = [&](const uint2& ca, const uint2& cb, const bf16x8 (&xa0)[2], const bf16x8 (&xa1)[2], float sa, float sb,
+                          f32x4& acc) {
+        f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t d0 = h ? ca.y : ca.x, d1 = h ? cb.y : cb.x;
+            uint32_t w0[4], w1[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t sel = 0x0c0c0400u | ((uint32_t)j << 8);
+                w0[j] = lds_read_u32(__builtin_amdgcn_perm(d0, col4, sel));
+                w1[j] = lds_read_u32(__builtin_amdgcn_perm(d1, col4, sel));
+            }
+            const uint4 p0 = make_uint4(w0[0], w0[1], w0[2], w0[3]), p1 = make_uint4(w1[0], w1[1], w1[2], w1[3]);
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa0[h], __builtin_bit_cast(bf16x8, p0), c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa1[h], __builtin_bit_cast(bf16x8, p1), c1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(c0[i], sa, acc[i]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(c1[i], sb, acc[i]);
+    };
+
     auto tile_body = [&](int t, auto s0_tag, auto s1_tag) {
         constexpr int S0 = decltype(s0_tag)::value, S1 = decltype(s1_tag)::value;
-        // codes of this tile have landed: the four youngest loads (half tile 2t + 2, absmax t + 1, half tiles 2t + 3,
-        // 2t + 4) may still be under way -- three in the first tile.  (A wave that stored outputs since then has those
-        // stores among its youngest operations and so waits for a load or two more than it needs.)
+        // Codes of this tile have landed.  A wave's vector memory operations in issue order: absmax 0, 1, half tiles
+        // 0..4, then per tile t' absmax t' + 2, half tiles 2t' + 5, 2t' + 6 and, in a finishing wave from tile 1 on, the
+        // store of tile t' - 1.  The youngest load this tile needs is half tile 2t + 1 (first code load of tile t - 2);
+        // younger are the second code load of tile t - 2 and the three loads of tile t - 1 -- four (three in tile 0) --
+        // plus the stores issued in tiles t - 2 and t - 1 (from tile 1 on).
         if (t == 0)
             wait_vm<3>();
-        else
+        else if (!counted_store || t == 1)
             wait_vm<4>();
-        load_absmax(t + 2);  // into the buffer tile t - 1 used: every wave is past the barrier that ended it
+        else if (t == 2)
+            wait_vm<5>();
+        else
+            wait_vm<6>();
 
+        // this tile's codes and scales into registers, so that their LDS slots can be refilled while the tile is multiplied
         const uint32_t cread = cread0 + (n < 8 ? S0 * SLOT_BYTES : S1 * SLOT_BYTES);
         uint2 cd[4];
 #pragma unroll
         for (int b = 0; b < 4; ++b) cd[b] = lds_read_u32x2(cread ^ (uint32_t)(b << 5));
         const float4 am4 = lds_read_f32x4(aread + (t % ABS_BUFS) * ABS_BYTES);
-        const float am[4] = {am4.x, am4.y, am4.z, am4.w};
+        // the previous tile's partial sums (all written before the barrier that ended it): requested now, added up at the
+        // end of this tile
+        Pending pd = {};
+        if (reducer && t > 0) pd = read_partials(t - 1);
 
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int bp = 0; bp < 4; bp += 2) {  // two blocks at a time, their MFMAs interleaved (independent accumulators)
-            f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t d0 = h ? cd[bp].y : cd[bp].x, d1 = h ? cd[bp + 1].y : cd[bp + 1].x;
-                uint32_t w0[4], w1[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t sel = 0x0c0c0400u | ((uint32_t)j << 8);
-                    w0[j] = lds_read_u32(__builtin_amdgcn_perm(d0, col4, sel));
-                    w1[j] = lds_read_u32(__builtin_amdgcn_perm(d1, col4, sel));
-                }
-                const uint4 p0 = make_uint4(w0[0], w0[1], w0[2], w0[3]), p1 = make_uint4(w1[0], w1[1], w1[2], w1[3]);
-                c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[bp][h], __builtin_bit_cast(bf16x8, p0), c0, 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[bp + 1][h], __builtin_bit_cast(bf16x8, p1), c1, 0, 0, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] = fmaf(c0[i], am[bp], acc[i]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] = fmaf(c1[i], am[bp + 1], acc[i]);
-        }
-        if (!wave_on) acc = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (g < MGROUPS) lds_write_f32x4(red_addr((uint32_t)(t & 1) * RED_BUF_BYTES + red_write), acc);
+        two_blocks(cd[0], cd[1], xa[0], xa[1], am4.x, am4.y, acc);
 
-        // the two slots are free: the next half tiles but three (all reads of the slots have returned their data)
+        // Everything this tile reads from its ring slots and its absmax buffer is in registers (LDS reads return in
+        // order, the scales were requested last): the slots are refilled while the second half is multiplied.  The
+        // absmax request goes into the buffer tile t - 1 used; every wave is past the barrier that ended it.
+        asm volatile("" ::"v"(cd[2].x), "v"(cd[3].y), "v"(am4.w));
+        load_absmax(t + 2);
         load_codes(2 * t + RING_SLOTS, S0);
         load_codes(2 * t + RING_SLOTS + 1, S1);
 
+        two_blocks(cd[2], cd[3], xa[2], xa[3], am4.z, am4.w, acc);
+        if (!wave_on) acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (g < MGROUPS) lds_write_f32x4(red_addr((uint32_t)(t & 1) * RED_BUF_BYTES + red_write), acc);
+        if (reducer && t > 0) finish_tile(t - 1, pd);
+
         // absmax of tile t + 1 (requested one tile ago) has landed in every wave before anyone reads it: younger are
-        // the two code loads of the previous tile's end, this tile's absmax request and its two code loads
-        wait_vm<5>();
+        // the two code loads of the previous tile, this tile's three loads, and the stores issued in the previous tile
+        // and in this one (from tile 1 on)
+        if (!counted_store || t == 0)
+            wait_vm<5>();
+        else if (t == 1)
+            wait_vm<6>();
+        else
+            wait_vm<7>();
         wait_lds();
         __builtin_amdgcn_s_barrier();
-
-        // ---- wave m finishes row m of x for this tile -------------------------------------------------------------------
-        if (reducer) {
-            const int m = wave;
-            // lane (n, G = g): partial sums of waves G, G + 4, G + 8, G + 12 in that order, then the four groups
-            const uint32_t src = (uint32_t)(t & 1) * RED_BUF_BYTES + (uint32_t)(16 * (m >> 2) + n) * 16u + (uint32_t)(m & 3) * 4u;
-            float sum = 0.0f;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) sum += lds_read_f32(red_addr(src + (uint32_t)(g + 4 * q) * 1024u));
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
-            const int row = r0 + 16 * t + n;
-            if (splits == 1) {
-                if (g == 0 && row < r1) {
-                    if (a.bias) sum += bf16_bits_to_f32(a.bias[row]);
-                    a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(sum);
-                }
-            } else {
-                // K split over workgroups: this wave's 16 sums of (tile, m) meet those of the other ranges in the workspace
-                const int tile_id = (r0 >> 4) + t;  // (with K split, a workgroup's rows start at a multiple of 16)
-                if (g == 0 && row < r1)
-                    __hip_atomic_store(&partial[((int64_t)split * M + m) * N + row], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                publish_partials();
-                unsigned prev = 0;
-                if (lane == 0)
-                    prev = __hip_atomic_fetch_add(&counters[tile_id * 16 + m], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                prev = __builtin_amdgcn_readfirstlane(prev);
-                acquire_partials();
-                if (prev == (unsigned)splits - 1u) {
-                    if (g == 0 && row < r1) {
-                        float tot = 0.0f;
-                        for (int s = 0; s < splits; ++s)
-                            tot += __hip_atomic_load(&partial[((int64_t)s * M + m) * N + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (a.bias) tot += bf16_bits_to_f32(a.bias[row]);
-                        a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(tot);
-                    }
-                    if (lane == 0) __hip_atomic_store(&counters[tile_id * 16 + m], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-                wait_vm<0>();  // (this path's own loads and stores were not counted above: start the counting afresh)
-            }
-        }
     };
 
     using I0 = std::integral_constant<int, 0>;
@@ -321,6 +390,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         if (t + 3 < tiles) tile_body(t + 3, I1{}, I2{});
         if (t + 4 < tiles) tile_body(t + 4, I3{}, I4{});
     }
+    if (reducer) finish_tile(tiles - 1, read_partials(tiles - 1));
     wait_vm<0>();  // loads issued past the end of the range still target this workgroup's LDS
 #endif
 }
@@ -353,12 +423,18 @@ hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream
 }  // namespace
 
 // What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 8192 (beyond, the bf16 code book is not
-// accurate enough), no epilogue, offsets that fit 32 bits.
+// accurate enough), offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up)
+// pairs (even N), and only while K is not split over workgroups.
 bool gemv_stage_possible(const MatmulArgs& a) {
-    if (a.nested.q || a.block_log2 != 6 || a.epi.flags != EPI_NONE) return false;
+    if (a.nested.q || a.block_log2 != 6) return false;
     if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 8192) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
+    if (a.epi.flags != EPI_NONE) {
+        if ((a.epi.flags & ~(EPI_ROWSCALE | EPI_SILU_PAIRS)) || splits != 1) return false;
+        if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > 512) return false;
+        if ((a.epi.flags & EPI_SILU_PAIRS) && a.N % 2) return false;
+    }
     return splits == 1 || ((int64_t)((a.N + 15) / 16) * 16 <= GEMV_COUNTER_BYTES / 4);
 }
 

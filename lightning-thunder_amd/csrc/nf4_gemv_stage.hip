@@ -231,10 +231,6 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
 
-    // splits == 1 without a bias: a finishing wave issues exactly one store per tile, which the counted waits below
-    // take into account; otherwise they assume none, which only makes them wait for a load or two more than needed
-    const bool counted_store = reducer && splits == 1 && !a.bias;
-
     // Finishing tile t (wave m, row m of x): lane (n, G = g) reads the partial sums of waves G, G + 4, G + 8, G + 12 ...
     struct Pending {
         float p[4];
@@ -324,19 +320,16 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
 
     auto tile_body = [&](int t, auto s0_tag, auto s1_tag) {
         constexpr int S0 = decltype(s0_tag)::value, S1 = decltype(s1_tag)::value;
-        // Codes of this tile have landed.  A wave's vector memory operations in issue order: absmax 0, 1, half tiles
-        // 0..4, then per tile t' absmax t' + 2, half tiles 2t' + 5, 2t' + 6 and, in a finishing wave from tile 1 on, the
-        // store of tile t' - 1.  The youngest load this tile needs is half tile 2t + 1 (first code load of tile t - 2);
-        // younger are the second code load of tile t - 2 and the three loads of tile t - 1 -- four (three in tile 0) --
-        // plus the stores issued in tiles t - 2 and t - 1 (from tile 1 on).
+        // Codes of this tile have landed.  A wave's LOADS in issue order: absmax 0, 1, half tiles 0..4, then per tile t'
+        // absmax t' + 2, half tiles 2t' + 5, 2t' + 6.  The youngest load this tile needs is half tile 2t + 1 (first code
+        // load of tile t - 2); younger are the second code load of tile t - 2 and the three loads of tile t - 1: four
+        // (three in tile 0).  A finishing wave's stores are counted by the same counter but may complete in any order
+        // with respect to loads: the count assumes none is outstanding, which is exact when they have completed and waits
+        // for a load or two more than needed when they have not.
         if (t == 0)
             wait_vm<3>();
-        else if (!counted_store || t == 1)
-            wait_vm<4>();
-        else if (t == 2)
-            wait_vm<5>();
         else
-            wait_vm<6>();
+            wait_vm<4>();
 
         // this tile's codes and scales into registers, so that their LDS slots can be refilled while the tile is multiplied
         const uint32_t cread = cread0 + (n < 8 ? S0 * SLOT_BYTES : S1 * SLOT_BYTES);
@@ -360,20 +353,17 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         load_codes(2 * t + RING_SLOTS, S0);
         load_codes(2 * t + RING_SLOTS + 1, S1);
 
+        // the previous tile is finished here, between the two halves, so that its chain of additions, swaps and the
+        // store runs in the shadow of the second half's table reads
+        if (reducer && t > 0) finish_tile(t - 1, pd);
+
         two_blocks(cd[2], cd[3], xa[2], xa[3], am4.z, am4.w, acc);
         if (!wave_on) acc = f32x4{0.f, 0.f, 0.f, 0.f};
         if (g < MGROUPS) lds_write_f32x4(red_addr((uint32_t)(t & 1) * RED_BUF_BYTES + red_write), acc);
-        if (reducer && t > 0) finish_tile(t - 1, pd);
 
-        // absmax of tile t + 1 (requested one tile ago) has landed in every wave before anyone reads it: younger are
-        // the two code loads of the previous tile, this tile's three loads, and the stores issued in the previous tile
-        // and in this one (from tile 1 on)
-        if (!counted_store || t == 0)
-            wait_vm<5>();
-        else if (t == 1)
-            wait_vm<6>();
-        else
-            wait_vm<7>();
+        // absmax of tile t + 1 (requested one tile ago) has landed in every wave before anyone reads it: younger loads are
+        // the two code loads of the previous tile and this tile's three
+        wait_vm<5>();
         wait_lds();
         __builtin_amdgcn_s_barrier();
     };

@@ -113,7 +113,8 @@ __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(uintptr_t)lds_base, 16, byte_offset, 0, 0, 2 /* nt */);
 }
 
-template <int MGROUPS>  // lane groups of four rows of x that carry rows < M: ceil(M / 4)
+// MGROUPS: lane groups of four rows of x that carry rows < M: ceil(M / 4).  EPI: the epilogue flags of the call.
+template <int MGROUPS, int EPI>
 __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAMS, int hot_rows_per_wg, int hot_wgs_per_split,
                                                                      int hot_splits_slices, MatmulArgs a_rest) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     const float lut_hi = a.lut16[tid >> 6], lut_lo = a.lut16[(tid >> 2) & 15];
     // EPI_ROWSCALE: wave m's share of the partial sums of squares of row m of x (at most 512: eight per lane)
     float ssq = 0.0f;
-    if ((a.epi.flags & EPI_ROWSCALE) && wave < M)
+    if ((EPI & EPI_ROWSCALE) && wave < M)
         for (int p = lane; p < a.epi.in_parts; p += 64) ssq += a.epi.in_sumsq[wave * a.epi.in_parts + p];
     asm volatile("" ::: "memory");
 
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     __builtin_amdgcn_s_barrier();
 
     float rstd = 1.0f;  // EPI_ROWSCALE: 1 / rms of row `wave` of the producer's residual stream
-    if (a.epi.flags & EPI_ROWSCALE) {
+    if (EPI & EPI_ROWSCALE) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o, 64);
         rstd = rsqrtf(ssq / (float)K + a.epi.eps);
@@ -258,8 +259,8 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         }
         const int row = r0 + 16 * t + n;
         if (splits == 1) {
-            sum *= rstd;
-            if (a.epi.flags & EPI_SILU_PAIRS) {
+            if (EPI & EPI_ROWSCALE) sum *= rstd;
+            if (EPI & EPI_SILU_PAIRS) {
                 // rows 2j, 2j + 1 = gate j, up j: the even row's lane takes the odd row's value (lane ^ 1)
                 if (a.bias && row < r1) sum += bf16_bits_to_f32(a.bias[row]);
                 const float mine = nf4x::round_bf16(sum);
@@ -403,11 +404,31 @@ StagePlan make_stage_plan(int64_t N, int64_t K, int cus) {
     return p;
 }
 
-template <int MG>
-hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
-    hipLaunchKernelGGL((gemv_stage_kernel<MG>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
+template <int MG, int EPI>
+hipError_t launch_mg_epi(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
+    hipLaunchKernelGGL((gemv_stage_kernel<MG, EPI>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
                        NF4_HOT_VALUES(a), p.rows_per_wg, p.wgs_per_split, p.splits | (p.slices_per_split << 16), a);
     return hipGetLastError();
+}
+
+template <int MG>
+hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
+    switch (a.epi.flags) {
+        case EPI_NONE: return launch_mg_epi<MG, EPI_NONE>(a, p, stream);
+        case EPI_ROWSCALE: return launch_mg_epi<MG, EPI_ROWSCALE>(a, p, stream);
+        case EPI_SILU_PAIRS: return launch_mg_epi<MG, EPI_SILU_PAIRS>(a, p, stream);
+        case EPI_ROWSCALE | EPI_SILU_PAIRS: return launch_mg_epi<MG, EPI_ROWSCALE | EPI_SILU_PAIRS>(a, p, stream);
+    }
+    return hipErrorNotSupported;
+}
+
+template <int MG>
+hipError_t allow_lds_mg() {
+    hipError_t e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_SILU_PAIRS>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    return gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE | EPI_SILU_PAIRS>, ST_SMEM_BYTES);
 }
 
 }  // namespace
@@ -435,10 +456,10 @@ size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 hipError_t gemv_stage_setup() {
     hipError_t e;
-    if ((e = gemv_allow_lds(gemv_stage_kernel<1>, ST_SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_stage_kernel<2>, ST_SMEM_BYTES)) != hipSuccess) return e;
-    if ((e = gemv_allow_lds(gemv_stage_kernel<3>, ST_SMEM_BYTES)) != hipSuccess) return e;
-    return gemv_allow_lds(gemv_stage_kernel<4>, ST_SMEM_BYTES);
+    if ((e = allow_lds_mg<1>()) != hipSuccess) return e;
+    if ((e = allow_lds_mg<2>()) != hipSuccess) return e;
+    if ((e = allow_lds_mg<3>()) != hipSuccess) return e;
+    return allow_lds_mg<4>();
 }
 
 hipError_t launch_gemv_stage(const MatmulArgs& a, int cus, hipStream_t stream) {

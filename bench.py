@@ -14,7 +14,8 @@ Prints ONE JSON line:
               HIP events recorded inside the timed region on the launch stream, against the
               8 TB/s HBM peak; config.kernels lists all three
   config.prefill = BASELINE config 3 (M in {512, 2048, 8192}) run after the timed region: TFLOP/s of the fused GEMM
-              kernel and of HIP dequantize + dense GEMM, vs the bf16 MFMA peak; which of the two the router picks
+              kernel, of HIP dequantize + the hand-written dense kernel and of HIP dequantize + the library GEMM, vs
+              the bf16 MFMA peak; which of them the router picks
   config.llama70b_double_quant = BASELINE config 5 (nested absmax, M in {1, 16, 2048}) run after the timed region
   config.decode = BASELINE config 4 (full Llama-3-8B architecture, greedy decode, batch 1 and 8)
               run after the timed region: decode tokens/s, the second half of the metric
@@ -277,18 +278,22 @@ def _cpu_seeded(torch, shape, seed, std):
 
 def prefill_section(torch, ta) -> dict:
     """BASELINE config 3, outside the timed region of the GEMV metric: the five Llama-3-8B projection shapes (and the
-    fused gate/up weight [28672, 4096]) with M in {512, 2048, 8192} rows of x.  Every case is timed on BOTH routes
-    -- the hand-written fused kernel (nf4hip_gemm: NF4 codes expanded on chip straight into MFMA operands) and
-    nf4hip_dequantize + the dense library GEMM -- and ``router`` names the one ``matmul_nf4`` picks.  TFLOP/s = 2 M N K /
-    time against the bf16 MFMA peak; HIP events bracket 10 calls (4 beyond 4 TFLOP per call) after 3 warm-up calls.
+    fused gate/up weight [28672, 4096]) with M in {512, 2048, 8192} rows of x.  Every case is timed on THREE routes
+    -- the hand-written fused kernel (nf4hip_gemm: NF4 codes expanded on chip straight into MFMA operands),
+    nf4hip_dequantize + the hand-written dense MFMA kernel (nf4hip_linear), and nf4hip_dequantize + the vendor
+    library's GEMM -- and ``router_pick`` marks the one ``matmul_nf4`` picks (it times all three on its first call of a
+    shape; the library has to win by more than 3 %).  TFLOP/s = 2 M N K / time against the bf16 MFMA peak; HIP events
+    bracket 10 calls (4 beyond 4 TFLOP per call) after 3 warm-up calls.  ``dense_kernel_alone``: nf4hip_linear and the
+    library GEMM on the already dequantized weight.
     ``rows64``: the same weights with 64 rows of x (fused kernel with K split over workgroups vs the dense route)."""
     dev = torch.device("cuda:0")
     F = ta.functional
     L, lib = ta._lib, ta._lib.load()
     code = ta.nf4_code(dev)
     sptr = torch.cuda.current_stream().cuda_stream
-    names = {"dequant+gemm": "nf4hip_dequantize + dense GEMM", "gemm": "nf4hip_gemm (fused)"}
-    rows, mid = [], []
+    names = {"dequant+gemm": "nf4hip_dequantize + nf4hip_linear", "gemm": "nf4hip_gemm (fused)",
+             "dequant+libgemm": "nf4hip_dequantize + library GEMM"}
+    rows, mid, alone = [], [], []
     shapes = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096), (28672, 4096)]
     for si, (N, K) in enumerate(shapes):
         w = _cpu_seeded(torch, (N, K), 2000 + si if si < 5 else 2900, 0.02).to(dev)  # configs 2 and 3 share their weights
@@ -307,15 +312,26 @@ def prefill_section(torch, ta) -> dict:
                                         out.data_ptr(), ws.data_ptr(), ws.numel(), sptr))
 
             def dense():
+                return F.linear_bf16(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)))
+
+            def dense_lib():
                 return torch.nn.functional.linear(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K)))
 
-            tf, td = _timed(torch, fused, reps), _timed(torch, dense, reps)
-            # the router's pick: matmul_nf4 times both routes itself on its first call of a shape on this device
+            tf, td, tl = _timed(torch, fused, reps), _timed(torch, dense, reps), _timed(torch, dense_lib, reps)
+            # the router's pick: matmul_nf4 times the routes itself on its first call of a shape on this device
             ta.matmul_nf4(x, qw, None, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K))
             router = names[F.fused_route(x, None, BLOCKSIZE, torch.bfloat16, (N, K))]
-            for route, t in ((names["gemm"], tf), (names["dequant+gemm"], td)):
+            for route, t in ((names["gemm"], tf), (names["dequant+gemm"], td), (names["dequant+libgemm"], tl)):
                 rows.append({"N": N, "K": K, "M": M, "route": route, "router_pick": route == router, "us": round(t * 1e6, 1),
                              "tflops": round(flops / t / 1e12, 1), "frac_of_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+            if M >= 2048:
+                wd = F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K))
+                ta_, tb_ = _timed(torch, lambda: F.linear_bf16(x, wd), reps), _timed(torch, lambda: torch.nn.functional.linear(x, wd), reps)
+                alone.append({"N": N, "K": K, "M": M, "nf4hip_linear_us": round(ta_ * 1e6, 1),
+                              "nf4hip_linear_frac_of_mfma_peak": round(flops / ta_ / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                              "library_us": round(tb_ * 1e6, 1),
+                              "library_frac_of_mfma_peak": round(flops / tb_ / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+                del wd
             del x, out
         # 64 rows of x (between the decode and the prefill regime): the router's choice, which is the fused
         # kernel with K split over workgroups, next to the dense route (dequantize + library GEMM) forced
@@ -325,7 +341,7 @@ def prefill_section(torch, ta) -> dict:
         td = _timed(torch, lambda: torch.nn.functional.linear(x, F.dequantize_nf4(qw, absmax, code, BLOCKSIZE, torch.bfloat16, (N, K))), 20)
         mid.append({"N": N, "K": K, "M": 64, "route": route, "us": round(t * 1e6, 1), "dense_route_us": round(td * 1e6, 1)})
         del qw, absmax
-    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows, "rows64": mid}
+    return {"peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": rows, "dense_kernel_alone": alone, "rows64": mid}
 
 
 def double_quant_section(torch, ta) -> dict:

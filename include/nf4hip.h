@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define NF4HIP_ABI_VERSION 4
+#define NF4HIP_ABI_VERSION 5
 
 #define NF4HIP_BF16 0
 #define NF4HIP_F16 1
@@ -216,6 +216,21 @@ int nf4hip_gemm_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]);
 int nf4hip_gemm(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
                 const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
                 size_t workspace_bytes, void* stream);
+/*
+ * Dense linear on a dequantized weight: out[M, N] = x[M, K] . w[N, K]^T (+ bias), bf16 operands, fp32 accumulation,
+ * bf16 output.  The GEMM of the dequantize_4bit + torch.nn.functional.linear route of bitsandbytes.matmul_4bit
+ * (MatMul4Bit.forward, the route thunder/transforms/quantization.py:39 reaches for more than one row of x): w is
+ * what nf4hip_dequantize / nf4hip_dequantize_dq wrote.  K must be a multiple of 64 and at least 128 (NF4HIP_E_SHAPE
+ * otherwise: the caller then keeps its own dense GEMM); M and N are free.  Calls with at most 128 tiles of 256 x 256
+ * outputs and K >= 2048 cut every tile in two along K and need nf4hip_linear_workspace_bytes(M, N, K) bytes of
+ * workspace whose first 256 KiB are zero before the first call (every call leaves them zero); the result is
+ * deterministic.  nf4hip_linear_plan: plan[0] rows of x per tile (256), plan[1] tiles, plan[2] pieces per tile,
+ * plan[3] workgroups launched (no GPU needed).
+ */
+size_t nf4hip_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int nf4hip_linear_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]);
+int nf4hip_linear(const void* x, int x_dtype, int64_t M, const void* w, const void* bias_or_null, int64_t N, int64_t K,
+                  void* out, void* workspace, size_t workspace_bytes, void* stream);
 int nf4hip_gemm_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,
                    const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
                    const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,

@@ -11,7 +11,7 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 BF16, F16, F32 = 0, 1, 2
 
@@ -66,6 +66,9 @@ SYMBOLS = {
     "nf4hip_gemm_plan": (_i32, [_i64, _i64, _i64, ctypes.POINTER(_i32 * 4)]),
     "nf4hip_gemm": (_i32, _MATMUL),
     "nf4hip_gemm_dq": (_i32, _MATMUL_DQ),
+    "nf4hip_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "nf4hip_linear_plan": (_i32, [_i64, _i64, _i64, ctypes.POINTER(_i32 * 4)]),
+    "nf4hip_linear": (_i32, [_vp, _i32, _i64, _vp, _vp, _i64, _i64, _vp, _vp, _sz, _vp]),
 }
 
 

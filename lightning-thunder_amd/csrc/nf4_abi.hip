@@ -364,6 +364,54 @@ int nf4hip_gemm(const void* x, int x_dtype, int64_t M, const uint8_t* packed, co
                          workspace, workspace_bytes, stream);
 }
 
+size_t nf4hip_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || !nf4::gemm_dense_possible(M, N, K)) return 0;
+    return nf4::gemm_dense_workspace_bytes(M, N, K);
+}
+
+int nf4hip_linear_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]) {
+    if (!plan) return fail(NF4HIP_E_NULL, "nf4hip_linear_plan: plan is null");
+    if (M <= 0 || N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX || M > INT32_MAX || !nf4::gemm_dense_possible(M, N, K))
+        return fail(NF4HIP_E_SHAPE, "nf4hip_linear_plan: M, N, K must be positive and K a multiple of 64, at least 128");
+    int p[4];
+    nf4::gemm_dense_plan(M, N, K, p);
+    for (int i = 0; i < 4; ++i) plan[i] = p[i];
+    return NF4HIP_OK;
+}
+
+int nf4hip_linear(const void* x, int x_dtype, int64_t M, const void* w, const void* bias_or_null, int64_t N, int64_t K,
+                  void* out, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* name = "nf4hip_linear";
+    if (!x || !w || !out) return fail(NF4HIP_E_NULL, "%s: null pointer", name);
+    if (x_dtype != NF4HIP_BF16) return fail(NF4HIP_E_DTYPE, "%s: only bf16 operands (got dtype %d)", name, x_dtype);
+    if (M <= 0 || N <= 0 || K <= 0) return fail(NF4HIP_E_SHAPE, "%s: M, N, K must be positive", name);
+    if (N > INT32_MAX || K > INT32_MAX || M > INT32_MAX) return fail(NF4HIP_E_SHAPE, "%s: dimension too large", name);
+    if (!nf4::gemm_dense_possible(M, N, K))
+        return fail(NF4HIP_E_SHAPE, "%s: K = %lld must be a multiple of 64, at least 128", name, (long long)K);
+    if (!aligned16(x) || !aligned16(w) || !aligned16(out) || (bias_or_null && (reinterpret_cast<uintptr_t>(bias_or_null) & 1u)))
+        return fail(NF4HIP_E_ALIGN, "%s: x / w / out not 16-byte aligned or bias not 2-byte aligned", name);
+    const size_t need = nf4::gemm_dense_workspace_bytes(M, N, K);
+    if (need) {
+        if (!workspace || workspace_bytes < need)
+            return fail(NF4HIP_E_WORKSPACE, "%s: workspace of %zu bytes required, got %zu", name, need,
+                        workspace ? workspace_bytes : (size_t)0);
+        if (!aligned16(workspace)) return fail(NF4HIP_E_ALIGN, "%s: workspace not 16-byte aligned", name);
+    }
+    nf4::DenseArgs a;
+    a.x = static_cast<const uint16_t*>(x);
+    a.w = static_cast<const uint16_t*>(w);
+    a.bias = static_cast<const uint16_t*>(bias_or_null);
+    a.out = static_cast<uint16_t*>(out);
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.workspace = need ? workspace : nullptr;
+    a.workspace_bytes = need ? workspace_bytes : 0;
+    const hipError_t e = nf4::launch_gemm_dense(a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(name, e);
+    return NF4HIP_OK;
+}
+
 int nf4hip_gemm_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const uint8_t* absmax_q,
                    const float* absmax2, const float* map256, float offset, int nested_blocksize, const float* lut16,
                    const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,

@@ -53,6 +53,17 @@ struct MatmulArgs {
     Epilogue epi;
 };
 
+// Dense bf16 GEMM out[M, N] = x[M, K] . w[N, K]^T (+ bias): the GEMM of the dequantize + linear route.
+struct DenseArgs {
+    const uint16_t* x;     // [M, K] bf16
+    const uint16_t* w;     // [N, K] bf16 (what nf4hip_dequantize wrote)
+    const uint16_t* bias;  // [N] bf16 or NULL
+    uint16_t* out;         // [M, N] bf16
+    int M, N, K;
+    void* workspace;
+    size_t workspace_bytes;
+};
+
 // Launchers (defined next to their kernels).  They assume validated arguments and return the
 // hipError_t of the launch.
 hipError_t launch_quantize(const void* w, int w_dtype, int64_t n, int block_log2, uint8_t* packed, float* absmax,
@@ -83,6 +94,11 @@ size_t gemm_wide_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // plan[3] workgroups launched.
 void gemm_wide_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
 void gemm_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
+// dense bf16 GEMM (nf4_gemm_dense.hip): K a multiple of 64, at least 128
+bool gemm_dense_possible(int64_t M, int64_t N, int64_t K);
+size_t gemm_dense_workspace_bytes(int64_t M, int64_t N, int64_t K);
+void gemm_dense_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
+hipError_t launch_gemm_dense(const DenseArgs& a, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // device helpers

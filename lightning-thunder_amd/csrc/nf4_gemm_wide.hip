@@ -237,12 +237,14 @@ void gemm_wide_kernel(MatmulArgs a, WideSchedule sch) {
         const int row = min(m0 + 8 * c + rr, a.M - 1);
         xoff[j] = (uint32_t)row * (uint32_t)(a.K * 2) + (uint32_t)(((lane & 7) ^ rr) << 4) + (uint32_t)(kfirst * (BK * 2));
     }
-    auto load_x = [&](int kt, int stage) {  // k step kt into a stage
+    auto load_x_one = [&](int kt, int stage, int j) {  // load j of k step kt into a stage
         const uint32_t st = stage0 + stage * T::STAGE_BYTES + T::XL * wave * CHUNK_BYTES;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_void_ptr)(uintptr_t)(st + j * CHUNK_BYTES), 16, xoff[j],
+                                                 kt * (BK * 2), 0, 0);
+    };
+    auto load_x = [&](int kt, int stage) {  // k step kt into a stage
 #pragma unroll
-        for (int j = 0; j < T::XL; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_void_ptr)(uintptr_t)(st + j * CHUNK_BYTES), 16, xoff[j],
-                                                     kt * (BK * 2), 0, 0);
+        for (int j = 0; j < T::XL; ++j) load_x_one(kt, stage, j);
     };
     // fragment of x tile i, slice s: row r = 32 i + l % 32 lies in chunk 4 i + (l % 32) / 8 (whose parity is that of
     // (l % 32) / 8) at slot (r % 8) ^ parity; its piece 4 (l / 32) + s sits at position piece ^ (r % 8).
@@ -317,7 +319,6 @@ void gemm_wide_kernel(MatmulArgs a, WideSchedule sch) {
                     for (int g = 0; g < NG; ++g) asm volatile("" ::"v"(nxt[g].w.x), "v"(nxt[g].scale));
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (more3) load_x(kt + 3, ST);
                 __builtin_amdgcn_sched_barrier(0);
             }
             Expansion ex[NG];
@@ -347,6 +348,12 @@ void gemm_wide_kernel(MatmulArgs a, WideSchedule sch) {
                 micro_steps(true);
                 __builtin_amdgcn_sched_barrier(0);
                 if (g == NG - 1 && expand) fa[i] = lds_frag(next_frag + i * 4 * CHUNK_BYTES);
+                // the refill of this stage, one load behind every SPREAD-th MFMA of the last slice: issued together they
+                // would queue up in the CU's one address unit and hold the waves (and their MFMAs) at the issue
+                if (s == 3 && more3) {
+                    constexpr int SPREAD = T::NM / T::XL;
+                    if (j % SPREAD == 0 && j / SPREAD < T::XL) load_x_one(kt + 3, ST, j / SPREAD);
+                }
                 micro_steps(false);
                 __builtin_amdgcn_sched_barrier(0);
             }

@@ -451,10 +451,18 @@ def _calibration_enabled() -> bool:
     return os.environ.get("NF4HIP_CALIBRATE", "1") != "0"
 
 
+def _library_gemm_allowed() -> bool:
+    """Is dequantize + the vendor library's GEMM ("dequant+libgemm") one of the routes that are timed against each
+    other?  Yes unless NF4HIP_LIBRARY_GEMM=0, which keeps every fused-eligible call on this package's own kernels.  It
+    is only ever chosen by measurement, and only when it beats both hand-written routes by more than 3 %."""
+    return os.environ.get("NF4HIP_LIBRARY_GEMM", "1") != "0"
+
+
 def _measure_route(key: tuple, candidates: dict, launches: int = 3) -> str:
     """Time every candidate (a callable per route name) on the current stream: one untimed call, then ``launches``
-    calls between two events; remember and return the fastest.  A candidate within 2 % of the best that needs no
-    transient bf16 weight ("gemm") is preferred."""
+    calls between two events; remember and return the fastest.  The vendor library's GEMM ("dequant+libgemm") has to
+    beat the best hand-written route by more than 3 %; a candidate within 2 % of the best that needs no transient
+    bf16 weight ("gemm") is preferred."""
     times = {}
     for name, fn in candidates.items():
         fn()
@@ -466,6 +474,9 @@ def _measure_route(key: tuple, candidates: dict, launches: int = 3) -> str:
         e1.synchronize()
         times[name] = e0.elapsed_time(e1)
     best = min(times, key=times.get)
+    own = {name: t for name, t in times.items() if name != "dequant+libgemm"}
+    if best == "dequant+libgemm" and own and min(own.values()) <= 1.03 * times[best]:
+        best = min(own, key=own.get)
     if "gemm" in times and times["gemm"] <= 1.02 * times[best]:
         best = "gemm"
     _route_measured[key] = best
@@ -474,9 +485,10 @@ def _measure_route(key: tuple, candidates: dict, launches: int = 3) -> str:
 
 def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape, nested: bool = False) -> str:
     """Which kernel serves this call: ``"gemv"``, ``"gemv-chunks"`` (the decode kernel once per 16
-    rows of x), ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP
-    dequantize, then the dense library GEMM, because that is the faster of the two for many rows
-    of x) or ``"dequant+linear"`` (the same two steps, for dtypes and shapes no fused kernel takes).
+    rows of x), ``"gemm"`` (fused), ``"dequant+gemm"`` (HIP dequantize, then the hand-written dense MFMA kernel
+    ``nf4hip_linear``, because that is the faster of the two for many rows of x), ``"dequant+libgemm"`` (HIP
+    dequantize, then the vendor library's GEMM; only when NF4HIP_LIBRARY_GEMM=1 and measured faster) or
+    ``"dequant+linear"`` (dequantize + ``torch.nn.functional.linear``, for dtypes and shapes no kernel here takes).
 
     Mirrors bitsandbytes.matmul_4bit: the fused single-row kernel when the shape allows, else
     dequantize followed by a dense matmul.
@@ -529,9 +541,10 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
         key = _route_key(x.device, M, N, K, blocksize, nested, bias is not None)
         if key not in _route_measured:
             with _on_device(x.device):
+                names = ["gemm", "dequant+gemm"] + (["dequant+libgemm"] if _library_gemm_allowed() else [])
                 route = _measure_route(key, {
-                    "gemm": lambda: _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, "gemm"),
-                    "dequant+gemm": lambda: _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, "dequant+gemm"),
+                    name: (lambda name=name: _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, name))
+                    for name in names
                 })
     return _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, route)
 
@@ -539,8 +552,10 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
 def _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, route: str) -> torch.Tensor:
     """:func:`matmul_nf4` on a given route (one of ``fused_route``'s answers)."""
     N, K = shape
-    if route in ("dequant+linear", "dequant+gemm"):
+    if route in ("dequant+linear", "dequant+gemm", "dequant+libgemm"):
         w = dequantize_nf4(qweight, absmax, quant_map, blocksize, dtype, shape).to(x.dtype)
+        if route == "dequant+gemm":
+            return linear_bf16(x, w, bias)  # the hand-written dense kernel
         return torch.nn.functional.linear(x, w, bias)
 
     lib = _lib.load()
@@ -584,6 +599,38 @@ def _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape,
                 mc = min(step, M - m0)
                 _lib.check(fn(x2.data_ptr() + 2 * m0 * K, _lib.BF16, mc, qweight.data_ptr(), absmax.data_ptr(), quant_map.data_ptr(), bptr,
                               N, K, blocksize, out.data_ptr() + 2 * m0 * N, ws_ptr, ws_bytes, stream))  # fmt: skip
+    return out.reshape(*x.shape[:-1], N)
+
+
+def linear_possible(x: torch.Tensor, w: torch.Tensor, bias=None) -> bool:
+    """Does ``linear_bf16`` take these operands (bf16, K a multiple of 64 and at least 128)?"""
+    K = w.shape[-1]
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and (bias is None or bias.dtype == torch.bfloat16)
+            and w.dim() == 2 and x.shape[-1] == K and K % 64 == 0 and K >= 128 and x.numel() > 0 and w.numel() > 0)
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias=None) -> torch.Tensor:
+    """``torch.nn.functional.linear(x, w, bias)`` for bf16 operands on the hand-written dense MFMA kernel
+    (``nf4hip_linear``): the GEMM that follows ``dequantize_nf4`` on the dequantize + linear route of
+    bitsandbytes.matmul_4bit (MatMul4Bit.forward, reached from thunder/transforms/quantization.py:39).  ``w`` is [N, K]."""
+    if not linear_possible(x, w, bias):
+        raise ValueError(f"linear_bf16: bf16 operands with K a multiple of 64 (>= 128) only, got x {tuple(x.shape)} {x.dtype}, "
+                         f"w {tuple(w.shape)} {w.dtype}")
+    _require_gpu(x, w, bias)
+    lib = _lib.load()
+    N, K = w.shape
+    x2 = _aligned(x.reshape(-1, K))
+    w = _aligned(w)
+    M = x2.shape[0]
+    b = None if bias is None else bias.contiguous()
+    with _on_device(x.device):
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        stream = _stream()
+        need = lib.nf4hip_linear_workspace_bytes(M, N, K)
+        ws = _gemv_workspace(x.device, need, stream) if need else None
+        ws_ptr, ws_bytes = (None, 0) if ws is None else (ws.data_ptr(), ws.numel())
+        _lib.check(lib.nf4hip_linear(x2.data_ptr(), _lib.BF16, M, w.data_ptr(), None if b is None else b.data_ptr(), N, K,
+                                     out.data_ptr(), ws_ptr, ws_bytes, stream))
     return out.reshape(*x.shape[:-1], N)
 
 

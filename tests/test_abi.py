@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(ta):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/nf4hip.h but not exported"
     assert sorted(ta._lib.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
-    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 4
+    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 5
 
 
 def test_missing_library_fails_loudly(ta, tmp_path):
@@ -33,6 +33,35 @@ def test_missing_library_fails_loudly(ta, tmp_path):
 
 def _err(ta):
     return ta._lib.load().nf4hip_last_error().decode()
+
+
+def test_linear_argument_errors_and_plan(ta):
+    """nf4hip_linear validates before its first HIP call; its plan and workspace queries need no GPU."""
+    import ctypes
+
+    L, lib = ta._lib, ta._lib.load()
+    A = 4096
+    assert lib.nf4hip_linear(None, L.BF16, 4, A, None, 8, 128, A, None, 0, None) == L.E_NULL
+    assert lib.nf4hip_linear(A, L.F16, 4, A, None, 8, 128, A, None, 0, None) == L.E_DTYPE
+    assert lib.nf4hip_linear(A, L.BF16, 0, A, None, 8, 128, A, None, 0, None) == L.E_SHAPE
+    assert lib.nf4hip_linear(A, L.BF16, 4, A, None, 8, 96, A, None, 0, None) == L.E_SHAPE and "64" in _err(ta)
+    assert lib.nf4hip_linear(A, L.BF16, 4, A, None, 8, 64, A, None, 0, None) == L.E_SHAPE  # one k step: not served
+    assert lib.nf4hip_linear(A + 2, L.BF16, 4, A, None, 8, 128, A, None, 0, None) == L.E_ALIGN
+    assert lib.nf4hip_linear(A, L.BF16, 4, A, A + 1, 8, 128, A, None, 0, None) == L.E_ALIGN
+    # [4096, 14336] with 2048 rows of x: 128 tiles cut in two along K -> two partial tiles each and the counter region
+    need = lib.nf4hip_linear_workspace_bytes(2048, 4096, 14336)
+    assert need == 65536 * 4 + 128 * 2 * 256 * 256 * 4
+    assert lib.nf4hip_linear(A, L.BF16, 2048, A, None, 4096, 14336, A, None, 0, None) == L.E_WORKSPACE
+    assert lib.nf4hip_linear(A, L.BF16, 2048, A, None, 4096, 14336, A, A, need - 1, None) == L.E_WORKSPACE
+    assert lib.nf4hip_linear_workspace_bytes(2048, 14336, 4096) == 0  # 448 tiles: taken whole
+    assert lib.nf4hip_linear_workspace_bytes(2048, 4096, 1024) == 0  # too few k steps to cut
+    assert lib.nf4hip_linear_workspace_bytes(4, 8, 96) == 0
+    plan = (ctypes.c_int * 4)()
+    assert lib.nf4hip_linear_plan(2048, 4096, 14336, ctypes.byref(plan)) == 0 and list(plan) == [256, 128, 2, 256]
+    assert lib.nf4hip_linear_plan(2048, 14336, 4096, ctypes.byref(plan)) == 0 and list(plan) == [256, 448, 1, 448]
+    assert lib.nf4hip_linear_plan(300, 520, 192, ctypes.byref(plan)) == 0 and list(plan) == [256, 6, 1, 6]
+    assert lib.nf4hip_linear_plan(2048, 4096, 96, ctypes.byref(plan)) == L.E_SHAPE
+    assert lib.nf4hip_linear_plan(2048, 4096, 128, None) == L.E_NULL
 
 
 A = 4096  # any non-null, 16-byte aligned fake device address: validation never dereferences

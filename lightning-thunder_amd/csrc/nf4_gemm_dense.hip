@@ -144,8 +144,8 @@ void gemm_dense_kernel(DenseArgs a, DenseSchedule sch) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) load_one(0, 0, j);
 #pragma unroll
-    for (int j = 0; j < 16; ++j) load_one(1, 1, j);  // every piece has two steps or more (the launcher checks)
-    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+    for (int j = 0; j < 8; ++j) load_one(1, 1, j);  // x of step 1 (every piece has two steps or more); w follows in step 0
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
 
     bf16x8 fa[2][4], fb[2][4];
 #pragma unroll
@@ -186,7 +186,7 @@ void gemm_dense_kernel(DenseArgs a, DenseSchedule sch) {
                 }
                 if ((j & 1) == 0) {
                     if (s == 3 && more2) load_one(kt + 2, ST, j >> 1);
-                    if (s == 0 && kt > 0 && more) load_one(kt + 1, ST ^ 1, 8 + (j >> 1));
+                    if (s == 0 && more) load_one(kt + 1, ST ^ 1, 8 + (j >> 1));
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }

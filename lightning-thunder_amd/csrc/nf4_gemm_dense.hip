@@ -57,6 +57,7 @@ __device__ __forceinline__ bf16x8 lds_frag(uint32_t addr) {
 // Tile number -> (x-row tile, weight-row tile), inside the kernel: workgroups are handed out to the XCDs in turn and
 // every XCD gets a contiguous run of tile numbers; numbers run through GROUP_M x-row tiles first, then through the
 // weight-row tiles, so the 32 tiles an XCD works on at a time share eight tiles of x and four of w in its L2.
+template <bool TWO_PIECES>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm_dense_kernel(DenseArgs a, DenseSchedule sch) {
     // The body exists in the device pass only: the host pass cannot instantiate the buffer-resource type.
@@ -68,7 +69,8 @@ void gemm_dense_kernel(DenseArgs a, DenseSchedule sch) {
     const int wm = wave >> 1, wn = wave & 1;
 
     // ---- what this workgroup works on ----
-    const int total = sch.tiles * sch.pieces;
+    constexpr int PIECES = TWO_PIECES ? 2 : 1;
+    const int total = sch.tiles * PIECES;
     int u = blockIdx.x;
     {
         const int full = total & ~7;
@@ -88,8 +90,8 @@ void gemm_dense_kernel(DenseArgs a, DenseSchedule sch) {
     }
     const int m0 = mt * BM, n0 = nt * BN;
     const int ksteps_all = a.K / BK;
-    const int kfirst = piece * ksteps_all / sch.pieces;
-    const int ksteps = (piece + 1) * ksteps_all / sch.pieces - kfirst;
+    const int kfirst = piece * ksteps_all / PIECES;
+    const int ksteps = (piece + 1) * ksteps_all / PIECES - kfirst;
 
     // Buffer resources that start at the tile's first row: offsets inside a tile fit 32 bits whatever the tensor's size.
     const uint32_t row_bytes = (uint32_t)a.K * 2u;
@@ -212,7 +214,7 @@ void gemm_dense_kernel(DenseArgs a, DenseSchedule sch) {
     // the other partial to its registers and writes the tile.  Either way the tile is a + b with the two halves'
     // fp32 sums as a and b, so the result does not depend on who arrives when; nobody waits for anybody.
     bool write_tile = true;
-    if (sch.pieces == 2) {
+    if (TWO_PIECES) {
         uint32_t* cP = sch.counters + 2 * tile;
         uint32_t* cT = cP + 1;
         float* mine = sch.partials + (int64_t)(2 * tile + piece) * SLOT_FLOATS;
@@ -357,7 +359,10 @@ hipError_t launch_gemm_dense(const DenseArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
     if (!ready[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dense_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dense_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                SMEM_BYTES);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dense_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 SMEM_BYTES);
         if (e != hipSuccess) return e;
         ready[dev] = true;
@@ -366,7 +371,10 @@ hipError_t launch_gemm_dense(const DenseArgs& a, hipStream_t stream) {
     if (sch.tiles * 2 > (int)(GEMV_COUNTER_BYTES / sizeof(uint32_t))) sch.pieces = 1;
     sch.counters = static_cast<uint32_t*>(a.workspace);
     sch.partials = a.workspace ? reinterpret_cast<float*>(static_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES) : nullptr;
-    hipLaunchKernelGGL(gemm_dense_kernel, dim3((unsigned)(sch.tiles * sch.pieces)), dim3(THREADS), SMEM_BYTES, stream, a, sch);
+    if (sch.pieces == 2)
+        hipLaunchKernelGGL(gemm_dense_kernel<true>, dim3((unsigned)(sch.tiles * 2)), dim3(THREADS), SMEM_BYTES, stream, a, sch);
+    else
+        hipLaunchKernelGGL(gemm_dense_kernel<false>, dim3((unsigned)sch.tiles), dim3(THREADS), SMEM_BYTES, stream, a, sch);
     return hipGetLastError();
 }
 

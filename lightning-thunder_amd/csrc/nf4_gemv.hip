@@ -94,6 +94,10 @@ bool stage_serves(const MatmulArgs& a) {
     const int mode = stage_mode();
     if (mode == 0 || !gemv_stage_possible(a)) return false;
     if (mode == 1) return true;
+    // K beyond what the sixteen waves of a workgroup cover (4096) is split over workgroups, and that hand-off drains the
+    // stream once per tile: [28672, 8192] takes 44 / 47 / 56 us there with one / four / sixteen rows of x against 26 / 26 / 46
+    // in the other kernels.
+    if (gemv_stage_splits(a.K) > 1) return false;
     const int64_t weights = (int64_t)a.N * a.K;
     if (weights >= 100000000) return true;
     if (weights >= 40000000) return a.M >= 5;

@@ -449,6 +449,8 @@ bool gemv_stage_possible(const MatmulArgs& a) {
     return splits == 1 || ((int64_t)((a.N + 15) / 16) * 16 <= GEMV_COUNTER_BYTES / 4);
 }
 
+int gemv_stage_splits(int64_t K) { return stage_splits(K); }
+
 size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int s = stage_splits(K);
     return (size_t)GEMV_COUNTER_BYTES + (s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0);

@@ -12,7 +12,8 @@ Prints ONE JSON line:
   roofline  = the kernel that takes the largest share of a step (the three decode kernels are
               timed group by group): algorithmic bytes per launch / average launch duration, from
               HIP events recorded inside the timed region on the launch stream, against the
-              8 TB/s HBM peak; config.kernels lists all three
+              8 TB/s HBM peak; config.kernels lists all three groups, each with the time of a
+              launch that only reads the same weights (pure_read_launch_us, frac_of_pure_read)
   config.prefill = BASELINE config 3 (M in {512, 2048, 8192}) run after the timed region: TFLOP/s of the fused GEMM
               kernel, of HIP dequantize + the hand-written dense kernel and of HIP dequantize + the library GEMM, vs
               the bf16 MFMA peak; which of them the router picks
@@ -172,6 +173,37 @@ def main() -> int:
     def pct(sorted_vals, q):
         return sorted_vals[min(len(sorted_vals) - 1, int(q * len(sorted_vals)))]
 
+    # What one launch that only reads the same bytes takes (codes and absmax of a weight, cold, from the same rings;
+    # libnf4hip_probe.so: 16 bytes per lane, whole lines, non-temporal, nothing computed): per shape the average of 20
+    # launches back to back between two events -- the same protocol as the groups above, launch gaps included.
+    pure_read_us = {}
+    probe_path = os.path.join(ROOT, "lightning-thunder_amd", "libnf4hip_probe.so")
+    if os.path.exists(probe_path):
+        import ctypes
+
+        probe = ctypes.CDLL(probe_path)
+        probe.nf4hip_probe_stream_read.restype = ctypes.c_int
+        probe.nf4hip_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        for (N, K) in SHAPES:
+            ring = weights[(N, K)]
+
+            def read(i):
+                qw, absmax = ring[i % len(ring)]
+                rc = probe.nf4hip_probe_stream_read(qw.data_ptr(), qw.numel() // 16 * 16, absmax.data_ptr(), absmax.numel() * 4 // 16 * 16,
+                                                    sink.data_ptr(), sptr)
+                assert rc == 0, rc
+
+            for i in range(3):
+                read(i)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(20):
+                read(3 + i)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            pure_read_us[(N, K)] = e0.elapsed_time(e1) * 1e3 / 20
+
     kernels = []
     for gi, (name, what, calls) in enumerate(groups):
         G = len(groups)
@@ -190,6 +222,12 @@ def main() -> int:
             "achieved_GBs": round(group_bytes[gi] / (ms * 1e-3) / 1e9, 1),
             "share_of_step_time": round(ms / ms_per_step, 3),
         })
+        if pure_read_us:
+            # a launch that only reads each weight of the group, and how close the group's launches come to it
+            pr = sum(pure_read_us[(N, K)] for (_, N, K) in calls) / len(calls)
+            kernels[-1]["pure_read_launch_us"] = round(pr, 3)
+            kernels[-1]["pure_read_us_by_shape"] = {f"[{N},{K}]": round(pure_read_us[(N, K)], 2) for (_, N, K) in calls}
+            kernels[-1]["frac_of_pure_read"] = round(pr / (ms * per_launch), 4)
     dom = max(kernels, key=lambda k: k["share_of_step_time"])
 
     # HBM traffic per launch of that group: counter figures (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE) cannot be taken

@@ -26,6 +26,23 @@ def test_library_exports_every_declared_symbol(ta):
     assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 5
 
 
+def test_probe_library_loads_and_validates(ta):
+    """libnf4hip_probe.so (bench.py's read-only kernel) is built next to the path's library and refuses bad arguments
+    before it launches anything."""
+    import ctypes
+    import os
+
+    path = os.path.join(os.path.dirname(ta.__file__), "libnf4hip_probe.so")
+    assert os.path.exists(path), "run __graft_entry__.build()"
+    probe = ctypes.CDLL(path)
+    fn = probe.nf4hip_probe_stream_read
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    assert fn(None, 1024, None, 0, None, None) != 0
+    assert fn(4096, 1000, None, 0, None, None) != 0  # not a multiple of 16
+    assert fn(4096, 1024, None, 16, None, None) != 0  # bytes of b without b
+
+
 def test_missing_library_fails_loudly(ta, tmp_path):
     with pytest.raises(RuntimeError, match="not found"):
         ta._lib.load(str(tmp_path / "libnf4hip.so"))

@@ -13,7 +13,9 @@ Prints ONE JSON line:
               timed group by group): algorithmic bytes per launch / average launch duration, from
               HIP events recorded inside the timed region on the launch stream, against the
               8 TB/s HBM peak; config.kernels lists all three groups, each with the time of a
-              launch that only reads the same weights (pure_read_launch_us, frac_of_pure_read)
+              launch that only reads the same weights (pure_read_launch_us, frac_of_pure_read);
+              config.by_kernel: the same calls grouped by the kernel the library launches for them (nf4hip_gemv_plan),
+              timed after the timed region
   config.prefill = BASELINE config 3 (M in {512, 2048, 8192}) run after the timed region: TFLOP/s of the fused GEMM
               kernel, of HIP dequantize + the hand-written dense kernel and of HIP dequantize + the library GEMM, vs
               the bf16 MFMA peak; which of them the router picks
@@ -170,6 +172,55 @@ def main() -> int:
     warm_events[-1].record(stream)
     torch.cuda.synchronize()
 
+    # By KERNEL, after the timed region (which kernel serves a call is the library's answer, nf4hip_gemv_plan): the same
+    # 15 calls, cold, issued in four segments with an event between them -- the calls with one row of x that the kernel
+    # with the largest share of the bytes (the staged kernel, where in use) does not serve, those it serves, then the same
+    # for the remaining calls.  An event record costs about 3 us of the stream and launches of the staged kernel that
+    # follow each other directly run a few per cent slower than in the order of the timed region, so these figures are a
+    # little pessimistic.
+    import ctypes
+
+    KERNEL_NAMES = {1: "gemv_rows_kernel", 2: "gemv_quad_kernel", 3: "gemv_quad_kernel on two halves of x", 4: "gemv_tiles_kernel",
+                    5: "gemv_stage_kernel"}
+
+    def kernel_of(M, N, K):
+        plan = (ctypes.c_int * 4)()
+        ta._lib.check(lib.nf4hip_gemv_plan(M, N, K, BLOCKSIZE, 0, ctypes.byref(plan)))
+        return plan[0]
+
+    calls_all = [(M, N, K) for M in MS for (N, K) in SHAPES]
+    kern = {c: kernel_of(*c) for c in calls_all}
+    weight_of = {}
+    for c in calls_all:
+        weight_of[kern[c]] = weight_of.get(kern[c], 0) + algorithmic_bytes(*c)
+    main_kernel = max(weight_of, key=weight_of.get)
+    segments = [[c for c in calls_all if (c[0] == MS[0]) == first and (kern[c] == main_kernel) == is_main]
+                for first in (True, False) for is_main in (False, True)]
+    segments = [seg for seg in segments if seg]
+    k_events = [torch.cuda.Event(enable_timing=True) for _ in range(len(segments) * args.steps + 1)]
+    for st in range(args.steps):
+        for si_, seg in enumerate(segments):
+            k_events[st * len(segments) + si_].record(stream)
+            for c in seg:
+                launch(*c, args.warmup + args.steps + st)
+    k_events[-1].record(stream)
+    torch.cuda.synchronize()
+    by_kernel = {}
+    for si_, seg in enumerate(segments):
+        name = " + ".join(KERNEL_NAMES[k] for k in sorted({kern[c] for c in seg}))
+        ms = sum(k_events[st * len(segments) + si_].elapsed_time(k_events[st * len(segments) + si_ + 1]) for st in range(args.steps)) / args.steps
+        e = by_kernel.setdefault(name, {"calls": [], "ms": 0.0})
+        e["calls"] += seg
+        e["ms"] += ms
+    by_kernel_rows = []
+    for name, e in by_kernel.items():
+        byts = sum(algorithmic_bytes(*c) for c in e["calls"])
+        by_kernel_rows.append({
+            "kernel": name, "calls": "; ".join(f"M={M} [{N},{K}]" for (M, N, K) in e["calls"]), "launches_per_step": len(e["calls"]),
+            "algorithmic_bytes_per_launch": byts // len(e["calls"]), "avg_launch_us": round(e["ms"] * 1e3 / len(e["calls"]), 3),
+            "achieved_GBs": round(byts / (e["ms"] * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(byts / (e["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        })
+
     def pct(sorted_vals, q):
         return sorted_vals[min(len(sorted_vals) - 1, int(q * len(sorted_vals)))]
 
@@ -179,8 +230,6 @@ def main() -> int:
     pure_read_us = {}
     probe_path = os.path.join(ROOT, "lightning-thunder_amd", "libnf4hip_probe.so")
     if os.path.exists(probe_path):
-        import ctypes
-
         probe = ctypes.CDLL(probe_path)
         probe.nf4hip_probe_stream_read.restype = ctypes.c_int
         probe.nf4hip_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
@@ -226,7 +275,6 @@ def main() -> int:
             # a launch that only reads each weight of the group, and how close the group's launches come to it
             pr = sum(pure_read_us[(N, K)] for (_, N, K) in calls) / len(calls)
             kernels[-1]["pure_read_launch_us"] = round(pr, 3)
-            kernels[-1]["pure_read_us_by_shape"] = {f"[{N},{K}]": round(pure_read_us[(N, K)], 2) for (_, N, K) in calls}
             kernels[-1]["frac_of_pure_read"] = round(pr / (ms * per_launch), 4)
     dom = max(kernels, key=lambda k: k["share_of_step_time"])
 
@@ -260,6 +308,8 @@ def main() -> int:
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
             "algorithmic_bytes_per_step": bytes_step,
             "kernels": kernels,
+            "by_kernel": by_kernel_rows,
+            "pure_read_us_by_shape": {f"[{N},{K}]": round(t, 2) for (N, K), t in pure_read_us.items()},
             "inputs_sha256_16": fingerprints,
         },
         "roofline": {

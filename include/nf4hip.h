@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define NF4HIP_ABI_VERSION 5
+#define NF4HIP_ABI_VERSION 6
 
 #define NF4HIP_BF16 0
 #define NF4HIP_F16 1
@@ -116,6 +116,15 @@ size_t nf4hip_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * tests; nf4hip_gemv_workspace_bytes covers every choice.
  */
 int nf4hip_gemv_prefer_staged(int mode);
+/*
+ * Which of the decode kernels nf4hip_gemv launches for a call without an epilogue (no GPU needed; follows
+ * nf4hip_gemv_prefer_staged): plan[0] = 1 row-streaming, 2 four weight rows per lane quad, 3 the same on two halves of
+ * x, 4 MFMA tiles with x in LDS, 5 codes and absmax staged through LDS; plan[1] = the arithmetic of the call: 0 bf16 code
+ * book, 1 fp16 code book, 2 every weight rounded to bf16(code value * absmax) as the reference rounds it; plan[2],
+ * plan[3] reserved (0).  `nested` non-zero: the call would go through nf4hip_gemv_dq.  For benchmarks and profiles that
+ * attribute time to kernels; results never depend on the choice beyond the tolerance of the call.
+ */
+int nf4hip_gemv_plan(int64_t M, int64_t N, int64_t K, int blocksize, int nested, int32_t plan[4]);
 int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
                 const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
                 size_t workspace_bytes, void* stream);

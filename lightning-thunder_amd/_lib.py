@@ -11,7 +11,7 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 BF16, F16, F32 = 0, 1, 2
 
@@ -62,6 +62,7 @@ SYMBOLS = {
     "nf4hip_gemv_norm_parts": (_i32, [_i64, _i64, _i64]),
     "nf4hip_gemv_epilogue_served": (_i32, [_i64, _i64, _i64, _i32, _i32, _i32]),
     "nf4hip_gemv_static": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp]),
+    "nf4hip_gemv_plan": (_i32, [_i64, _i64, _i64, _i32, _i32, ctypes.POINTER(_i32 * 4)]),
     "nf4hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "nf4hip_gemm_plan": (_i32, [_i64, _i64, _i64, ctypes.POINTER(_i32 * 4)]),
     "nf4hip_gemm": (_i32, _MATMUL),

@@ -299,6 +299,20 @@ int nf4hip_gemm_plan(int64_t M, int64_t N, int64_t K, int32_t plan[4]) {
     return NF4HIP_OK;
 }
 
+int nf4hip_gemv_plan(int64_t M, int64_t N, int64_t K, int blocksize, int nested, int32_t plan[4]) {
+    if (!plan) return fail(NF4HIP_E_NULL, "nf4hip_gemv_plan: plan is null");
+    const int bl = block_log2(blocksize);
+    if (bl < 0) return fail(NF4HIP_E_BLOCKSIZE, "nf4hip_gemv_plan: blocksize %d unsupported", blocksize);
+    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX || (M <= 4 ? K % 32 : K % 512) ||
+        (M > 4 && K > (1 << 24)))
+        return fail(NF4HIP_E_SHAPE, "nf4hip_gemv_plan: not a shape nf4hip_gemv takes (M = %lld, N = %lld, K = %lld)", (long long)M,
+                    (long long)N, (long long)K);
+    int p[4];
+    nf4::gemv_plan(M, N, K, bl, nested != 0, p);
+    for (int i = 0; i < 4; ++i) plan[i] = p[i];
+    return NF4HIP_OK;
+}
+
 int nf4hip_gemv(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax, const float* lut16,
                 const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out, void* workspace,
                 size_t workspace_bytes, void* stream) {

@@ -94,6 +94,8 @@ size_t gemm_wide_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // plan[3] workgroups launched.
 void gemm_wide_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
 void gemm_plan(int64_t M, int64_t N, int64_t K, int plan[4]);
+// which decode kernel serves a call without an epilogue (GEMV_KERNEL_* of nf4_gemv.h) and its arithmetic mode (ARITH_*)
+void gemv_plan(int64_t M, int64_t N, int64_t K, int block_log2, bool nested, int plan[4]);
 // dense bf16 GEMM (nf4_gemm_dense.hip): K a multiple of 64, at least 128
 bool gemm_dense_possible(int64_t M, int64_t N, int64_t K);
 size_t gemm_dense_workspace_bytes(int64_t M, int64_t N, int64_t K);

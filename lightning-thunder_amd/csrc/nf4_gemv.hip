@@ -141,6 +141,29 @@ int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     return gemv_tiles_norm_parts(N);
 }
 
+// Which kernel launch_gemv picks for a call without an epilogue: GEMV_KERNEL_* of nf4_gemv.h.
+int gemv_kernel_for(int64_t M, int64_t N, int64_t K, int block_log2, bool nested) {
+    MatmulArgs a{};
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.block_log2 = block_log2;
+    static const uint8_t some_codes = 0;
+    a.nested.q = nested ? &some_codes : nullptr;  // (only looked at for being non-null)
+    if (stage_serves(a)) return GEMV_KERNEL_STAGED;
+    if (rows_serve(M, N, K)) return GEMV_KERNEL_ROWS;
+    if (quad_halves_serve(M, N, K)) return GEMV_KERNEL_QUAD_HALVES;
+    return quad_serves(M, N, K) ? GEMV_KERNEL_QUAD : GEMV_KERNEL_TILES;
+}
+
+void gemv_plan(int64_t M, int64_t N, int64_t K, int block_log2, bool nested, int plan[4]) {
+    plan[0] = gemv_kernel_for(M, N, K, block_log2, nested);
+    // (the tile kernel has its fp16 mode only where a workgroup's K range is one slice of x: reported as exact beyond 8192)
+    plan[1] = plan[0] == GEMV_KERNEL_STAGED ? ARITH_BF16 : gemv_arith_mode(K, plan[0] != GEMV_KERNEL_TILES);
+    plan[2] = 0;
+    plan[3] = 0;
+}
+
 hipError_t launch_gemv(const MatmulArgs& a, hipStream_t stream) {
     if (!gemv_epilogue_possible(a)) return hipErrorNotSupported;
     int cus = 0;

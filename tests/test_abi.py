@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(ta):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/nf4hip.h but not exported"
     assert sorted(ta._lib.SYMBOLS) == declared, "ctypes prototypes out of sync with the header"
-    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 5
+    assert lib.nf4hip_abi_version() == ta._lib.ABI_VERSION == 6
 
 
 def test_probe_library_loads_and_validates(ta):
@@ -50,6 +50,32 @@ def test_missing_library_fails_loudly(ta, tmp_path):
 
 def _err(ta):
     return ta._lib.load().nf4hip_last_error().decode()
+
+
+def test_gemv_plan_names_the_kernel(ta):
+    """nf4hip_gemv_plan: which decode kernel a call goes to, without a GPU; it follows nf4hip_gemv_prefer_staged."""
+    import ctypes
+
+    L, lib = ta._lib, ta._lib.load()
+    plan = (ctypes.c_int * 4)()
+
+    def kernel(M, N, K, nested=0):
+        assert lib.nf4hip_gemv_plan(M, N, K, 64, nested, ctypes.byref(plan)) == 0
+        return plan[0], plan[1]
+
+    assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+    assert kernel(1, 4096, 4096) == (1, 0) and kernel(4, 4096, 4096) == (2, 0) and kernel(16, 1024, 4096) == (3, 0)
+    assert kernel(1, 128256, 4096) == (5, 0) and kernel(16, 14336, 4096) == (5, 0) and kernel(4, 14336, 4096) == (2, 0)
+    assert kernel(1, 4096, 14336) == (1, 1) and kernel(16, 4096, 14336)[0] == 4
+    assert kernel(1, 28672, 8192) == (1, 0) and kernel(16, 28672, 8192)[0] == 4  # K beyond one workgroup's sixteen slices
+    assert kernel(1, 128256, 4096, nested=1)[0] == 1  # nested absmax never goes to the staged kernel
+    assert lib.nf4hip_gemv_prefer_staged(0) == 0
+    assert kernel(1, 128256, 4096)[0] == 1
+    assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+    assert lib.nf4hip_gemv_plan(17, 4096, 4096, 64, 0, ctypes.byref(plan)) == L.E_SHAPE
+    assert lib.nf4hip_gemv_plan(8, 4096, 4096 + 64, 64, 0, ctypes.byref(plan)) == L.E_SHAPE
+    assert lib.nf4hip_gemv_plan(1, 4096, 4096, 48, 0, ctypes.byref(plan)) == L.E_BLOCKSIZE
+    assert lib.nf4hip_gemv_plan(1, 4096, 4096, 64, 0, None) == L.E_NULL
 
 
 def test_linear_argument_errors_and_plan(ta):

@@ -60,7 +60,7 @@ constexpr int ABS_OFF = RING_OFF + ST_WAVES * RING_SLOTS * SLOT_BYTES;
 constexpr int ABS_BYTES = 16 * ST_WAVES * 16;  // 16 rows x 16 waves x 16 B
 constexpr int ABS_BUFS = 3;
 constexpr int ST_SMEM_BYTES = ABS_OFF + ABS_BUFS * ABS_BYTES;  // 64 + 80 + 12 = 156 KB
-constexpr int RED_BUF_BYTES = ST_WAVES * 1024;                 // per buffer: 16 waves x 64 lanes x 16 B
+constexpr int RED_BUF_BYTES = ST_WAVES * 1024;                 // per buffer: 16 rows of x, a plane of 16 waves x 16 weight rows x 4 B each
 static_assert(2 * RED_BUF_BYTES <= TABLE_SPAN / 2, "reduction buffers live in the table's unused half rows");
 static_assert(ST_SMEM_BYTES <= 160 * 1024, "LDS of one CU");
 
@@ -94,6 +94,10 @@ __device__ __forceinline__ float4 lds_read_f32x4(uint32_t addr) {
     const f32x4_t v = *reinterpret_cast<p_t>((uintptr_t)addr);
     return make_float4(v.x, v.y, v.z, v.w);
 }
+__device__ __forceinline__ void lds_write_f32(uint32_t addr, float v) {
+    typedef __attribute__((address_space(3))) float* p_t;
+    *reinterpret_cast<p_t>((uintptr_t)addr) = v;
+}
 __device__ __forceinline__ void lds_write_f32x4(uint32_t addr, f32x4 v) {
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) f32x4_t* p_t;
@@ -108,9 +112,19 @@ __device__ __forceinline__ void wait_vm() {
 }
 __device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-// 16 bytes per active lane from a buffer straight into LDS at lds_base + lane * 16 (nontemporal)
-__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t byte_offset) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(uintptr_t)lds_base, 16, byte_offset, 0, 0, 2 /* nt */);
+// 16 bytes per active lane from a buffer straight into LDS at lds_base + lane * 16 (nontemporal); the byte offset is a
+// per-lane part that never changes (a register) plus a wave-uniform part (a scalar register: no vector arithmetic
+// per load)
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t lane_offset, uint32_t wave_offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(uintptr_t)lds_base, 16, lane_offset, wave_offset, 0, 2 /* nt */);
+}
+
+// float -> bf16 bits, round to nearest even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t bf16_bits_hw(float f) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {f, f};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t)) & 0xffffu;
 }
 
 // MGROUPS: lane groups of four rows of x that carry rows < M: ceil(M / 4).  EPI: the epilogue flags of the call.
@@ -172,32 +186,34 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     // ---- load side: lane constants ----------------------------------------------------------------------------------
     // code loads: lane i takes row (i >> 3) of the 8-row half tile and the 16-byte piece (i & 7) ^ f(row in tile),
     // f(n) = n >> 1 (rows 0..7: the even half tile; rows 8..15: the odd one)
+    // The lane's share of the offset is fixed for the whole launch; which half tile is a wave-uniform offset.  A half
+    // tile beyond the workgroup's range is replaced by its last one (rows of a workgroup come in whole half tiles, so
+    // nothing outside the weight is ever addressed).
     const int lrow = lane >> 3;
-    const uint32_t cpiece_even = (uint32_t)((lane & 7) ^ (lrow >> 1)) << 4;
-    const uint32_t cpiece_odd = (uint32_t)((lane & 7) ^ (4 + (lrow >> 1))) << 4;
-    const uint32_t ccol = (uint32_t)slice * 128u;
+    const uint32_t ccol = (uint32_t)lrow * (uint32_t)row_bytes + (uint32_t)slice * 128u;
+    const uint32_t clane_even = ccol + ((uint32_t)((lane & 7) ^ (lrow >> 1)) << 4);
+    const uint32_t clane_odd = ccol + ((uint32_t)((lane & 7) ^ (4 + (lrow >> 1))) << 4);
     const uint32_t ring = RING_OFF + wave * (RING_SLOTS * SLOT_BYTES);
-    auto load_codes = [&](int h, int slot) {  // half tile h of this workgroup into ring slot `slot`
-        const int row = min(r0 + 8 * h + lrow, rmax);
-        const uint32_t off = (uint32_t)row * (uint32_t)row_bytes + ccol + ((h & 1) ? cpiece_odd : cpiece_even);
-        dma16(codes_rsrc, ring + slot * SLOT_BYTES, off);
+    auto load_codes = [&](int h, bool odd, int slot) {  // half tile h of this workgroup into ring slot `slot` (odd = h & 1)
+        const uint32_t base = (uint32_t)(r0 + 8 * min(h, halves - 1)) * (uint32_t)row_bytes;
+        dma16(codes_rsrc, ring + slot * SLOT_BYTES, odd ? clane_odd : clane_even, base);
     };
     // absmax loads: wave r fetches row r of a tile, lanes 0..15 the pieces of the range's k slices; lane q stores
     // piece q ^ r at position q (readers of slice w look at position w ^ row)
     const uint32_t abs_row_bytes = (uint32_t)(K >> 6) * 4u;
     const int apiece = (lane & 15) ^ wave;
     const bool abs_lane = lane < 16 && apiece < nslices;
+    const uint32_t alane = (uint32_t)(slice0 + apiece) * 16u;
     auto load_absmax = [&](int t) {
         const int row = min(r0 + 16 * t + wave, rmax);
-        const uint32_t off = (uint32_t)row * abs_row_bytes + (uint32_t)(slice0 + apiece) * 16u;
-        if (abs_lane) dma16(abs_rsrc, ABS_OFF + (t % ABS_BUFS) * ABS_BYTES + wave * 256, off);
+        if (abs_lane) dma16(abs_rsrc, ABS_OFF + (t % ABS_BUFS) * ABS_BYTES + wave * 256, alane, (uint32_t)row * abs_row_bytes);
     };
 
     // ---- get the stream going: absmax of tiles 0 and 1, the first five half tiles -----------------------------------
     load_absmax(0);
     load_absmax(1);
 #pragma unroll
-    for (int h = 0; h < RING_SLOTS; ++h) load_codes(h, h);
+    for (int h = 0; h < RING_SLOTS; ++h) load_codes(h, h & 1, h);
 
     // ---- byte -> (bf16, bf16) table: entry e = tid >> 2, 32 bytes per thread -----------------------------------------
     {
@@ -206,6 +222,22 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         const uint32_t dst = (uint32_t)(tid >> 2) * 256u + (uint32_t)(tid & 3) * 32u;  // (the table starts at LDS address 0)
         lds_write_f32x4(dst, f32x4{v, v, v, v});
         lds_write_f32x4(dst + 16, f32x4{v, v, v, v});
+    }
+    // a wave without a slice contributes zeros to every sum: written once, into both reduction buffers
+    // Reduction buffers: the sum of wave w for (row m of x, weight row n) is dword (16 w + n) ^ (16 * ((m >> 2) & 1)) of
+    // plane m (1 KB).  Only the 32 banks of the table rows' second halves are there to be used; with this order both
+    // the writers (lane (n, g): m = 4g .. 4g + 3, a plane each) and the readers (lane (n, G): waves G, G + 4, G + 8,
+    // G + 12 of one plane) put two lanes on a bank, the least possible.  Planes are 2 KB of LDS addresses apart, the
+    // four waves a reader adds 512 bytes.
+    constexpr uint32_t RED_PLANE = (1024u >> 7) << 8;
+    const uint32_t red_w0 = red_addr((uint32_t)(4 * g) * 1024u + (uint32_t)((16 * wave + n) ^ ((g & 1) << 4)) * 4u);
+    auto write_partials = [&](uint32_t at, const f32x4& v) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds_write_f32(at + (uint32_t)i * RED_PLANE, v[i]);
+    };
+    if (!wave_on && g < MGROUPS) {
+        write_partials(red_w0, f32x4{0.f, 0.f, 0.f, 0.f});
+        write_partials(red_w0 + ((RED_BUF_BYTES >> 7) << 8), f32x4{0.f, 0.f, 0.f, 0.f});
     }
     wait_vm<RING_SLOTS>();  // everything older than the five code loads: x, code book, absmax of tiles 0 and 1
     // (x is in its registers from here on: said once, so that the loop does not carry waits for it)
@@ -224,26 +256,45 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     // ---- read side: lane constants ------------------------------------------------------------------------------------
     const uint32_t col4 = (uint32_t)(lane & 31) * 4u;
     const int f = n >> 1;
-    // codes of block b: 8 bytes at piece (2b + (g >> 1)) ^ f, half (g & 1), of row n & 7 of the even / odd half tile
-    const uint32_t cread0 = ring + (uint32_t)(n & 7) * 128u + ((uint32_t)((g >> 1) ^ f) << 4) + (uint32_t)(g & 1) * 8u;
+    // codes of block b: 8 bytes at piece (2b + (g >> 1)) ^ f, half (g & 1), of row n & 7 of the even (n < 8) / odd half
+    // tile.  The odd half tile's slot follows the even one's, except where the ring wraps (slots 4 and 0): one address
+    // per block for either case, the slot itself is a constant offset of the read.
+    uint32_t cread[4], cread_wrap[4];
+    {
+        const uint32_t c0 = ring + (uint32_t)(n & 7) * 128u + ((uint32_t)((g >> 1) ^ f) << 4) + (uint32_t)(g & 1) * 8u;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            cread[b] = (c0 ^ (uint32_t)(b << 5)) + (n < 8 ? 0u : (uint32_t)SLOT_BYTES);
+            cread_wrap[b] = (c0 ^ (uint32_t)(b << 5)) + (n < 8 ? (uint32_t)((RING_SLOTS - 1) * SLOT_BYTES) : 0u);
+        }
+    }
     const uint32_t aread = ABS_OFF + (uint32_t)(n * 16 + ((wave_on ? wave : 0) ^ n)) * 16u;
-    const uint32_t red_write = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
     const bool reducer = wave < M;  // wave m finishes row m of x
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
 
-    // Finishing tile t (wave m, row m of x): lane (n, G = g) reads the partial sums of waves G, G + 4, G + 8, G + 12 ...
+    // The two reduction buffers are 32 KB of LDS addresses apart: a wave's write address and a finishing wave's read
+    // address change buffers by flipping that bit.  Tile t is written into buffer t & 1.
+    constexpr uint32_t RED_FLIP = (RED_BUF_BYTES >> 7) << 8;
+    uint32_t red_w = red_w0;
+    // Finishing a tile (wave m, row m of x): lane (n, G = g) reads the partial sums of waves G, G + 4, G + 8, G + 12 ...
+    uint32_t red_r = red_addr((uint32_t)wave * 1024u + (uint32_t)((16 * g + n) ^ (((wave >> 2) & 1) << 4)) * 4u);
     struct Pending {
         float p[4];
     };
-    auto read_partials = [&](int t) {
-        const int m = wave;
-        const uint32_t src = (uint32_t)(t & 1) * RED_BUF_BYTES + (uint32_t)(16 * (m >> 2) + n) * 16u + (uint32_t)(m & 3) * 4u;
+    auto read_partials = [&]() {  // of the oldest tile not yet finished
         Pending pd;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) pd.p[q] = lds_read_f32(red_addr(src + (uint32_t)(g + 4 * q) * 1024u));
+        for (int q = 0; q < 4; ++q) pd.p[q] = lds_read_f32(red_r + (uint32_t)q * 512u);
+        red_r ^= RED_FLIP;
         return pd;
     };
+    // where row r0 + n of this workgroup sits in row m of the output, in bytes; stores go through a buffer that ends
+    // with the workgroup's last row, so that the rows of a last, half-filled tile are dropped by the range check
+    const uint32_t out_lane = (uint32_t)(r0 + n) * 2u;
+    const bool pairs = (EPI & EPI_SILU_PAIRS) != 0;
+    const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        a.out + (int64_t)(reducer ? wave : 0) * (pairs ? (N >> 1) : N), 0, pairs ? r1 : 2 * r1, 0x00020000);
     // ... adds them in that order, then the four lane groups (two register swaps across the wave: no LDS round trip),
     // and stores the 16 outputs
     auto finish_tile = [&](int t, const Pending& pd) {
@@ -257,21 +308,25 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
             const auto r2 = __builtin_amdgcn_permlane32_swap(w, w, false, false);
             sum = __uint_as_float(r2[0]) + __uint_as_float(r2[1]);             // lanes l and l ^ 32
         }
-        const int row = r0 + 16 * t + n;
         if (splits == 1) {
+            const uint32_t at = out_lane + 32u * (uint32_t)t;  // byte offset of row r0 + 16 t + n
             if (EPI & EPI_ROWSCALE) sum *= rstd;
+            if (a.bias) {
+                const int row = r0 + 16 * t + n;
+                if (row < r1) sum += bf16_bits_to_f32(a.bias[row]);
+            }
             if (EPI & EPI_SILU_PAIRS) {
                 // rows 2j, 2j + 1 = gate j, up j: the even row's lane takes the odd row's value (lane ^ 1)
-                if (a.bias && row < r1) sum += bf16_bits_to_f32(a.bias[row]);
                 const float mine = nf4x::round_bf16(sum);
                 const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine), 0xB1, 0xf, 0xf, true));
-                if (g == 0 && row < r1 && !(n & 1)) a.out[(int64_t)m * (N >> 1) + (row >> 1)] = (uint16_t)nf4x::silu_mul_bf16(mine, other);
-            } else if (g == 0 && row < r1) {
-                if (a.bias) sum += bf16_bits_to_f32(a.bias[row]);
-                a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(sum);
+                if (g == 0 && !(n & 1))
+                    __builtin_amdgcn_raw_buffer_store_b16((short)nf4x::silu_mul_bf16(mine, other), out_rsrc, at >> 1, 0, 0);
+            } else if (g == 0) {
+                __builtin_amdgcn_raw_buffer_store_b16((short)bf16_bits_hw(sum), out_rsrc, at, 0, 0);
             }
         } else {
             // K split over workgroups: this wave's 16 sums of (tile, m) meet those of the other ranges in the workspace
+            const int row = r0 + 16 * t + n;
             const int tile_id = (r0 >> 4) + t;  // (with K split, a workgroup's rows start at a multiple of 16)
             if (g == 0 && row < r1)
                 __hip_atomic_store(&partial[((int64_t)split * M + m) * N + row], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -319,29 +374,30 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         for (int i = 0; i < 4; ++i) acc[i] = fmaf(c1[i], sb, acc[i]);
     };
 
-    auto tile_body = [&](int t, auto s0_tag, auto s1_tag) {
+    auto tile_body = [&](int t, auto s0_tag, auto s1_tag, auto first_tag) {
         constexpr int S0 = decltype(s0_tag)::value, S1 = decltype(s1_tag)::value;
+        constexpr bool FIRST = decltype(first_tag)::value;  // tile 0: nothing to finish yet
+        static_assert(S1 == (S0 + 1) % RING_SLOTS, "the odd half tile's slot follows the even one's");
         // Codes of this tile have landed.  A wave's LOADS in issue order: absmax 0, 1, half tiles 0..4, then per tile t'
         // absmax t' + 2, half tiles 2t' + 5, 2t' + 6.  The youngest load this tile needs is half tile 2t + 1 (first code
         // load of tile t - 2); younger are the second code load of tile t - 2 and the three loads of tile t - 1: four
         // (three in tile 0).  A finishing wave's stores are counted by the same counter but may complete in any order
         // with respect to loads: the count assumes none is outstanding, which is exact when they have completed and waits
         // for a load or two more than needed when they have not.
-        if (t == 0)
+        if (FIRST)
             wait_vm<3>();
         else
             wait_vm<4>();
 
         // this tile's codes and scales into registers, so that their LDS slots can be refilled while the tile is multiplied
-        const uint32_t cread = cread0 + (n < 8 ? S0 * SLOT_BYTES : S1 * SLOT_BYTES);
         uint2 cd[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) cd[b] = lds_read_u32x2(cread ^ (uint32_t)(b << 5));
+        for (int b = 0; b < 4; ++b) cd[b] = S1 > S0 ? lds_read_u32x2(cread[b] + S0 * SLOT_BYTES) : lds_read_u32x2(cread_wrap[b]);
         const float4 am4 = lds_read_f32x4(aread + (t % ABS_BUFS) * ABS_BYTES);
-        // the previous tile's partial sums (all written before the barrier that ended it): requested now, added up at the
-        // end of this tile
-        Pending pd = {};
-        if (reducer && t > 0) pd = read_partials(t - 1);
+        // the previous tile's partial sums (all written before the barrier that ended it): requested now, added up
+        // between the halves of this tile
+        Pending pd;
+        if (!FIRST && reducer) pd = read_partials();
 
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         two_blocks(cd[0], cd[1], xa[0], xa[1], am4.x, am4.y, acc);
@@ -351,16 +407,16 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         // absmax request goes into the buffer tile t - 1 used; every wave is past the barrier that ended it.
         asm volatile("" ::"v"(cd[2].x), "v"(cd[3].y), "v"(am4.w));
         load_absmax(t + 2);
-        load_codes(2 * t + RING_SLOTS, S0);
-        load_codes(2 * t + RING_SLOTS + 1, S1);
+        load_codes(2 * t + RING_SLOTS, true, S0);
+        load_codes(2 * t + RING_SLOTS + 1, false, S1);
 
         // the previous tile is finished here, between the two halves, so that its chain of additions, swaps and the
         // store runs in the shadow of the second half's table reads
-        if (reducer && t > 0) finish_tile(t - 1, pd);
+        if (!FIRST && reducer) finish_tile(t - 1, pd);
 
         two_blocks(cd[2], cd[3], xa[2], xa[3], am4.z, am4.w, acc);
-        if (!wave_on) acc = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (g < MGROUPS) lds_write_f32x4(red_addr((uint32_t)(t & 1) * RED_BUF_BYTES + red_write), acc);
+        if (g < MGROUPS && wave_on) write_partials(red_w, acc);
+        red_w ^= RED_FLIP;
 
         // absmax of tile t + 1 (requested one tile ago) has landed in every wave before anyone reads it: younger loads are
         // the two code loads of the previous tile and this tile's three
@@ -374,14 +430,15 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
     using I4 = std::integral_constant<int, 4>;
-    for (int t = 0; t < tiles; t += RING_SLOTS) {
-        tile_body(t, I0{}, I1{});
-        if (t + 1 < tiles) tile_body(t + 1, I2{}, I3{});
-        if (t + 2 < tiles) tile_body(t + 2, I4{}, I0{});
-        if (t + 3 < tiles) tile_body(t + 3, I1{}, I2{});
-        if (t + 4 < tiles) tile_body(t + 4, I3{}, I4{});
+    tile_body(0, I0{}, I1{}, std::true_type{});
+    for (int t = 1; t < tiles; t += RING_SLOTS) {
+        tile_body(t, I2{}, I3{}, std::false_type{});
+        if (t + 1 < tiles) tile_body(t + 1, I4{}, I0{}, std::false_type{});
+        if (t + 2 < tiles) tile_body(t + 2, I1{}, I2{}, std::false_type{});
+        if (t + 3 < tiles) tile_body(t + 3, I3{}, I4{}, std::false_type{});
+        if (t + 4 < tiles) tile_body(t + 4, I0{}, I1{}, std::false_type{});
     }
-    if (reducer) finish_tile(tiles - 1, read_partials(tiles - 1));
+    if (reducer) finish_tile(tiles - 1, read_partials());
     wait_vm<0>();  // loads issued past the end of the range still target this workgroup's LDS
 #endif
 }
@@ -434,11 +491,11 @@ hipError_t allow_lds_mg() {
 }  // namespace
 
 // What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 8192 (beyond, the bf16 code book is not
-// accurate enough), offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up)
+// accurate enough), N a multiple of 8 (loads fetch eight whole rows), offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up)
 // pairs (even N), and only while K is not split over workgroups.
 bool gemv_stage_possible(const MatmulArgs& a) {
     if (a.nested.q || a.block_log2 != 6) return false;
-    if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 8192) return false;
+    if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 8192 || a.N % 8) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
     if (a.epi.flags != EPI_NONE) {

@@ -64,7 +64,8 @@ def _run(ta, lib, oracle, M, N, K, seed, bias=False, reps=1):
         assert torch.equal(r.view(torch.int16), results[0].view(torch.int16)), "a repeated launch gave other bits"
 
 
-# K = 4096: sixteen slices, one K range.  N: one half tile, ragged rows (N % 8 != 0), more rows than one round of workgroups
+# K = 4096: sixteen slices, one K range.  N: one half tile, a last tile that is half filled (N % 16 == 8), more rows than
+# one round of workgroups
 @pytest.mark.parametrize("M", [1, 2, 4, 5, 8, 9, 13, 16])
 @pytest.mark.parametrize("N,K", [(8, 4096), (1000, 4096), (4096, 4096), (6152, 4096)])
 def test_staged_kernel_one_k_range(ta, oracle, staged, M, N, K):
@@ -88,7 +89,9 @@ def test_staged_kernel_many_launches_are_bit_stable(ta, oracle, staged):
 
 
 def test_staged_kernel_is_refused_where_it_does_not_apply(ta, oracle, staged):
-    """K not a multiple of 256, or beyond 8192: nf4hip_gemv falls back to its other kernels (same result contract)."""
+    """K not a multiple of 256 or beyond 8192, N not a multiple of 8: nf4hip_gemv falls back to its other kernels (same
+    result contract)."""
     print("staged gemv, shapes it leaves to the other kernels", flush=True)
     _run(ta, staged, oracle, 4, 512, 4096 + 512 + 32, seed=5)
     _run(ta, staged, oracle, 16, 512, 14336, seed=6)
+    _run(ta, staged, oracle, 3, 1004, 4096, seed=7)

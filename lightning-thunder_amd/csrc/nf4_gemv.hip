@@ -94,11 +94,17 @@ bool stage_serves(const MatmulArgs& a) {
     const int mode = stage_mode();
     if (mode == 0 || !gemv_stage_possible(a)) return false;
     if (mode == 1) return true;
-    // K beyond what the sixteen waves of a workgroup cover (4096) is split over workgroups, and that hand-off drains the
-    // stream once per tile: [28672, 8192] takes 44 / 47 / 56 us there with one / four / sixteen rows of x against 26 / 26 / 46
-    // in the other kernels.
-    if (gemv_stage_splits(a.K) > 1) return false;
     const int64_t weights = (int64_t)a.N * a.K;
+    // K beyond what the sixteen waves of a workgroup cover (4096) is split over workgroups that meet in the workspace
+    // after their last tile, 1-2 us that the other kernels do not pay: [28672, 8192] 26.6 / 27.8 / 29.8 / 29.8 / 33.2 us with
+    // 1 / 4 / 8 / 9 / 16 rows of x against 25.5 / 25.7 / 28.9 / 44.0 / 44.2; [8192, 8192] 13.3 / 13.3 / 13.6 / 13.5 / 14.9 against
+    // 11.0 / 11.7 / 13.9 / 18.0 / 18.1; [4096, 8192] 10.4 / 10.4 / 10.7 / 10.8 / 12.0 against 7.3 / 9.2 / 10.9 / 13.3 / 13.6; beyond
+    // 8192 (fp16 arithmetic on both sides) [4096, 14336] 14.1 / 14.5 / 14.5 / 14.8 / 15.1 / 16.2 with 1 / 4 / 5 / 8 / 9 / 16 rows
+    // against 10.6 / 13.9 / 17.0 / 17.2 / 17.4 / 17.8, [8192, 14336] 18.6 / 19.3 / 19.4 / 19.6 / 21.0 / 22.4 against 16.0 / 18.6 /
+    // 22.0 / 22.3 / 27.4 / 27.6.
+    // (from five rows of x on beyond K = 8192 by these numbers; kept at nine, where the tile kernel takes over on the
+    // other side, so that the decode step's eight-row products and their epilogues stay in one kernel)
+    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= 9;
     if (weights >= 100000000) return true;
     if (weights >= 40000000) return a.M >= 5;
     return weights >= ((int64_t)1 << 24) && a.M >= 9;
@@ -111,7 +117,7 @@ bool stage_serves(const MatmulArgs& a) {
 void gemv_set_staged(int mode) { g_stage_mode.store(mode < -1 || mode > 1 ? -1 : mode, std::memory_order_relaxed); }
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    const size_t staged = K % 256 == 0 && K <= 8192 ? gemv_stage_workspace_bytes(M, N, K) : 0;
+    const size_t staged = K % 256 == 0 && K <= 16384 ? gemv_stage_workspace_bytes(M, N, K) : 0;
     const size_t other = gemv_workspace_bytes_unstaged(M, N, K);
     return staged > other ? staged : other;
 }
@@ -125,6 +131,14 @@ size_t gemv_workspace_bytes_unstaged(int64_t M, int64_t N, int64_t K) {
 bool gemv_epilogue_possible(const MatmulArgs& a) {
     if (a.epi.flags == EPI_NONE) return true;
     if (stage_serves(a)) return true;
+    // The same product without an epilogue would go to the staged kernel, which does not have this one: refused, so that
+    // a caller who runs the product and the operation one after the other adds to the same sums either way (an
+    // epilogue promises the stored roundings of that two-step route)
+    {
+        MatmulArgs plain = a;
+        plain.epi = Epilogue{};
+        if (stage_serves(plain)) return false;
+    }
     if (rows_serve(a.M, a.N, a.K)) return gemv_rows_epilogue_possible(a);
     if (quad_halves_serve(a.M, a.N, a.K) || quad_serves(a.M, a.N, a.K)) return gemv_quad_epilogue_possible(a);
     return gemv_tiles_epilogue_possible(a);
@@ -135,6 +149,15 @@ bool gemv_epilogue_possible(const MatmulArgs& a) {
 int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     int cus = 256;
     if (device_setup(&cus) != hipSuccess) cus = 256;
+    {
+        // where the product by itself goes to the staged kernel, the residual epilogue is not served (gemv_epilogue_possible)
+        MatmulArgs plain{};
+        plain.M = (int)M;
+        plain.N = (int)N;
+        plain.K = (int)K;
+        plain.block_log2 = 6;
+        if (stage_serves(plain)) return 0;
+    }
     if (rows_serve(M, N, K)) return gemv_rows_norm_parts(M, N, K, cus);
     if (quad_halves_serve(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, true);
     if (quad_serves(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, false);
@@ -159,7 +182,7 @@ int gemv_kernel_for(int64_t M, int64_t N, int64_t K, int block_log2, bool nested
 void gemv_plan(int64_t M, int64_t N, int64_t K, int block_log2, bool nested, int plan[4]) {
     plan[0] = gemv_kernel_for(M, N, K, block_log2, nested);
     // (the tile kernel has its fp16 mode only where a workgroup's K range is one slice of x: reported as exact beyond 8192)
-    plan[1] = plan[0] == GEMV_KERNEL_STAGED ? ARITH_BF16 : gemv_arith_mode(K, plan[0] != GEMV_KERNEL_TILES);
+    plan[1] = gemv_arith_mode(K, plan[0] != GEMV_KERNEL_TILES);
     plan[2] = 0;
     plan[3] = 0;
 }

@@ -28,8 +28,9 @@
 //    buffered, one barrier per tile); wave m adds the sixteen partials of row m of x in a fixed order, adds the bias,
 //    rounds and stores 16 consecutive outputs -- one tile late: it asks for the partials of tile t - 1 at the top of
 //    tile t and adds them up at its end, so that the reads' latency hides behind the tile's own work.
-//  * K > 4096 is split over workgroups (each keeps its slice of x): per-(tile, m) partial sums go to the workspace
-//    through agent-scope atomics, the last wave to arrive (counter per (tile, m)) adds them in split order.
+//  * K > 4096 is split over workgroups (each keeps its slice of x): the sums of a K range go to the workspace as they
+//    are finished (agent-scope stores, nothing waits for them); after its last tile a workgroup counts its arrival
+//    (one counter per row range), and the last of a row range's workgroups adds the ranges in order and stores.
 //
 //  * Epilogues (K not split): wave m may scale its finished sums of row m by 1 / rms (EPI_ROWSCALE: the producer's
 //    partial sums of squares are added up once per workgroup, by wave m for its row, while the first weights are on their
@@ -46,6 +47,7 @@ namespace nf4 {
 namespace {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
@@ -128,7 +130,11 @@ __device__ __forceinline__ uint32_t bf16_bits_hw(float f) {
 }
 
 // MGROUPS: lane groups of four rows of x that carry rows < M: ceil(M / 4).  EPI: the epilogue flags of the call.
-template <int MGROUPS, int EPI>
+// F16 (8192 < K <= 16384, where sums of bf16 code-book values drift past the matmul's tolerance): the table holds the
+// code book rounded to fp16, and the wave's slice of x is converted to fp16 once, every row scaled by a power of two
+// that puts its largest value of the slice just below 2^15 (exact for bf16 inputs); a wave's sums are scaled back before
+// they leave for the reduction.
+template <int MGROUPS, int EPI, bool F16 = false>
 __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAMS, int hot_rows_per_wg, int hot_wgs_per_split,
                                                                      int hot_splits_slices, MatmulArgs a_rest) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -217,7 +223,8 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
 
     // ---- byte -> (bf16, bf16) table: entry e = tid >> 2, 32 bytes per thread -----------------------------------------
     {
-        const uint32_t vb = f32_to_bf16_bits(lut_hi) | (f32_to_bf16_bits(lut_lo) << 16);
+        const uint32_t vb = F16 ? (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lut_hi) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lut_lo) << 16)
+                                : f32_to_bf16_bits(lut_hi) | (f32_to_bf16_bits(lut_lo) << 16);
         const float v = __uint_as_float(vb);
         const uint32_t dst = (uint32_t)(tid >> 2) * 256u + (uint32_t)(tid & 3) * 32u;  // (the table starts at LDS address 0)
         lds_write_f32x4(dst, f32x4{v, v, v, v});
@@ -243,6 +250,39 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     // (x is in its registers from here on: said once, so that the loop does not carry waits for it)
 #pragma unroll
     for (int b = 0; b < 4; ++b) asm volatile("" ::"v"(xa[b][0]), "v"(xa[b][1]));
+    // fp16 arithmetic: the lane's 64 values of row n of x -> fp16, scaled by what the row's largest value in this slice
+    // (over the four lane groups) allows; unscale[i] undoes it for output row 4g + i of this lane's sums
+    float unscale[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    if constexpr (F16) {
+        u16x2_t mx = {0, 0};
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint4 v = __builtin_bit_cast(uint4, xa[b][h]);
+                mx = absmax_of_bf16_pair(v.x, mx);
+                mx = absmax_of_bf16_pair(v.y, mx);
+                mx = absmax_of_bf16_pair(v.z, mx);
+                mx = absmax_of_bf16_pair(v.w, mx);
+            }
+        uint32_t mb = absmax_bits(mx);
+        mb = max(mb, (uint32_t)__shfl_xor((int)mb, 16, 64));
+        mb = max(mb, (uint32_t)__shfl_xor((int)mb, 32, 64));
+        const F16Scale fs = f16_scale_for(mb);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                uint4 v = __builtin_bit_cast(uint4, xa[b][h]);
+                v.x = bf16_pair_to_f16(v.x, fs.to_f16);
+                v.y = bf16_pair_to_f16(v.y, fs.to_f16);
+                v.z = bf16_pair_to_f16(v.z, fs.to_f16);
+                v.w = bf16_pair_to_f16(v.w, fs.to_f16);
+                xa[b][h] = __builtin_bit_cast(bf16x8, v);
+            }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) unscale[i] = __shfl(fs.from_f16, 4 * g + i, 64);
+    }
     wait_lds();
     __builtin_amdgcn_s_barrier();
 
@@ -325,28 +365,11 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
                 __builtin_amdgcn_raw_buffer_store_b16((short)bf16_bits_hw(sum), out_rsrc, at, 0, 0);
             }
         } else {
-            // K split over workgroups: this wave's 16 sums of (tile, m) meet those of the other ranges in the workspace
+            // K split over workgroups: this wave's 16 sums of (tile, m) go to the workspace (a store that is visible to
+            // every workgroup once acknowledged); the ranges meet after the last tile
             const int row = r0 + 16 * t + n;
-            const int tile_id = (r0 >> 4) + t;  // (with K split, a workgroup's rows start at a multiple of 16)
             if (g == 0 && row < r1)
                 __hip_atomic_store(&partial[((int64_t)split * M + m) * N + row], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            publish_partials();
-            unsigned prev = 0;
-            if (lane == 0)
-                prev = __hip_atomic_fetch_add(&counters[tile_id * 16 + m], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            prev = __builtin_amdgcn_readfirstlane(prev);
-            acquire_partials();
-            if (prev == (unsigned)splits - 1u) {
-                if (g == 0 && row < r1) {
-                    float tot = 0.0f;
-                    for (int s = 0; s < splits; ++s)
-                        tot += __hip_atomic_load(&partial[((int64_t)s * M + m) * N + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (a.bias) tot += bf16_bits_to_f32(a.bias[row]);
-                    a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(tot);
-                }
-                if (lane == 0) __hip_atomic_store(&counters[tile_id * 16 + m], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            wait_vm<0>();  // (this path's own loads and stores are not counted below: start the counting afresh)
         }
     };
 
@@ -365,8 +388,13 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
                 w1[j] = lds_read_u32(__builtin_amdgcn_perm(d1, col4, sel));
             }
             const uint4 p0 = make_uint4(w0[0], w0[1], w0[2], w0[3]), p1 = make_uint4(w1[0], w1[1], w1[2], w1[3]);
-            c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa0[h], __builtin_bit_cast(bf16x8, p0), c0, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa1[h], __builtin_bit_cast(bf16x8, p1), c1, 0, 0, 0);
+            if constexpr (F16) {
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa0[h]), __builtin_bit_cast(f16x8, p0), c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa1[h]), __builtin_bit_cast(f16x8, p1), c1, 0, 0, 0);
+            } else {
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa0[h], __builtin_bit_cast(bf16x8, p0), c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa1[h], __builtin_bit_cast(bf16x8, p1), c1, 0, 0, 0);
+            }
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] = fmaf(c0[i], sa, acc[i]);
@@ -415,6 +443,10 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         if (!FIRST && reducer) finish_tile(t - 1, pd);
 
         two_blocks(cd[2], cd[3], xa[2], xa[3], am4.z, am4.w, acc);
+        if constexpr (F16) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] *= unscale[i];
+        }
         if (g < MGROUPS && wave_on) write_partials(red_w, acc);
         red_w ^= RED_FLIP;
 
@@ -440,6 +472,31 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     }
     if (reducer) finish_tile(tiles - 1, read_partials());
     wait_vm<0>();  // loads issued past the end of the range still target this workgroup's LDS
+    if (splits > 1) {
+        // The workgroups that share these rows (one per K range) count their arrival once all their partial sums have
+        // been acknowledged; whichever comes last adds the ranges in order, for every row of x, and stores the outputs.
+        // (the flag sits where the absmax buffers were: nothing is in flight towards LDS any more)
+        publish_partials();
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = __hip_atomic_fetch_add(&counters[part], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lds_write_f32(ABS_OFF, prev == (unsigned)splits - 1u ? 1.0f : 0.0f);
+        }
+        __syncthreads();
+        acquire_partials();
+        if (lds_read_f32(ABS_OFF) != 0.0f) {
+            const int nrows = r1 - r0;
+            for (int idx = tid; idx < nrows * M; idx += ST_THREADS) {
+                const int m = idx / nrows, row = r0 + idx - m * nrows;
+                float tot = 0.0f;
+                for (int s = 0; s < splits; ++s)
+                    tot += __hip_atomic_load(&partial[((int64_t)s * M + m) * N + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (a.bias) tot += bf16_bits_to_f32(a.bias[row]);
+                a.out[(int64_t)m * N + row] = (uint16_t)f32_to_bf16_bits(tot);
+            }
+            if (tid == 0) __hip_atomic_store(&counters[part], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
 #endif
 }
 
@@ -452,8 +509,8 @@ StagePlan make_stage_plan(int64_t N, int64_t K, int cus) {
     p.slices_per_split = (total + p.splits - 1) / p.splits;
     int wgs = cus / p.splits;
     if (wgs < 1) wgs = 1;
-    // contiguous row ranges in units of 8 rows (one load); with K split, of 16 (one (tile, m) counter per tile)
-    const int unit = p.splits > 1 ? 16 : 8;
+    // contiguous row ranges in units of 8 rows (one load)
+    const int unit = 8;
     int64_t rows = (N + wgs - 1) / wgs;
     rows = (rows + unit - 1) / unit * unit;
     p.rows_per_wg = (int)rows;
@@ -461,15 +518,16 @@ StagePlan make_stage_plan(int64_t N, int64_t K, int cus) {
     return p;
 }
 
-template <int MG, int EPI>
+template <int MG, int EPI, bool F16 = false>
 hipError_t launch_mg_epi(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
-    hipLaunchKernelGGL((gemv_stage_kernel<MG, EPI>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
+    hipLaunchKernelGGL((gemv_stage_kernel<MG, EPI, F16>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
                        NF4_HOT_VALUES(a), p.rows_per_wg, p.wgs_per_split, p.splits | (p.slices_per_split << 16), a);
     return hipGetLastError();
 }
 
 template <int MG>
 hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
+    if (gemv_arith_mode(a.K, true) == ARITH_F16) return a.epi.flags == EPI_NONE ? launch_mg_epi<MG, EPI_NONE, true>(a, p, stream) : hipErrorNotSupported;
     switch (a.epi.flags) {
         case EPI_NONE: return launch_mg_epi<MG, EPI_NONE>(a, p, stream);
         case EPI_ROWSCALE: return launch_mg_epi<MG, EPI_ROWSCALE>(a, p, stream);
@@ -483,6 +541,7 @@ template <int MG>
 hipError_t allow_lds_mg() {
     hipError_t e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_SILU_PAIRS>, ST_SMEM_BYTES)) != hipSuccess) return e;
     return gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE | EPI_SILU_PAIRS>, ST_SMEM_BYTES);
@@ -490,12 +549,12 @@ hipError_t allow_lds_mg() {
 
 }  // namespace
 
-// What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 8192 (beyond, the bf16 code book is not
-// accurate enough), N a multiple of 8 (loads fetch eight whole rows), offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up)
+// What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 16384 (fp16 arithmetic beyond 8192; beyond
+// 16384 every weight would have to be rounded like the dequantised one), N a multiple of 8 (loads fetch eight whole rows), offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up)
 // pairs (even N), and only while K is not split over workgroups.
 bool gemv_stage_possible(const MatmulArgs& a) {
     if (a.nested.q || a.block_log2 != 6) return false;
-    if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 8192 || a.N % 8) return false;
+    if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 16384 || a.N % 8) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
     if (a.epi.flags != EPI_NONE) {
@@ -503,7 +562,7 @@ bool gemv_stage_possible(const MatmulArgs& a) {
         if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > 512) return false;
         if ((a.epi.flags & EPI_SILU_PAIRS) && a.N % 2) return false;
     }
-    return splits == 1 || ((int64_t)((a.N + 15) / 16) * 16 <= GEMV_COUNTER_BYTES / 4);
+    return true;  // (one arrival counter per workgroup row range: at most as many as there are CUs)
 }
 
 int gemv_stage_splits(int64_t K) { return stage_splits(K); }

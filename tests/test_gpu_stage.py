@@ -73,25 +73,28 @@ def test_staged_kernel_one_k_range(ta, oracle, staged, M, N, K):
     _run(ta, staged, oracle, M, N, K, seed=M + N, bias=(N == 1000))
 
 
-# fewer than sixteen slices (waves without a slice), and K beyond 4096: two K ranges meeting in the workspace
+# fewer than sixteen slices (waves without a slice), and K beyond 4096: two to four K ranges meeting in the workspace,
+# in fp16 arithmetic beyond 8192
 @pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,K", [(520, 512), (2048, 1024), (1024, 2560), (4096, 8192), (1160, 6144), (304, 7168)])
+@pytest.mark.parametrize("N,K", [(520, 512), (2048, 1024), (1024, 2560), (4096, 8192), (1160, 6144), (304, 7168),
+                                 (1032, 14336), (4096, 16384), (640, 9216), (2048, 12288)])
 def test_staged_kernel_short_and_split_k(ta, oracle, staged, M, N, K):
     print(f"staged gemv M={M} N={N} K={K}", flush=True)
     _run(ta, staged, oracle, M, N, K, seed=3 * M + N + K, bias=(K == 6144), reps=3)
 
 
 def test_staged_kernel_many_launches_are_bit_stable(ta, oracle, staged):
-    """[4096, 8192], sixteen rows of x: K is split over two workgroups per tile, whichever arrives last adds the
-    partial sums in range order -- 200 launches on one workspace must give one result."""
+    """[4096, 8192] and [4096, 14336], sixteen rows of x: K is split over two / four workgroups per row range, whichever
+    arrives last adds the partial sums in range order -- 200 launches on one workspace must give one result."""
     print("staged gemv, 200 launches with K split", flush=True)
     _run(ta, staged, oracle, 16, 4096, 8192, seed=99, reps=200)
+    _run(ta, staged, oracle, 16, 4096, 14336, seed=98, reps=200)
 
 
 def test_staged_kernel_is_refused_where_it_does_not_apply(ta, oracle, staged):
-    """K not a multiple of 256 or beyond 8192, N not a multiple of 8: nf4hip_gemv falls back to its other kernels (same
+    """K not a multiple of 256 or beyond 16384, N not a multiple of 8: nf4hip_gemv falls back to its other kernels (same
     result contract)."""
     print("staged gemv, shapes it leaves to the other kernels", flush=True)
     _run(ta, staged, oracle, 4, 512, 4096 + 512 + 32, seed=5)
-    _run(ta, staged, oracle, 16, 512, 14336, seed=6)
+    _run(ta, staged, oracle, 16, 512, 16384 + 512, seed=6)
     _run(ta, staged, oracle, 3, 1004, 4096, seed=7)

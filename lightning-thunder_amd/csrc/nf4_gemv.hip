@@ -102,9 +102,7 @@ bool stage_serves(const MatmulArgs& a) {
     // 8192 (fp16 arithmetic on both sides) [4096, 14336] 14.1 / 14.5 / 14.5 / 14.8 / 15.1 / 16.2 with 1 / 4 / 5 / 8 / 9 / 16 rows
     // against 10.6 / 13.9 / 17.0 / 17.2 / 17.4 / 17.8, [8192, 14336] 18.6 / 19.3 / 19.4 / 19.6 / 21.0 / 22.4 against 16.0 / 18.6 /
     // 22.0 / 22.3 / 27.4 / 27.6.
-    // (from five rows of x on beyond K = 8192 by these numbers; kept at nine, where the tile kernel takes over on the
-    // other side, so that the decode step's eight-row products and their epilogues stay in one kernel)
-    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= 9;
+    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= (a.K > 8192 ? 5 : 9);
     if (weights >= 100000000) return true;
     if (weights >= 40000000) return a.M >= 5;
     return weights >= ((int64_t)1 << 24) && a.M >= 9;
@@ -150,13 +148,14 @@ int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     int cus = 256;
     if (device_setup(&cus) != hipSuccess) cus = 256;
     {
-        // where the product by itself goes to the staged kernel, the residual epilogue is not served (gemv_epilogue_possible)
+        // where the product by itself goes to the staged kernel, so does the residual epilogue, which that kernel only has
+        // with K split over workgroups (gemv_epilogue_possible)
         MatmulArgs plain{};
         plain.M = (int)M;
         plain.N = (int)N;
         plain.K = (int)K;
         plain.block_log2 = 6;
-        if (stage_serves(plain)) return 0;
+        if (stage_serves(plain)) return gemv_stage_norm_parts(N, K, cus);
     }
     if (rows_serve(M, N, K)) return gemv_rows_norm_parts(M, N, K, cus);
     if (quad_halves_serve(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, true);

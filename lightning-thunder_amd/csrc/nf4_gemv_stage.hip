@@ -484,7 +484,30 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         }
         __syncthreads();
         acquire_partials();
-        if (lds_read_f32(ABS_OFF) != 0.0f) {
+        if (lds_read_f32(ABS_OFF) != 0.0f && (EPI & EPI_RESID_NORM)) {
+            // wave m takes row m of x: residual add, norm weight, and the sum of squares of the new residual over this
+            // workgroup's rows (lanes in a fixed order) as partial sum `part` of the row
+            if (reducer) {
+                const int m = wave;
+                float ss = 0.0f;
+                for (int row = r0 + lane; row < r1; row += 64) {
+                    float tot = 0.0f;
+                    for (int s = 0; s < splits; ++s)
+                        tot += __hip_atomic_load(&partial[((int64_t)s * M + m) * N + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (a.bias) tot += bf16_bits_to_f32(a.bias[row]);
+                    const int64_t at = (int64_t)m * N + row;
+                    const float d = nf4x::round_bf16(tot);
+                    const float res = nf4x::resid_add(bf16_bits_to_f32(a.epi.resid_in[at]), d);
+                    a.epi.resid_out[at] = (uint16_t)f32_to_bf16_bits(res);
+                    a.epi.xnext_out[at] = (uint16_t)f32_to_bf16_bits(res * bf16_bits_to_f32(a.epi.norm_weight[row]));
+                    ss = fmaf(res, res, ss);
+                }
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                if (lane == 0) a.epi.out_sumsq[m * hot_wgs_per_split + part] = ss;
+            }
+            if (tid == 0) __hip_atomic_store(&counters[part], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (lds_read_f32(ABS_OFF) != 0.0f) {
             const int nrows = r1 - r0;
             for (int idx = tid; idx < nrows * M; idx += ST_THREADS) {
                 const int m = idx / nrows, row = r0 + idx - m * nrows;
@@ -527,8 +550,12 @@ hipError_t launch_mg_epi(const MatmulArgs& a, const StagePlan& p, hipStream_t st
 
 template <int MG>
 hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
-    if (gemv_arith_mode(a.K, true) == ARITH_F16) return a.epi.flags == EPI_NONE ? launch_mg_epi<MG, EPI_NONE, true>(a, p, stream) : hipErrorNotSupported;
+    if (gemv_arith_mode(a.K, true) == ARITH_F16)
+        return a.epi.flags == EPI_NONE         ? launch_mg_epi<MG, EPI_NONE, true>(a, p, stream)
+               : a.epi.flags == EPI_RESID_NORM ? launch_mg_epi<MG, EPI_RESID_NORM, true>(a, p, stream)
+                                               : hipErrorNotSupported;
     switch (a.epi.flags) {
+        case EPI_RESID_NORM: return launch_mg_epi<MG, EPI_RESID_NORM>(a, p, stream);
         case EPI_NONE: return launch_mg_epi<MG, EPI_NONE>(a, p, stream);
         case EPI_ROWSCALE: return launch_mg_epi<MG, EPI_ROWSCALE>(a, p, stream);
         case EPI_SILU_PAIRS: return launch_mg_epi<MG, EPI_SILU_PAIRS>(a, p, stream);
@@ -542,6 +569,8 @@ hipError_t allow_lds_mg() {
     hipError_t e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_RESID_NORM, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_RESID_NORM>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_SILU_PAIRS>, ST_SMEM_BYTES)) != hipSuccess) return e;
     return gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE | EPI_SILU_PAIRS>, ST_SMEM_BYTES);
@@ -550,14 +579,17 @@ hipError_t allow_lds_mg() {
 }  // namespace
 
 // What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 16384 (fp16 arithmetic beyond 8192; beyond
-// 16384 every weight would have to be rounded like the dequantised one), N a multiple of 8 (loads fetch eight whole rows), offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up)
-// pairs (even N), and only while K is not split over workgroups.
+// 16384 every weight would have to be rounded like the dequantised one), N a multiple of 8 (loads fetch eight whole rows),
+// offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up) pairs (even N)
+// while K is not split over workgroups, the residual step only where it is.
 bool gemv_stage_possible(const MatmulArgs& a) {
     if (a.nested.q || a.block_log2 != 6) return false;
     if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 16384 || a.N % 8) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
-    if (a.epi.flags != EPI_NONE) {
+    if (a.epi.flags == EPI_RESID_NORM) {
+        if (splits == 1) return false;  // (the workgroup that adds the K ranges does the residual step; one K range has no such place)
+    } else if (a.epi.flags != EPI_NONE) {
         if ((a.epi.flags & ~(EPI_ROWSCALE | EPI_SILU_PAIRS)) || splits != 1) return false;
         if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > 512) return false;
         if ((a.epi.flags & EPI_SILU_PAIRS) && a.N % 2) return false;
@@ -566,6 +598,8 @@ bool gemv_stage_possible(const MatmulArgs& a) {
 }
 
 int gemv_stage_splits(int64_t K) { return stage_splits(K); }
+
+int gemv_stage_norm_parts(int64_t N, int64_t K, int cus) { return stage_splits(K) > 1 ? make_stage_plan(N, K, cus).wgs_per_split : 0; }
 
 size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int s = stage_splits(K);

@@ -91,14 +91,9 @@ def test_resid_norm_epilogue(ta, F, M, shape):
     got = F.matmul_nf4_epilogue(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw))
     assert got is not None
     r, xnext, sumsq = got
-    # the plain kernel's bf16 output -- of the kernel that serves the residual epilogue (the LDS-staged kernel, which
-    # may serve the plain call at this shape, has no such epilogue and adds its partial sums in another order)
-    lib = ta._lib.load()
-    assert lib.nf4hip_gemv_prefer_staged(0) == 0
-    try:
-        delta = F.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))
-    finally:
-        assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+    # the plain call's bf16 output: a shape's plain product and its residual epilogue are served by the same kernel (where
+    # the LDS-staged kernel takes the product and has no such epilogue, the epilogue is refused instead)
+    delta = F.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))
     torch.cuda.synchronize()
     r_ref = (resid_before.float() + delta.float()).to(torch.bfloat16)
     assert torch.equal(resid, resid_before)

@@ -150,7 +150,8 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
  *                           -- what SiLU(gate) * up on the bf16 output of nf4hip_gemv gives, bit for bit.
  *   NF4HIP_EPI_RESID_NORM   d = bf16(sum[m][n] + bias[n]); r = bf16(resid_in[m][n] + d) -> resid_out[m][n];
  *                           bf16(r * norm_weight[n]) -> xnext_out[m][n]; the sum of r^2 over the outputs of one
- *                           workgroup (of one 16-row tile in the tile kernel) -> out_sumsq[m * parts + i], i < parts =
+ *                           workgroup (of one 16-row tile in the tile kernel, of one row range of a K-split launch
+ *                           of the LDS-staged kernel) -> out_sumsq[m * parts + i], i < parts =
  *                           nf4hip_gemv_norm_parts(M, N, K); what slot i holds does not depend on timing.
  *                           `out` is not written (NULL accepted).  resid_out may be resid_in.
  *   NF4HIP_EPI_ROWSCALE     x is the xnext_out of a RESID_NORM call and in_sumsq / in_parts its out_sumsq / parts:
@@ -175,7 +176,9 @@ typedef struct nf4hip_epilogue {
 /* partial sums per row of x that a RESID_NORM call on the current device writes (0: the shape is not served) */
 int nf4hip_gemv_norm_parts(int64_t M, int64_t N, int64_t K);
 /* 1 if nf4hip_gemv_epilogue takes this shape with these flags (in_parts: what a ROWSCALE call would pass, else 0),
- * 0 if it would answer NF4HIP_E_SHAPE: for callers that must know before they launch the first kernel of a chain. */
+ * 0 if it would answer NF4HIP_E_SHAPE: for callers that must know before they launch the first kernel of a chain.
+ * An epilogue is served by the kernel that serves the shape's plain product or not at all, so that the stored results
+ * are those of nf4hip_gemv followed by the step, bit for bit (ROWSCALE excepted, see above). */
 int nf4hip_gemv_epilogue_served(int64_t M, int64_t N, int64_t K, int blocksize, int flags, int in_parts);
 int nf4hip_gemv_epilogue(const void* x, int x_dtype, int64_t M, const uint8_t* packed, const float* absmax,
                          const float* lut16, const void* bias_or_null, int64_t N, int64_t K, int blocksize, void* out,

@@ -102,7 +102,12 @@ bool stage_serves(const MatmulArgs& a) {
     // 8192 (fp16 arithmetic on both sides) [4096, 14336] 14.1 / 14.5 / 14.5 / 14.8 / 15.1 / 16.2 with 1 / 4 / 5 / 8 / 9 / 16 rows
     // against 10.6 / 13.9 / 17.0 / 17.2 / 17.4 / 17.8, [8192, 14336] 18.6 / 19.3 / 19.4 / 19.6 / 21.0 / 22.4 against 16.0 / 18.6 /
     // 22.0 / 22.3 / 27.4 / 27.6.
-    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= (a.K > 8192 ? 5 : 9);
+    // Nested absmax (the other kernels resolve the 8-bit codes per lane and load): [28672, 8192] 25.8 / 27.0 / 27.9 / 29.8 / 29.4 /
+    // 31.9 with 1 / 4 / 5 / 8 / 9 / 16 rows against 29.8 / 24.5 / 29.6 / 30.6 / 50.7 / 50.0; [8192, 8192] 13.5 / 13.6 / 13.6 / 13.7 / 13.9 / 15.4
+    // against 11.6 / 11.8 / 13.9 / 14.2 / 18.5 / 18.6; without a split the lm_head 45.6 / 45.7 / 49.2 / 51.7 with 1 / 4 / 8 / 16 rows
+    // against 62.0 / 55.6 / 67.0 / 70.1, [28672, 4096] 14.6 / 14.6 / 15.1 / 17.0 against 17.5 / 15.5 / 22.1 / 24.5, [14336, 4096] 11.0 /
+    // 11.0 / 11.4 / 13.0 against 10.6 / 10.1 / 12.5 / 16.6: the same rule, from five rows on with K split.
+    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= (a.K > 8192 || a.nested.q ? 5 : 9);
     if (weights >= 100000000) return true;
     if (weights >= 40000000) return a.M >= 5;
     return weights >= ((int64_t)1 << 24) && a.M >= 9;
@@ -172,6 +177,7 @@ int gemv_kernel_for(int64_t M, int64_t N, int64_t K, int block_log2, bool nested
     a.block_log2 = block_log2;
     static const uint8_t some_codes = 0;
     a.nested.q = nested ? &some_codes : nullptr;  // (only looked at for being non-null)
+    a.nested.nested_log2 = 8;                     // (the nested blocksize of the format: 256)
     if (stage_serves(a)) return GEMV_KERNEL_STAGED;
     if (rows_serve(M, N, K)) return GEMV_KERNEL_ROWS;
     if (quad_halves_serve(M, N, K)) return GEMV_KERNEL_QUAD_HALVES;

@@ -62,6 +62,15 @@ constexpr int ABS_OFF = RING_OFF + ST_WAVES * RING_SLOTS * SLOT_BYTES;
 constexpr int ABS_BYTES = 16 * ST_WAVES * 16;  // 16 rows x 16 waves x 16 B
 constexpr int ABS_BUFS = 3;
 constexpr int ST_SMEM_BYTES = ABS_OFF + ABS_BUFS * ABS_BYTES;  // 64 + 80 + 12 = 156 KB
+// nested absmax: the same 12 KB hold three buffers of 8-bit absmax codes (16 rows x 64 bytes, rows 80 bytes apart so that
+// the sixteen rows a wave reads spread over the banks), the 256-entry map and the second-level absmax of the workgroup's
+// blocks
+constexpr int ABSQ_ROW = 80;
+constexpr int ABSQ_BYTES = 16 * ABSQ_ROW;
+constexpr int MAP_OFF = ABS_OFF + ABS_BUFS * ABSQ_BYTES;
+constexpr int AM2_OFF = MAP_OFF + 256 * 4;
+constexpr int AM2_MAX = 1024;  // second-level absmax values one workgroup may need
+static_assert(AM2_OFF + AM2_MAX * 4 <= ST_SMEM_BYTES, "the nested tables live where the fp32 absmax buffers are");
 constexpr int RED_BUF_BYTES = ST_WAVES * 1024;                 // per buffer: 16 rows of x, a plane of 16 waves x 16 weight rows x 4 B each
 static_assert(2 * RED_BUF_BYTES <= TABLE_SPAN / 2, "reduction buffers live in the table's unused half rows");
 static_assert(ST_SMEM_BYTES <= 160 * 1024, "LDS of one CU");
@@ -114,6 +123,11 @@ __device__ __forceinline__ void wait_vm() {
 }
 __device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
+// 4 bytes per active lane from a buffer straight into LDS at lds_base + lane * 4
+__device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t lane_offset, uint32_t wave_offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(uintptr_t)lds_base, 4, lane_offset, wave_offset, 0, 2 /* nt */);
+}
+
 // 16 bytes per active lane from a buffer straight into LDS at lds_base + lane * 16 (nontemporal); the byte offset is a
 // per-lane part that never changes (a register) plus a wave-uniform part (a scalar register: no vector arithmetic
 // per load)
@@ -134,11 +148,13 @@ __device__ __forceinline__ uint32_t bf16_bits_hw(float f) {
 // code book rounded to fp16, and the wave's slice of x is converted to fp16 once, every row scaled by a power of two
 // that puts its largest value of the slice just below 2^15 (exact for bf16 inputs); a wave's sums are scaled back before
 // they leave for the reduction.
-template <int MGROUPS, int EPI, bool F16 = false>
+// NESTED: absmax arrives as 8-bit codes (one byte per block, a quarter of the bytes) and is reconstructed per lane and
+// tile as map[code] * absmax2[block / nested blocksize] + offset, each rounded once, like everywhere else.
+template <int MGROUPS, int EPI, bool F16 = false, bool NESTED = false>
 __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAMS, int hot_rows_per_wg, int hot_wgs_per_split,
                                                                      int hot_splits_slices, MatmulArgs a_rest) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    const MatmulArgs a = with_hot_args<false>(a_rest, NF4_HOT_NAMES);
+    const MatmulArgs a = with_hot_args<NESTED>(a_rest, NF4_HOT_NAMES);
     const int splits = hot_splits_slices & 0xffff, slices_per_split = hot_splits_slices >> 16;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -163,8 +179,9 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
 
     const __amdgpu_buffer_rsrc_t codes_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.packed), 0, (int)(uint32_t)((int64_t)N * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t abs_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float*>(a.absmax), 0, (int)(uint32_t)((int64_t)N * (K >> 6) * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t abs_rsrc =
+        NESTED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.nested.q), 0, (int)(uint32_t)((int64_t)N * (K >> 6)), 0x00020000)
+               : __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.absmax), 0, (int)(uint32_t)((int64_t)N * (K >> 6) * 4), 0x00020000);
 
     // the two code-book values of this thread's table entry (entry tid >> 2): requested first, so that waiting for them
     // later waits for nothing that is requested after them
@@ -173,6 +190,16 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     float ssq = 0.0f;
     if ((EPI & EPI_ROWSCALE) && wave < M)
         for (int p = lane; p < a.epi.in_parts; p += 64) ssq += a.epi.in_sumsq[wave * a.epi.in_parts + p];
+    // nested absmax: this thread's entry of the map and of the workgroup's second-level absmax (blocks of the rows r0 ..
+    // r1 - 1 in this K range are consecutive per row; their second-level indices run from am2_first on)
+    const int kblocks = K >> 6;
+    const int am2_first = NESTED ? (int)(((int64_t)r0 * kblocks + slice0 * 4) >> a.nested.nested_log2) : 0;
+    float map_mine = 0.0f, am2_mine = 0.0f;
+    if (NESTED) {
+        const int am2_last = (int)(((int64_t)rmax * kblocks + (slice0 + nslices) * 4 - 1) >> a.nested.nested_log2);
+        if (tid < 256) map_mine = a.nested.map256[tid];
+        if (tid <= am2_last - am2_first) am2_mine = a.nested.absmax2[am2_first + tid];
+    }
     asm volatile("" ::: "memory");
 
     // ---- x: the A operands of the wave's eight MFMAs, loaded once -------------------------------------------------
@@ -210,9 +237,16 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     const int apiece = (lane & 15) ^ wave;
     const bool abs_lane = lane < 16 && apiece < nslices;
     const uint32_t alane = (uint32_t)(slice0 + apiece) * 16u;
+    // (nested: lane i fetches the four code bytes of slice i of the row, 64 consecutive bytes in all)
+    const bool absq_lane = lane < nslices;
+    const uint32_t aqlane = (uint32_t)(slice0 + lane) * 4u;
     auto load_absmax = [&](int t) {
         const int row = min(r0 + 16 * t + wave, rmax);
-        if (abs_lane) dma16(abs_rsrc, ABS_OFF + (t % ABS_BUFS) * ABS_BYTES + wave * 256, alane, (uint32_t)row * abs_row_bytes);
+        if (NESTED) {
+            if (absq_lane) dma4(abs_rsrc, ABS_OFF + (t % ABS_BUFS) * ABSQ_BYTES + wave * ABSQ_ROW, aqlane, (uint32_t)row * (uint32_t)kblocks);
+        } else {
+            if (abs_lane) dma16(abs_rsrc, ABS_OFF + (t % ABS_BUFS) * ABS_BYTES + wave * 256, alane, (uint32_t)row * abs_row_bytes);
+        }
     };
 
     // ---- get the stream going: absmax of tiles 0 and 1, the first five half tiles -----------------------------------
@@ -247,6 +281,10 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         write_partials(red_w0 + ((RED_BUF_BYTES >> 7) << 8), f32x4{0.f, 0.f, 0.f, 0.f});
     }
     wait_vm<RING_SLOTS>();  // everything older than the five code loads: x, code book, absmax of tiles 0 and 1
+    if (NESTED) {
+        if (tid < 256) lds_write_f32(MAP_OFF + tid * 4, map_mine);
+        lds_write_f32(AM2_OFF + tid * 4, am2_mine);
+    }
     // (x is in its registers from here on: said once, so that the loop does not carry waits for it)
 #pragma unroll
     for (int b = 0; b < 4; ++b) asm volatile("" ::"v"(xa[b][0]), "v"(xa[b][1]));
@@ -308,7 +346,10 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
             cread_wrap[b] = (c0 ^ (uint32_t)(b << 5)) + (n < 8 ? (uint32_t)((RING_SLOTS - 1) * SLOT_BYTES) : 0u);
         }
     }
-    const uint32_t aread = ABS_OFF + (uint32_t)(n * 16 + ((wave_on ? wave : 0) ^ n)) * 16u;
+    const uint32_t aread = NESTED ? ABS_OFF + (uint32_t)n * ABSQ_ROW + (uint32_t)(wave_on ? wave : 0) * 4u
+                                  : ABS_OFF + (uint32_t)(n * 16 + ((wave_on ? wave : 0) ^ n)) * 16u;
+    // nested: the lane's first block of tile 0 (its four blocks never straddle a nested block: both start at multiples of 4)
+    const uint32_t blk0 = (uint32_t)(r0 + n) * (uint32_t)kblocks + (uint32_t)slice * 4u;
     const bool reducer = wave < M;  // wave m finishes row m of x
     unsigned* counters = reinterpret_cast<unsigned*>(a.workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.workspace) + GEMV_COUNTER_BYTES);
@@ -421,12 +462,27 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         uint2 cd[4];
 #pragma unroll
         for (int b = 0; b < 4; ++b) cd[b] = S1 > S0 ? lds_read_u32x2(cread[b] + S0 * SLOT_BYTES) : lds_read_u32x2(cread_wrap[b]);
-        const float4 am4 = lds_read_f32x4(aread + (t % ABS_BUFS) * ABS_BYTES);
+        float4 am4;
+        uint32_t aq4 = 0;
+        float am2 = 0.0f;
+        if (NESTED) {
+            aq4 = lds_read_u32(aread + (t % ABS_BUFS) * ABSQ_BYTES);
+            am2 = lds_read_f32(AM2_OFF + ((((blk0 + (uint32_t)t * 16u * (uint32_t)kblocks) >> a.nested.nested_log2) - (uint32_t)am2_first) << 2));
+        } else {
+            am4 = lds_read_f32x4(aread + (t % ABS_BUFS) * ABS_BYTES);
+        }
         // the previous tile's partial sums (all written before the barrier that ended it): requested now, added up
         // between the halves of this tile
         Pending pd;
         if (!FIRST && reducer) pd = read_partials();
 
+        if (NESTED) {
+            const float off = a.nested.offset;
+            am4.x = __fadd_rn(__fmul_rn(lds_read_f32(MAP_OFF + ((aq4 & 0xffu) << 2)), am2), off);
+            am4.y = __fadd_rn(__fmul_rn(lds_read_f32(MAP_OFF + (((aq4 >> 8) & 0xffu) << 2)), am2), off);
+            am4.z = __fadd_rn(__fmul_rn(lds_read_f32(MAP_OFF + (((aq4 >> 16) & 0xffu) << 2)), am2), off);
+            am4.w = __fadd_rn(__fmul_rn(lds_read_f32(MAP_OFF + ((aq4 >> 24) << 2)), am2), off);
+        }
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         two_blocks(cd[0], cd[1], xa[0], xa[1], am4.x, am4.y, acc);
 
@@ -541,15 +597,20 @@ StagePlan make_stage_plan(int64_t N, int64_t K, int cus) {
     return p;
 }
 
-template <int MG, int EPI, bool F16 = false>
+template <int MG, int EPI, bool F16 = false, bool NESTED = false>
 hipError_t launch_mg_epi(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
-    hipLaunchKernelGGL((gemv_stage_kernel<MG, EPI, F16>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
+    hipLaunchKernelGGL((gemv_stage_kernel<MG, EPI, F16, NESTED>), dim3((unsigned)(p.wgs_per_split * p.splits)), dim3(ST_THREADS), ST_SMEM_BYTES, stream,
                        NF4_HOT_VALUES(a), p.rows_per_wg, p.wgs_per_split, p.splits | (p.slices_per_split << 16), a);
     return hipGetLastError();
 }
 
 template <int MG>
 hipError_t launch_mg(const MatmulArgs& a, const StagePlan& p, hipStream_t stream) {
+    if (a.nested.q) {
+        if (a.epi.flags != EPI_NONE) return hipErrorNotSupported;
+        return gemv_arith_mode(a.K, true) == ARITH_F16 ? launch_mg_epi<MG, EPI_NONE, true, true>(a, p, stream)
+                                                       : launch_mg_epi<MG, EPI_NONE, false, true>(a, p, stream);
+    }
     if (gemv_arith_mode(a.K, true) == ARITH_F16)
         return a.epi.flags == EPI_NONE         ? launch_mg_epi<MG, EPI_NONE, true>(a, p, stream)
                : a.epi.flags == EPI_RESID_NORM ? launch_mg_epi<MG, EPI_RESID_NORM, true>(a, p, stream)
@@ -569,6 +630,8 @@ hipError_t allow_lds_mg() {
     hipError_t e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE, false, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
+    if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_NONE, true, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_RESID_NORM, true>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_RESID_NORM>, ST_SMEM_BYTES)) != hipSuccess) return e;
     if ((e = gemv_allow_lds(gemv_stage_kernel<MG, EPI_ROWSCALE>, ST_SMEM_BYTES)) != hipSuccess) return e;
@@ -582,8 +645,18 @@ hipError_t allow_lds_mg() {
 // 16384 every weight would have to be rounded like the dequantised one), N a multiple of 8 (loads fetch eight whole rows),
 // offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up) pairs (even N)
 // while K is not split over workgroups, the residual step only where it is.
+// second-level absmax values a workgroup of the plan may need (nested absmax)
+static int64_t stage_am2_count(const MatmulArgs& a, const StagePlan& p) {
+    const int64_t blocks = (int64_t)p.rows_per_wg * (a.K >> 6);  // from the first block of its first row to the last of its last
+    return (blocks >> a.nested.nested_log2) + 2;
+}
+
 bool gemv_stage_possible(const MatmulArgs& a) {
-    if (a.nested.q || a.block_log2 != 6) return false;
+    if (a.block_log2 != 6) return false;
+    // nested absmax: plain calls; a lane's four blocks must share one second-level value; the workgroup's values fit
+    // their table (judged on the plan for 256 CUs; a launch on fewer checks again)
+    if (a.nested.q && (a.epi.flags != EPI_NONE || a.nested.nested_log2 < 2 || stage_am2_count(a, make_stage_plan(a.N, a.K, 256)) > AM2_MAX))
+        return false;
     if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 16384 || a.N % 8) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
@@ -617,6 +690,7 @@ hipError_t gemv_stage_setup() {
 hipError_t launch_gemv_stage(const MatmulArgs& a, int cus, hipStream_t stream) {
     if (!gemv_stage_possible(a)) return hipErrorNotSupported;
     const StagePlan p = make_stage_plan(a.N, a.K, cus);
+    if (a.nested.q && stage_am2_count(a, p) > AM2_MAX) return hipErrorNotSupported;
     switch ((a.M + 3) / 4) {
         case 1: return launch_mg<1>(a, p, stream);
         case 2: return launch_mg<2>(a, p, stream);

@@ -72,7 +72,7 @@ def test_gemv_plan_names_the_kernel(ta):
     assert kernel(16, 4096, 14336) == (5, 1)
     assert kernel(1, 28672, 8192) == (1, 0) and kernel(8, 28672, 8192)[0] != 5 and kernel(16, 28672, 8192) == (5, 0)
     assert kernel(16, 4096, 16384 + 512)[0] == 4
-    assert kernel(1, 128256, 4096, nested=1)[0] == 1  # nested absmax never goes to the staged kernel
+    assert kernel(1, 128256, 4096, nested=1)[0] == 5 and kernel(5, 28672, 8192, nested=1) == (5, 0)  # nested absmax too
     assert lib.nf4hip_gemv_prefer_staged(0) == 0
     assert kernel(1, 128256, 4096)[0] == 1
     assert lib.nf4hip_gemv_prefer_staged(-1) == 0

@@ -557,18 +557,18 @@ def test_llama70b_shapes_double_quant(ta, N, K):
         ref = x.double() @ deq[rows].double().t()
         torch.testing.assert_close(y[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
         if M <= 16:
-            # bit for bit the same kernel's result on the reconstructed fp32 absmax (the LDS-staged kernel, which may
-            # serve fp32 absmax at these shapes, takes no nested absmax and adds in another order: held off for the
-            # comparison, then checked against the same reference by itself)
+            # bit for bit the same kernel's result on the reconstructed fp32 absmax: with the LDS-staged kernel wherever it
+            # applies and with it held off (the library's own rule may send the two forms of absmax to different kernels)
             lib = ta._lib.load()
-            assert lib.nf4hip_gemv_prefer_staged(0) == 0
-            try:
-                y2 = ta.matmul_nf4(x, qw, None, absmax_rec, code, 64, torch.bfloat16, (N, K))
-            finally:
-                assert lib.nf4hip_gemv_prefer_staged(-1) == 0
-            assert torch.equal(y, y2)
-            y3 = ta.matmul_nf4(x, qw, None, absmax_rec, code, 64, torch.bfloat16, (N, K))
-            torch.testing.assert_close(y3[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
+            for mode in (1, 0):
+                assert lib.nf4hip_gemv_prefer_staged(mode) == 0
+                try:
+                    y3 = ta.matmul_nf4(x, qw, None, nested, code, 64, torch.bfloat16, (N, K))
+                    y4 = ta.matmul_nf4(x, qw, None, absmax_rec, code, 64, torch.bfloat16, (N, K))
+                finally:
+                    assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+                assert torch.equal(y3, y4), f"nested and reconstructed absmax differ, M = {M}, staged mode {mode}"
+                torch.testing.assert_close(y3[:, rows].double(), ref, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("N,K", [(28672, 4096), (128256, 4096), (16384 + 16, 4096)])

@@ -83,6 +83,30 @@ def test_staged_kernel_short_and_split_k(ta, oracle, staged, M, N, K):
     _run(ta, staged, oracle, M, N, K, seed=3 * M + N + K, bias=(K == 6144), reps=3)
 
 
+# nested (8-bit) absmax: against the same kernel on the reconstructed fp32 absmax, bit for bit (the reconstruction is the
+# same two roundings either way), and against the oracle like every other case
+@pytest.mark.parametrize("M", [1, 6, 16])
+@pytest.mark.parametrize("N,K", [(1000, 4096), (2048, 1024), (4096, 8192), (1032, 14336), (640, 9216)])
+def test_staged_kernel_nested_absmax(ta, oracle, staged, M, N, K):
+    import ctypes
+
+    print(f"staged gemv, nested absmax M={M} N={N} K={K}", flush=True)
+    plan = (ctypes.c_int * 4)()
+    assert staged.nf4hip_gemv_plan(M, N, K, 64, 1, ctypes.byref(plan)) == 0 and plan[0] == 5
+    g = torch.Generator().manual_seed(11 * M + N + K)
+    # rows of very different magnitude, so that the second-level absmax matters
+    w = (torch.randn(N, K, generator=g) * 0.02 * torch.logspace(-2, 0, N).unsqueeze(1)).to(torch.bfloat16)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    qw, absmax, code = ta.quantize_nf4(w.to(DEV))
+    nested = ta.compress_absmax(absmax)
+    rec = ta.reconstruct_absmax(nested)
+    y = ta.matmul_nf4(x.to(DEV), qw, None, nested, code, 64, torch.bfloat16, (N, K))
+    y_rec = ta.matmul_nf4(x.to(DEV), qw, None, rec, code, 64, torch.bfloat16, (N, K))
+    assert torch.equal(y.view(torch.int16), y_rec.view(torch.int16))
+    deq = oracle.C().dequantize(qw.cpu(), rec.cpu(), oracle.nf4_lut(), 64, torch.bfloat16, (N, K)).double()
+    torch.testing.assert_close(y.cpu().double(), x.double() @ deq.t(), rtol=2e-2, atol=2e-2)
+
+
 def test_staged_kernel_many_launches_are_bit_stable(ta, oracle, staged):
     """[4096, 8192] and [4096, 14336], sixteen rows of x: K is split over two / four workgroups per row range, whichever
     arrives last adds the partial sums in range order -- 200 launches on one workspace must give one result."""

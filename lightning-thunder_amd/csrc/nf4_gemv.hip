@@ -107,7 +107,10 @@ bool stage_serves(const MatmulArgs& a) {
     // against 11.6 / 11.8 / 13.9 / 14.2 / 18.5 / 18.6; without a split the lm_head 45.6 / 45.7 / 49.2 / 51.7 with 1 / 4 / 8 / 16 rows
     // against 62.0 / 55.6 / 67.0 / 70.1, [28672, 4096] 14.6 / 14.6 / 15.1 / 17.0 against 17.5 / 15.5 / 22.1 / 24.5, [14336, 4096] 11.0 /
     // 11.0 / 11.4 / 13.0 against 10.6 / 10.1 / 12.5 / 16.6: the same rule, from five rows on with K split.
-    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= (a.K > 8192 || a.nested.q ? 5 : 9);
+    // Other shapes, fp32 absmax, staged vs the other kernels with 5 / 8 / 9 / 16 rows: [10240, 8192] 14.2 / 14.7 / 14.9 / 16.7 vs
+    // 15.1 / 15.9 / 22.7 / 23.2; [57344, 8192] 52.8 / 53.6 / 54.4 / 60.2 vs 58.7 / 58.4 / 63.7 / 63.6 (1..4 rows: 49-52 vs 45-46);
+    // [13824, 5120] 16.1 / 16.7 / 16.8 / 18.5 vs 15.7 / 16.5 / 18.8 / 19.1; [5120, 5120] (26 M weights) loses at every M.
+    if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= 5;
     if (weights >= 100000000) return true;
     if (weights >= 40000000) return a.M >= 5;
     return weights >= ((int64_t)1 << 24) && a.M >= 9;

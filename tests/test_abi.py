@@ -66,11 +66,11 @@ def test_gemv_plan_names_the_kernel(ta):
     assert lib.nf4hip_gemv_prefer_staged(-1) == 0
     assert kernel(1, 4096, 4096) == (1, 0) and kernel(4, 4096, 4096) == (2, 0) and kernel(16, 1024, 4096) == (3, 0)
     assert kernel(1, 128256, 4096) == (5, 0) and kernel(16, 14336, 4096) == (5, 0) and kernel(4, 14336, 4096) == (2, 0)
-    # K beyond one workgroup's sixteen slices: the staged kernel splits K over workgroups, from 9 rows of x on (from 5
-    # beyond K = 8192, in fp16 arithmetic)
+    # K beyond one workgroup's sixteen slices: the staged kernel splits K over workgroups, from 5 rows of x on (in fp16
+    # arithmetic beyond K = 8192)
     assert kernel(1, 4096, 14336) == (1, 1) and kernel(4, 4096, 14336)[0] == 2 and kernel(5, 4096, 14336) == (5, 1)
     assert kernel(16, 4096, 14336) == (5, 1)
-    assert kernel(1, 28672, 8192) == (1, 0) and kernel(8, 28672, 8192)[0] != 5 and kernel(16, 28672, 8192) == (5, 0)
+    assert kernel(1, 28672, 8192) == (1, 0) and kernel(4, 28672, 8192)[0] != 5 and kernel(5, 28672, 8192) == (5, 0)
     assert kernel(16, 4096, 16384 + 512)[0] == 4
     assert kernel(1, 128256, 4096, nested=1)[0] == 5 and kernel(5, 28672, 8192, nested=1) == (5, 0)  # nested absmax too
     assert lib.nf4hip_gemv_prefer_staged(0) == 0
@@ -275,7 +275,8 @@ def test_epilogue_argument_errors(ta):
     assert call(L.Epilogue(L.EPI_SILU_PAIRS), long_k) == L.E_SHAPE and "not served" in err()
     assert call(L.Epilogue(L.EPI_ROWSCALE, 1e-5, A, 513)) == L.E_SHAPE  # more partial sums than a workgroup has threads
     assert lib.nf4hip_gemv_norm_parts(16, 16384, 4096) == 0 and lib.nf4hip_gemv_norm_parts(1, 64, 20480) == 0
-    assert lib.nf4hip_gemv_norm_parts(8, 8192, 8192) == 512
+    assert lib.nf4hip_gemv_norm_parts(4, 8192, 28672) > 0
+    assert lib.nf4hip_gemv_norm_parts(8, 8192, 8192) == 128  # staged kernel, K split two ways: 128 row ranges
     assert lib.nf4hip_gemv_norm_parts(16, 8192, 4096) == 0  # the product alone goes to the staged kernel, which has no residual epilogue
     assert lib.nf4hip_gemv_norm_parts(3, 64, 4096) > 0
     assert lib.nf4hip_gemv_norm_parts(8, 4096, 14336) == 64  # staged kernel, K split four ways: one partial sum per row range

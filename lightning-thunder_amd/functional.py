@@ -414,20 +414,33 @@ def _fused_gemm_wins(M: int, N: int, K: int, nested: bool = False) -> bool:
     return _wide_gemm_us(M, N, K) * (1.25 if nested else 1.0) <= 1.03 * _dense_gemm_us(M, N, K)
 
 
-def _chunked_gemv_wins(M: int, N: int, K: int) -> bool:
+def _gemv_pass_us(N: int, K: int, nested: bool = False) -> float:
+    """Model of one 16-row pass of the decode kernels over a weight of W million elements, from measurements on MI355X
+    (us): the LDS-staged kernel 7.6 + 0.09 W while one workgroup covers K ([14336, 4096] 12.9, [28672, 4096] 17.6,
+    [32000, 4096] 18.5, lm_head [128256, 4096] 54.7) and 9.5 + 0.108 W with K split over workgroups ([4096, 14336] 16.8,
+    [10240, 8192] 17.0, [28672, 8192] 33.8, [57344, 8192] 60.3); the other decode kernels 12 + 0.105 W.  Which kernel it is, the
+    library says (nf4hip_gemv_plan, no GPU needed)."""
+    w = N * K / 1e6
+    plan = (ctypes.c_int * 4)()
+    if _lib.load().nf4hip_gemv_plan(16, N, K, 64, 1 if nested else 0, ctypes.byref(plan)) == 0 and plan[0] == 5:
+        return 7.6 + 0.09 * w if K <= 4096 else 9.5 + 0.108 * w
+    return 12.0 + 0.105 * w
+
+
+def _chunked_gemv_wins(M: int, N: int, K: int, nested: bool = False) -> bool:
     """For a few more than 16 rows of x: are ceil(M / 16) passes of the decode kernel over the NF4
     weight cheaper than the alternatives?  All sides modelled from measurements on MI355X
-    (microseconds, W = weights in millions): a 16-row pass takes 12 + 0.105 W; the dense route
+    (microseconds, W = weights in millions): a 16-row pass takes _gemv_pass_us; the dense route
     20 + 0.62 W before its GEMM, and the passes must beat that by 20 %; the fused GEMM kernel, where
-    it applies, _fused_gemm_us.  [28672, 8192]: up to M = 32 (73 us vs 90 fused); [28672, 4096]: up to
-    M = 32 (a tie: 49 vs 45-50); lm_head [128256, 4096]: never (134 vs 121 at M = 32); [14336, 4096]: up to
-    M = 32 (36 vs 55 dense); [16384, 8192]: up to M = 48; below 40 M weights never."""
+    it applies, _fused_gemm_us.  Measured, passes vs fused GEMM, M = 32 / 48: [28672, 4096] 34.8 / 51.6 vs 43.6 / 40.2;
+    lm_head [128256, 4096] 115.7 / 166.5 vs 124.5 / 126.9; [4096, 14336] 32.6 / 47.4 vs 34.2 / 34.3; [14336, 4096] 24.6 / 36.6 vs
+    26.5 / 26.8; [28672, 8192] 66.4 / 98.1 vs 68.1 / 67.6; [6144, 4096] 18.6 / 27.3 vs 19.4 / 19.8: two passes win, three do not;
+    below 40 M weights never."""
     n_weights = N * K
     if M <= 16 or n_weights < 40_000_000:
         return False
-    w = n_weights / 1e6
     passes = (M + 15) // 16
-    t = passes * (12.0 + 0.105 * w)
+    t = passes * _gemv_pass_us(N, K, nested)
     if _fused_gemm_wins(M, N, K) and t >= _fused_gemm_us(M, N, K):
         return False
     return t < 0.8 * _dense_route_us(N, K)
@@ -512,7 +525,7 @@ def fused_route(x: torch.Tensor, bias, blocksize: int, dtype: torch.dtype, shape
         return "dequant+linear"
     if M <= 16 and K % 512 == 0:
         return "gemv"  # MFMA tile kernel (its exact-weights variant beyond EXACT_K)
-    if K % 512 == 0 and _chunked_gemv_wins(M, N, K):
+    if K % 512 == 0 and _chunked_gemv_wins(M, N, K, nested):
         return "gemv-chunks"  # a few 16-row passes over the 4-bit weights beat writing them out as bf16
     measured = _route_measured.get(_route_key(x.device, M, N, K, blocksize, nested, bias is not None))
     if measured is not None:

@@ -219,7 +219,11 @@ def test_fused_route_rules(ta):
     # modelled faster than the dense route's dequantize pass -- every projection shape of the Llama models
     assert route(17, 4096, 4096) == "gemm" and route(128, 4096, 4096) == "gemm"
     assert route(64, 1024, 4096) == "gemm" and route(65, 1024, 4096) == "dequant+gemm"
-    assert route(17, 14336, 4096) == "gemm" and route(128, 14336, 4096) == "gemm"
+    # 17..32 rows of x on a weight of 40 M elements and more: two passes of the decode kernel (the LDS-staged one at these
+    # shapes) beat the fused GEMM; three do not
+    assert route(17, 14336, 4096) == "gemv-chunks" and route(32, 28672, 4096) == "gemv-chunks" and route(32, 128256, 4096) == "gemv-chunks"
+    assert route(33, 14336, 4096) == "gemm" and route(48, 28672, 4096) == "gemm" and route(128, 14336, 4096) == "gemm"
+    assert route(17, 6144, 4096) == "gemm" and route(32, 4096, 4096) == "gemm"  # below 40 M weights never
     assert route(128, 4096, 14336) == "gemm"
     assert route(17, 8192, 28672) == "gemm"               # exact at any K
     assert route(17, 28672, 4096 + 64) == "gemm"          # the tile kernel needs K % 512, the fused GEMM K % 64

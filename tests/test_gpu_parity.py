@@ -363,7 +363,7 @@ def fused_gemm(ta, monkeypatch):
     """Route every M > 16 call to the fused GEMM kernel (the default router prefers HIP dequantize
     + the dense library GEMM from 17 rows on)."""
     monkeypatch.setattr(ta.functional, "DENSE_ROUTE_MIN_M", 1 << 30)
-    monkeypatch.setattr(ta.functional, "_chunked_gemv_wins", lambda M, N, K: False)
+    monkeypatch.setattr(ta.functional, "_chunked_gemv_wins", lambda M, N, K, nested=False: False)
 
 
 @pytest.mark.parametrize("M,N,K", [(200, 128, 4096), (129, 1024, 4096), (3000, 1024, 4096)])

@@ -83,13 +83,13 @@ int stage_mode() {
     return m;
 }
 
-// The dispatcher's own rule, from interleaved timings of both sides (us, staged vs the other kernels, one to sixteen
-// rows of x): lm_head [128256, 4096] 47.8 / 49.7 / 53.4 / 60.2 vs 52.4 / 57.7 / 60.9 / 60.8 at M = 1 / 4 / 8 / 16;
-// [28672, 4096] 14.9 / 15.4 / 16.2 / 18.4 vs 15.5 / 15.8 / 20.4 / 23.5; [14336, 4096] 11.2 / 11.5 / 11.9 / 13.6 vs 10.2 /
-// 10.2 / 12.8 / 16.5; [6144, 4096] 8.0 / 8.3 / 8.7 / 10.1 vs 6.7 / 7.0 / 8.4 / 11.8; [4096, 4096] 6.7 / 7.1 / 7.6 / 8.4 vs
-// 5.1 / 6.3 / 7.5 / 9.3; [1024, 4096] 6.2 / 6.7 / 7.4 / 8.4 vs 4.1 / 4.5 / 5.1 / 6.5.  The staged kernel streams faster and
-// starts more slowly (a workgroup of sixteen waves, a barrier behind the table build): every weight of a hundred
-// million elements or more, from five rows of x on beyond forty million, from nine rows on beyond 2^24.
+// The dispatcher's own rule, from interleaved timings of both sides (us, staged vs the other kernels, 1 / 4 / 8 / 16 rows
+// of x): lm_head [128256, 4096] 47.6 / 48.5 / 49.2 / 54.6 vs 52.4 / 57.7 / 60.9 / 60.8; [28672, 4096] 14.8 / 15.0 / 15.8 / 17.2 vs
+// 15.8 / 16.0 / 21.0 / 24.0; [14336, 4096] 11.1 / 11.3 / 11.5 / 12.8 vs 10.3 / 10.2 / 12.8 / 16.9; [6144, 4096] 7.8 / 8.0 / 8.7 / 9.7 vs
+// 6.7 / 7.0 / 8.5 / 11.8; [4096, 4096] 6.2 / 6.5 / 7.1 / 8.1 vs 5.1 / 6.3 / 7.7 / 9.4; [1024, 4096] 5.7 / 6.1 / 6.7 / 7.6 vs 4.1 / 4.6 / 5.1 /
+// 6.6.  The staged kernel streams faster and starts more slowly (its first tile needs the first requests of all sixteen
+// waves): every weight of a hundred million elements or more, from five rows of x on beyond forty million, from nine
+// rows on beyond 2^24.
 bool stage_serves(const MatmulArgs& a) {
     const int mode = stage_mode();
     if (mode == 0 || !gemv_stage_possible(a)) return false;

@@ -409,9 +409,9 @@ def _fused_gemm_wins(M: int, N: int, K: int, nested: bool = False) -> bool:
     which needs no transient bf16 weight."""
     if M <= 128:
         return _fused_gemm_us(M, N, K) < _dense_route_us(N, K)
-    # nested absmax: the fused kernel resolves an 8-bit code through two more look-ups per block and k step and runs
-    # 15-30 % longer ([8192, 8192] 2048 rows: 275 vs 235 us; [8192, 28672]: 1045 vs 784), the dequantize pass hardly does
-    return _wide_gemm_us(M, N, K) * (1.25 if nested else 1.0) <= 1.03 * _dense_gemm_us(M, N, K)
+    # nested absmax: the fp32 absmax is written out ahead of the fused kernel (_matmul_nf4_on), 2-7 % on top; the
+    # dequantize pass of the dense route resolves the codes itself at no measurable cost
+    return _wide_gemm_us(M, N, K) * (1.05 if nested else 1.0) <= 1.03 * _dense_gemm_us(M, N, K)
 
 
 def _gemv_pass_us(N: int, K: int, nested: bool = False) -> float:
@@ -562,6 +562,12 @@ def matmul_nf4(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape) -> 
     return _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, route)
 
 
+# nested absmax, fused GEMM: beyond this many rows of x the fp32 absmax is written out first (measured, us, nested kernel /
+# reconstruct + fp32 kernel / fp32 kernel alone: [8192, 8192] M = 256 64 / 58 / 53, M = 512 107 / 91 / 85, M = 2048 255 / 242 / 235;
+# [28672, 8192] M = 512 242 / 226 / 213, M = 2048 930 / 854 / 837; [8192, 28672] M = 1024 481 / 439 / 425; [1024, 8192] M = 512 38 / 37 / 34)
+NESTED_RECONSTRUCT_MIN_M = 128
+
+
 def _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape, route: str) -> torch.Tensor:
     """:func:`matmul_nf4` on a given route (one of ``fused_route``'s answers)."""
     N, K = shape
@@ -597,6 +603,11 @@ def _matmul_nf4_on(x, qweight, bias, absmax, quant_map, blocksize, dtype, shape,
         # row chunks of x and out: one call, or 16 rows at a time (rows are contiguous, K and N even,
         # so every chunk starts 16-byte aligned when the whole does and K, N are multiples of 8)
         step = 16 if route == "gemv-chunks" else M
+        if isinstance(absmax, NestedAbsmax) and route == "gemm" and M > NESTED_RECONSTRUCT_MIN_M:
+            # Many rows of x on nested absmax: the fused GEMM resolves an 8-bit code through two more loads per block and
+            # k step and runs 5-27 % longer than on fp32 absmax; writing the fp32 absmax out first (nf4hip_dq_reconstruct,
+            # 4 bytes per block into a transient buffer, 4-15 us) costs 2-7 %.  Same two roundings, same bits.
+            absmax = reconstruct_absmax(absmax)
         if isinstance(absmax, NestedAbsmax):
             q, a2, m256, off, nbs = _nested_args(absmax, nblocks)
             for m0 in range(0, M, step):

@@ -107,6 +107,38 @@ def test_staged_kernel_nested_absmax(ta, oracle, staged, M, N, K):
     torch.testing.assert_close(y.cpu().double(), x.double() @ deq.t(), rtol=2e-2, atol=2e-2)
 
 
+def _random_cases(count, seed):
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(count):
+        K = 256 * rnd.choice([1, 2, 3, 5, 8, 15, 16, 17, 20, 24, 31, 32, 33, 40, 47, 48, 49, 56, 63, 64])
+        N = 8 * rnd.randint(1, 160 if K <= 8192 else 80)
+        cases.append((rnd.randint(1, 16), N, K, rnd.random() < 0.4, rnd.random() < 0.3))
+    return cases
+
+
+@pytest.mark.parametrize("M,N,K,nested,bias", _random_cases(36, 20240611))
+def test_staged_kernel_random_shapes(ta, oracle, staged, M, N, K, nested, bias):
+    """Random (M, N, K) inside the kernel's rules -- every number of K ranges (1..4), last ranges with fewer slices than the
+    others, row ranges that end in a half tile, fp32 and nested absmax, with and without bias -- against the oracle."""
+    print(f"staged gemv, random case M={M} N={N} K={K} nested={nested} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    b = (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16) if bias else None
+    qw, absmax, code = ta.quantize_nf4(w.to(DEV))
+    state = ta.compress_absmax(absmax) if nested else absmax
+    rec = ta.reconstruct_absmax(state) if nested else absmax
+    y = ta.matmul_nf4(x.to(DEV), qw, None if b is None else b.to(DEV), state, code, 64, torch.bfloat16, (N, K))
+    deq = oracle.C().dequantize(qw.cpu(), rec.cpu(), oracle.nf4_lut(), 64, torch.bfloat16, (N, K)).double()
+    ref = x.double() @ deq.t()
+    if bias:
+        ref = ref + b.double()
+    torch.testing.assert_close(y.cpu().double(), ref, rtol=2e-2, atol=2e-2)
+
+
 def test_staged_kernel_many_launches_are_bit_stable(ta, oracle, staged):
     """[4096, 8192] and [4096, 14336], sixteen rows of x: K is split over two / four workgroups per row range, whichever
     arrives last adds the partial sums in range order -- 200 launches on one workspace must give one result."""

@@ -103,6 +103,36 @@ def test_resid_norm_epilogue(ta, F, M, shape):
     torch.testing.assert_close(sumsq.double().sum(-1), r_ref.double().pow(2).sum(-1), rtol=1e-5, atol=0)
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("shape", [(520, 8192), (1032, 14336), (256, 16384), (4096, 8192)])
+def test_resid_norm_epilogue_of_the_staged_kernel(ta, F, M, shape):
+    """The LDS-staged kernel forced (``nf4hip_gemv_prefer_staged(1)``) on shapes whose K it splits over workgroups: the
+    workgroup that adds the K ranges does the residual step -- bit for bit what the plain call of the same kernel and
+    the step by itself store, one partial sum of squares per row range."""
+    N, K = shape
+    lib = ta._lib.load()
+    print(f"staged resid_norm M={M} N={N} K={K}", flush=True)
+    qw, absmax, code = _quantized(ta, N, K, seed=N + K + 2)
+    x = _randn((M, K), seed=3 * N + M).to(DEV)
+    resid = _randn((M, N), seed=5 * N + M, std=2.0).to(DEV)
+    nw = (1.0 + _randn((N,), seed=N + 3, std=0.1).float()).to(torch.bfloat16).to(DEV)
+    bias = _randn((N,), seed=N + 4, std=0.5).to(DEV) if N == 520 else None
+    assert lib.nf4hip_gemv_prefer_staged(1) == 0
+    try:
+        assert _served(F, M, N, K, resid_norm=True)
+        got = F.matmul_nf4_epilogue(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw))
+        delta = F.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))
+        parts = lib.nf4hip_gemv_norm_parts(M, N, K)
+    finally:
+        assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+    assert got is not None
+    r, xnext, sumsq = got
+    r_ref = (resid.float() + delta.float()).to(torch.bfloat16)
+    assert torch.equal(_bits(r), _bits(r_ref)) and torch.equal(_bits(xnext), _bits((r_ref.float() * nw.float()).to(torch.bfloat16)))
+    assert sumsq.shape == (M, parts) and parts > 0
+    torch.testing.assert_close(sumsq.double().sum(-1), r_ref.double().pow(2).sum(-1), rtol=1e-5, atol=0)
+
+
 def _deq(oracle, qw, absmax, code, shape):
     return oracle.dequantize_4bit_eager(qw.cpu(), absmax.cpu(), code.cpu(), 64, torch.bfloat16, shape).double()
 

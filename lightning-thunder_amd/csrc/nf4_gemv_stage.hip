@@ -61,7 +61,11 @@ constexpr int RING_OFF = TABLE_SPAN;
 constexpr int ABS_OFF = RING_OFF + ST_WAVES * RING_SLOTS * SLOT_BYTES;
 constexpr int ABS_BYTES = 16 * ST_WAVES * 16;  // 16 rows x 16 waves x 16 B
 constexpr int ABS_BUFS = 3;
-constexpr int ST_SMEM_BYTES = ABS_OFF + ABS_BUFS * ABS_BYTES;  // 64 + 80 + 12 = 156 KB
+// bias of the workgroup's rows (bf16), fetched once: a load into a register inside the tile loop would have the compiler
+// wait for every load of the ring behind it
+constexpr int BIAS_OFF = ABS_OFF + ABS_BUFS * ABS_BYTES;
+constexpr int BIAS_ROWS = 1024;
+constexpr int ST_SMEM_BYTES = BIAS_OFF + BIAS_ROWS * 2;  // 64 + 80 + 12 + 2 = 158 KB
 // nested absmax: the same 12 KB hold three buffers of 8-bit absmax codes (16 rows x 64 bytes, rows 80 bytes apart so that
 // the sixteen rows a wave reads spread over the banks), the 256-entry map and the second-level absmax of the workgroup's
 // blocks
@@ -70,7 +74,7 @@ constexpr int ABSQ_BYTES = 16 * ABSQ_ROW;
 constexpr int MAP_OFF = ABS_OFF + ABS_BUFS * ABSQ_BYTES;
 constexpr int AM2_OFF = MAP_OFF + 256 * 4;
 constexpr int AM2_MAX = 1024;  // second-level absmax values one workgroup may need
-static_assert(AM2_OFF + AM2_MAX * 4 <= ST_SMEM_BYTES, "the nested tables live where the fp32 absmax buffers are");
+static_assert(AM2_OFF + AM2_MAX * 4 <= BIAS_OFF, "the nested tables live where the fp32 absmax buffers are");
 constexpr int RED_BUF_BYTES = ST_WAVES * 1024;                 // per buffer: 16 rows of x, a plane of 16 waves x 16 weight rows x 4 B each
 static_assert(2 * RED_BUF_BYTES <= TABLE_SPAN / 2, "reduction buffers live in the table's unused half rows");
 static_assert(ST_SMEM_BYTES <= 160 * 1024, "LDS of one CU");
@@ -87,6 +91,10 @@ __device__ __forceinline__ uint32_t red_addr(uint32_t o) { return ((o >> 7) << 8
 
 __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
     typedef __attribute__((address_space(3))) const uint32_t* p_t;
+    return *reinterpret_cast<p_t>((uintptr_t)addr);
+}
+__device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr) {
+    typedef __attribute__((address_space(3))) const uint16_t* p_t;
     return *reinterpret_cast<p_t>((uintptr_t)addr);
 }
 __device__ __forceinline__ float lds_read_f32(uint32_t addr) {
@@ -183,7 +191,15 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         NESTED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.nested.q), 0, (int)(uint32_t)((int64_t)N * (K >> 6)), 0x00020000)
                : __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.absmax), 0, (int)(uint32_t)((int64_t)N * (K >> 6) * 4), 0x00020000);
 
-    // the two code-book values of this thread's table entry (entry tid >> 2): requested first, so that waiting for them
+    // bias of this workgroup's rows into LDS, 128 rows per wave: the oldest request of the wave, so no count below
+    // changes with it (reads past the end of the bias return zeros; those rows are never stored).  Where K is split
+    // the workgroup that adds the ranges reads the bias from memory after its last tile.
+    const bool bias_staged = a.bias && splits == 1;
+    if (bias_staged && wave * 128 < r1 - r0) {
+        const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.bias), 0, (int)(2 * N), 0x00020000);
+        dma4(bias_rsrc, BIAS_OFF + wave * 256, (uint32_t)(r0 + wave * 128) * 2u + (uint32_t)lane * 4u, 0);
+    }
+    // the two code-book values of this thread's table entry (entry tid >> 2): requested next, so that waiting for them
     // later waits for nothing that is requested after them
     const float lut_hi = a.lut16[tid >> 6], lut_lo = a.lut16[(tid >> 2) & 15];
     // EPI_ROWSCALE: wave m's share of the partial sums of squares of row m of x (at most 512: eight per lane)
@@ -362,12 +378,19 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     uint32_t red_r = red_addr((uint32_t)wave * 1024u + (uint32_t)((16 * g + n) ^ (((wave >> 2) & 1) << 4)) * 4u);
     struct Pending {
         float p[4];
+        uint32_t bias;  // of row r0 + 16 t + n, bf16 bits
     };
+    uint32_t bias_r = BIAS_OFF + (uint32_t)n * 2u;
     auto read_partials = [&]() {  // of the oldest tile not yet finished
         Pending pd;
 #pragma unroll
         for (int q = 0; q < 4; ++q) pd.p[q] = lds_read_f32(red_r + (uint32_t)q * 512u);
         red_r ^= RED_FLIP;
+        pd.bias = 0;
+        if (bias_staged) {
+            pd.bias = lds_read_u16(bias_r);
+            bias_r += 32;
+        }
         return pd;
     };
     // where row r0 + n of this workgroup sits in row m of the output, in bytes; stores go through a buffer that ends
@@ -392,10 +415,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         if (splits == 1) {
             const uint32_t at = out_lane + 32u * (uint32_t)t;  // byte offset of row r0 + 16 t + n
             if (EPI & EPI_ROWSCALE) sum *= rstd;
-            if (a.bias) {
-                const int row = r0 + 16 * t + n;
-                if (row < r1) sum += bf16_bits_to_f32(a.bias[row]);
-            }
+            if (a.bias) sum += bf16_bits_to_f32((uint16_t)pd.bias);
             if (EPI & EPI_SILU_PAIRS) {
                 // rows 2j, 2j + 1 = gate j, up j: the even row's lane takes the odd row's value (lane ^ 1)
                 const float mine = nf4x::round_bf16(sum);
@@ -660,6 +680,9 @@ bool gemv_stage_possible(const MatmulArgs& a) {
     if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 16384 || a.N % 8) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
+    // a bias is staged in LDS by 4-byte loads, BIAS_ROWS rows per workgroup (judged like the nested tables)
+    if (a.bias && splits == 1 && ((reinterpret_cast<uintptr_t>(a.bias) & 3u) || make_stage_plan(a.N, a.K, 256).rows_per_wg > BIAS_ROWS))
+        return false;
     if (a.epi.flags == EPI_RESID_NORM) {
         if (splits == 1) return false;  // (the workgroup that adds the K ranges does the residual step; one K range has no such place)
     } else if (a.epi.flags != EPI_NONE) {
@@ -691,6 +714,7 @@ hipError_t launch_gemv_stage(const MatmulArgs& a, int cus, hipStream_t stream) {
     if (!gemv_stage_possible(a)) return hipErrorNotSupported;
     const StagePlan p = make_stage_plan(a.N, a.K, cus);
     if (a.nested.q && stage_am2_count(a, p) > AM2_MAX) return hipErrorNotSupported;
+    if (a.bias && p.splits == 1 && p.rows_per_wg > BIAS_ROWS) return hipErrorNotSupported;
     switch ((a.M + 3) / 4) {
         case 1: return launch_mg<1>(a, p, stream);
         case 2: return launch_mg<2>(a, p, stream);

@@ -199,13 +199,18 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.bias), 0, (int)(2 * N), 0x00020000);
         dma4(bias_rsrc, BIAS_OFF + wave * 256, (uint32_t)(r0 + wave * 128) * 2u + (uint32_t)lane * 4u, 0);
     }
+    // EPI_ROWSCALE: wave m's share of the partial sums of squares of row m of x (at most 512: eight per lane), all
+    // requested here and added up after the first barrier (a loop that adds as it loads waits for a round trip per
+    // 64 partial sums before the wave's first weight request: 1.8 us of a launch whose producer had 512 workgroups)
+    float ssp[8];
+    if (EPI & EPI_ROWSCALE) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            ssp[j] = (wave < M && lane + 64 * j < a.epi.in_parts) ? a.epi.in_sumsq[wave * a.epi.in_parts + lane + 64 * j] : 0.0f;
+    }
     // the two code-book values of this thread's table entry (entry tid >> 2): requested next, so that waiting for them
     // later waits for nothing that is requested after them
     const float lut_hi = a.lut16[tid >> 6], lut_lo = a.lut16[(tid >> 2) & 15];
-    // EPI_ROWSCALE: wave m's share of the partial sums of squares of row m of x (at most 512: eight per lane)
-    float ssq = 0.0f;
-    if ((EPI & EPI_ROWSCALE) && wave < M)
-        for (int p = lane; p < a.epi.in_parts; p += 64) ssq += a.epi.in_sumsq[wave * a.epi.in_parts + p];
     // nested absmax: this thread's entry of the map and of the workgroup's second-level absmax (blocks of the rows r0 ..
     // r1 - 1 in this K range are consecutive per row; their second-level indices run from am2_first on)
     const int kblocks = K >> 6;
@@ -342,6 +347,9 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
 
     float rstd = 1.0f;  // EPI_ROWSCALE: 1 / rms of row `wave` of the producer's residual stream
     if (EPI & EPI_ROWSCALE) {
+        float ssq = ssp[0];  // (sums of squares: 0 + ssp[0] has the same bits, and no addition is left where the load is)
+#pragma unroll
+        for (int j = 1; j < 8; ++j) ssq += ssp[j];
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o, 64);
         rstd = rsqrtf(ssq / (float)K + a.epi.eps);

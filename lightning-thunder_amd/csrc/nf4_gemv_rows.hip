@@ -236,7 +236,12 @@ __global__ __launch_bounds__(GEMV_THREADS, 4) void gemv_rows_kernel(NF4_HOT_PARA
             if (NESTED && tid < 256) reinterpret_cast<float*>(smem + MAP_OFFSET)[tid] = a.nested.map256[tid];
             table_built = true;
         }
-        if (EPI & EPI_RESID_NORM) pre_s[tid] = pre_res | (pre_w << 16);  // a slot per thread, read back by the same thread
+        if (EPI & EPI_RESID_NORM) {
+            // (the two values are first looked at here: without this the compiler moves the shift up to the loads, and the
+            // wait for them in front of the requests for x and the weights)
+            asm volatile("" : "+v"(pre_res), "+v"(pre_w));
+            pre_s[tid] = pre_res | (pre_w << 16);  // a slot per thread, read back by the same thread
+        }
         __syncthreads();  // table built (first task) / previous task's epilogue done with `part`
 
         // fp16 arithmetic: the lane's x values become fp16, scaled into range per row of x (here, behind the requests for

@@ -6,6 +6,7 @@
 // exist so that the decode-step harness is bound by the NF4 kernels rather than by ~18 small
 // launches per layer.  bf16 in and out, fp32 arithmetic.  C ABI: include/nf4hip_decode.h.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -191,34 +192,49 @@ __global__ __launch_bounds__(ATTN_THREADS) void attention_decode_kernel(const ui
 #pragma unroll
     for (int i = 0; i < 16; ++i) qv[i] = q_s[sub * 16 + i];
     float mx = -INFINITY;
-    for (int s0 = lo; s0 < hi; s0 += 4 * KPI) {
-        uint4 ka[4], kb[4];
+    // U keys per lane under way at a time.  A round of requests is a round trip to memory, so with few workgroups per
+    // CU (one sequence: 256 workgroups) a workgroup takes as few rounds as its keys need -- eight keys per lane, 256 a
+    // round.  With four workgroups per CU the CU's address unit is what the passes wait for, and a round wider than
+    // the keys left costs requests for clamped addresses: four per lane there.  The order of the additions does not
+    // depend on the width.
+    const bool wide = gridDim.x <= 512;
+    auto score_pass = [&](auto u_tag) {
+        constexpr int U = decltype(u_tag)::value;
+        for (int s0 = lo; s0 < hi; s0 += U * KPI) {
+            uint4 ka[U], kb[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int s = min(s0 + u * KPI + kslot, hi - 1);
-            const uint4* kp = reinterpret_cast<const uint4*>(kc + (int64_t)s * HD + sub * 16);
-            ka[u] = kp[0];
-            kb[u] = kp[1];
-        }
+            for (int u = 0; u < U; ++u) {
+                const int s = min(s0 + u * KPI + kslot, hi - 1);
+                const uint4* kp = reinterpret_cast<const uint4*>(kc + (int64_t)s * HD + sub * 16);
+                ka[u] = kp[0];
+                kb[u] = kp[1];
+            }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int s = s0 + u * KPI + kslot;
-            float a8[8], b8[8];
-            unpack8(ka[u], a8);
-            unpack8(kb[u], b8);
-            float dot = 0.0f;
+            for (int u = 0; u < U; ++u) {
+                const int s = s0 + u * KPI + kslot;
+                float a8[8], b8[8];
+                unpack8(ka[u], a8);
+                unpack8(kb[u], b8);
+                float dot = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) dot = fmaf(qv[i], a8[i], dot);
+                for (int i = 0; i < 8; ++i) dot = fmaf(qv[i], a8[i], dot);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) dot = fmaf(qv[8 + i], b8[i], dot);
+                for (int i = 0; i < 8; ++i) dot = fmaf(qv[8 + i], b8[i], dot);
 #pragma unroll
-            for (int o = 1; o < LPK; o <<= 1) dot += __shfl_xor(dot, o, 64);
-            if (s < hi) {
-                if (sub == 0) p_s[s] = dot;
-                mx = fmaxf(mx, dot);
+                for (int o = 1; o < LPK; o <<= 1) dot += __shfl_xor(dot, o, 64);
+                if (s < hi) {
+                    if (sub == 0) p_s[s] = dot;
+                    mx = fmaxf(mx, dot);
+                }
             }
         }
-    }
+    };
+    if (hi - lo <= 2 * KPI)
+        score_pass(std::integral_constant<int, 2>{});
+    else if (hi - lo <= 4 * KPI || !wide)
+        score_pass(std::integral_constant<int, 4>{});
+    else
+        score_pass(std::integral_constant<int, 8>{});
     if (has_new) {  // the new key, from LDS
         float dot = 0.0f;
 #pragma unroll
@@ -246,23 +262,33 @@ __global__ __launch_bounds__(ATTN_THREADS) void attention_decode_kernel(const ui
     // values: thread = (key group sg, 8 columns dg); four cached rows per thread in flight
     const int dg = tid % DG, sg = tid / DG;
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int s0 = lo + sg; s0 < hi; s0 += 4 * SG) {
-        uint4 vv[4];
-        float w[4];
+    // (rows per thread under way: as for the keys; a thread adds its rows in the same order whatever the width)
+    auto value_pass = [&](auto u_tag) {
+        constexpr int U = decltype(u_tag)::value;
+        for (int s0 = lo + sg; s0 < hi; s0 += U * SG) {
+            uint4 vv[U];
+            float w[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int s = s0 + u * SG;
-            vv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)min(s, hi - 1) * HD + dg * 8);
-            w[u] = s < hi ? p_s[s] : 0.0f;
+            for (int u = 0; u < U; ++u) {
+                const int s = s0 + u * SG;
+                vv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)min(s, hi - 1) * HD + dg * 8);
+                w[u] = s < hi ? p_s[s] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float vf[8];
+                unpack8(vv[u], vf);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = fmaf(w[u], vf[i], o[i]);
+            }
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            float vf[8];
-            unpack8(vv[u], vf);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = fmaf(w[u], vf[i], o[i]);
-        }
-    }
+    };
+    if (hi - lo <= 4 * SG || !wide)
+        value_pass(std::integral_constant<int, 4>{});
+    else if (hi - lo <= 8 * SG)
+        value_pass(std::integral_constant<int, 8>{});
+    else
+        value_pass(std::integral_constant<int, 12>{});
     if (sg == 0 && has_new) {  // the new value, from LDS
         const float w = p_s[p];
 #pragma unroll

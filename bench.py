@@ -54,8 +54,10 @@ def algorithmic_bytes(M: int, N: int, K: int) -> int:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # (defaults: a timed region of ~55 ms behind ~15 ms of the same work; the first few milliseconds after an idle
+    # GPU run 15-20 % slower -- clocks, first touch of every weight copy -- and a 5 + 20 step run measures mostly that)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU baseline sample (0 disables)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-regime section (BASELINE config 3) and the quantize/dequantize bandwidth section")
     ap.add_argument("--decode-tokens", type=int, default=128,

@@ -33,7 +33,7 @@ def _intact(raw, nbytes):
     return bool((raw[:GUARD] == SENTINEL).all()) and bool((raw[GUARD + nbytes:] == SENTINEL).all())
 
 
-def _run(ta, lib, oracle, M, N, K, seed, bias=False, reps=1):
+def _run(ta, lib, oracle, M, N, K, seed, bias=False, reps=1, bias_shift=0):
     L = ta._lib
     g = torch.Generator().manual_seed(seed)
     w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
@@ -41,7 +41,8 @@ def _run(ta, lib, oracle, M, N, K, seed, bias=False, reps=1):
     b = (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16) if bias else None
     qw, absmax, code = ta.quantize_nf4(w.to(DEV))
     xd = x.to(DEV)
-    bd = b.to(DEV) if bias else None
+    # (bias_shift = 1: the bias starts two bytes into its allocation, i.e. at an address that is not a multiple of four)
+    bd = torch.cat([torch.zeros(bias_shift, dtype=torch.bfloat16), b]).to(DEV)[bias_shift:] if bias else None
     need = lib.nf4hip_gemv_workspace_bytes(M, N, K)
     ws_raw, ws = _guarded(max(need, 256), fill=0)
     out_raw, out = _guarded(M * N * 2)
@@ -137,6 +138,17 @@ def test_staged_kernel_random_shapes(ta, oracle, staged, M, N, K, nested, bias):
     if bias:
         ref = ref + b.double()
     torch.testing.assert_close(y.cpu().double(), ref, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("M", [1, 16])
+def test_staged_kernel_bias(ta, oracle, staged, M):
+    """The bias of a workgroup's rows is staged in LDS, 128 rows per wave: workgroups with one, two and eight waves' worth
+    of rows, a last workgroup that ends inside a wave's 128 rows, and K split over workgroups (the bias is added by
+    the workgroup that adds the K ranges).  A bias at an address that is no multiple of four, or more than 1024 rows
+    per workgroup, is left to the other kernels: same result contract."""
+    for (N, K, shift) in [(4096, 4096, 0), (40000, 512, 0), (262144 - 8, 512, 0), (1000, 8192, 0), (4096, 4096, 1), (262144 + 4096, 512, 0)]:
+        print(f"staged gemv with bias M={M} N={N} K={K} shift={shift}", flush=True)
+        _run(ta, staged, oracle, M, N, K, seed=N + K + M, bias=True, bias_shift=shift)
 
 
 def test_staged_kernel_many_launches_are_bit_stable(ta, oracle, staged):

@@ -76,7 +76,7 @@ int stage_mode() {
     int m = g_stage_mode.load(std::memory_order_relaxed);
     if (m == -2) {
         const char* v = getenv("NF4HIP_STAGE");
-        m = v ? atoi(v) : -1;
+        m = (v && *v) ? atoi(v) : -1;  // (set but empty counts as not set)
         if (m < -1 || m > 1) m = -1;
         g_stage_mode.store(m, std::memory_order_relaxed);
     }

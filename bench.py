@@ -60,9 +60,13 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU baseline sample (0 disables)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-regime section (BASELINE config 3) and the quantize/dequantize bandwidth section")
+    ap.add_argument("--section-warm-seconds", type=float, default=0.08,
+                    help="warm-up ahead of every timing of the prefill / double-quant / codec sections (0: three calls, for counter runs)")
     ap.add_argument("--decode-tokens", type=int, default=128,
                     help="tokens of the Llama-3-8B greedy decode that follows the GEMV pass (0 disables)")
     args = ap.parse_args()
+    global SECTION_WARM_SECONDS
+    SECTION_WARM_SECONDS = args.section_warm_seconds
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only; --gpus {args.gpus} is not supported "
               "(the path would shard like a dense linear: by rows of W for q/k/v/gate/up/lm_head, by columns for o/down)", file=sys.stderr)
@@ -345,11 +349,23 @@ def main() -> int:
 MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CUs x 2.4 GHz x 4096 flop/clk/CU
 
 
-def _timed(torch, fn, reps, warm=3):
-    """Seconds per call: the median of three event-bracketed batches of ``reps`` calls after ``warm`` untimed ones."""
-    for _ in range(warm):
-        fn()
-    torch.cuda.synchronize()
+SECTION_WARM_SECONDS = 0.08  # (--section-warm-seconds)
+
+
+def _timed(torch, fn, reps, warm=3, warm_seconds=None):
+    """Seconds per call: the median of three event-bracketed batches of ``reps`` calls after at least ``warm`` untimed
+    ones and ``warm_seconds`` of them.  (Every case of the sections below starts on a GPU that sat idle while the
+    host drew its inputs; for tens of milliseconds after that the same kernel runs 10-15 % slower -- a 250 us GEMM
+    39 % of the MFMA peak after three calls, 41 % after thirty, 44 % after three hundred -- and three calls measured
+    that, not the kernel.)"""
+    if warm_seconds is None:
+        warm_seconds = SECTION_WARM_SECONDS
+    t0, n = time.perf_counter(), 0
+    while n < warm or time.perf_counter() - t0 < warm_seconds:
+        for _ in range(max(1, reps)):
+            fn()
+        torch.cuda.synchronize()
+        n += max(1, reps)
     per = []
     for _ in range(3):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -373,7 +389,7 @@ def prefill_section(torch, ta) -> dict:
     nf4hip_dequantize + the hand-written dense MFMA kernel (nf4hip_linear), and nf4hip_dequantize + the vendor
     library's GEMM -- and ``router_pick`` marks the one ``matmul_nf4`` picks (it times all three on its first call of a
     shape; the library has to win by more than 3 %).  TFLOP/s = 2 M N K / time against the bf16 MFMA peak; HIP events
-    bracket 10 calls (4 beyond 4 TFLOP per call) after 3 warm-up calls.  ``dense_kernel_alone``: nf4hip_linear and the
+    bracket 10 calls (4 beyond 4 TFLOP per call) after 80 ms of warm-up calls.  ``dense_kernel_alone``: nf4hip_linear and the
     library GEMM on the already dequantized weight.
     ``rows64``: the same weights with 64 rows of x (fused kernel with K split over workgroups vs the dense route)."""
     dev = torch.device("cuda:0")
@@ -514,9 +530,13 @@ def codec_section(torch, ta) -> dict:
         torch.cuda.synchronize()
 
         def timed(fn, reps=2 * ncopy):
-            for i in range(ncopy):
-                fn(i)
-            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            while True:  # (as in _timed: past the slow first milliseconds after an idle GPU)
+                for i in range(ncopy):
+                    fn(i)
+                torch.cuda.synchronize()
+                if time.perf_counter() - t0 >= SECTION_WARM_SECONDS:
+                    break
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for i in range(reps):

@@ -150,8 +150,8 @@ int nf4hip_gemv_dq(const void* x, int x_dtype, int64_t M, const uint8_t* packed,
  *                           -- what SiLU(gate) * up on the bf16 output of nf4hip_gemv gives, bit for bit.
  *   NF4HIP_EPI_RESID_NORM   d = bf16(sum[m][n] + bias[n]); r = bf16(resid_in[m][n] + d) -> resid_out[m][n];
  *                           bf16(r * norm_weight[n]) -> xnext_out[m][n]; the sum of r^2 over the outputs of one
- *                           workgroup (of one 16-row tile in the tile kernel, of one row range of a K-split launch
- *                           of the LDS-staged kernel) -> out_sumsq[m * parts + i], i < parts =
+ *                           workgroup (of one 16-row tile in the tile kernel, of one row range of a launch of the
+ *                           LDS-staged kernel) -> out_sumsq[m * parts + i], i < parts =
  *                           nf4hip_gemv_norm_parts(M, N, K); what slot i holds does not depend on timing.
  *                           `out` is not written (NULL accepted).  resid_out may be resid_in.
  *   NF4HIP_EPI_ROWSCALE     x is the xnext_out of a RESID_NORM call and in_sumsq / in_parts its out_sumsq / parts:

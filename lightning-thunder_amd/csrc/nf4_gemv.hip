@@ -156,14 +156,14 @@ int gemv_norm_parts(int64_t M, int64_t N, int64_t K) {
     int cus = 256;
     if (device_setup(&cus) != hipSuccess) cus = 256;
     {
-        // where the product by itself goes to the staged kernel, so does the residual epilogue, which that kernel only has
-        // with K split over workgroups (gemv_epilogue_possible)
+        // where the product by itself goes to the staged kernel, so does the residual epilogue (gemv_epilogue_possible),
+        // which that kernel has with K split over workgroups and, for few rows per workgroup, with one K range
         MatmulArgs plain{};
         plain.M = (int)M;
         plain.N = (int)N;
         plain.K = (int)K;
         plain.block_log2 = 6;
-        if (stage_serves(plain)) return gemv_stage_norm_parts(N, K, cus);
+        if (stage_serves(plain)) return gemv_stage_norm_parts(M, N, K, cus);
     }
     if (rows_serve(M, N, K)) return gemv_rows_norm_parts(M, N, K, cus);
     if (quad_halves_serve(M, N, K)) return gemv_quad_norm_parts(M, N, K, cus, true);

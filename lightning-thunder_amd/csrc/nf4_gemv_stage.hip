@@ -65,7 +65,12 @@ constexpr int ABS_BUFS = 3;
 // wait for every load of the ring behind it
 constexpr int BIAS_OFF = ABS_OFF + ABS_BUFS * ABS_BYTES;
 constexpr int BIAS_ROWS = 1024;
-constexpr int ST_SMEM_BYTES = BIAS_OFF + BIAS_ROWS * 2;  // 64 + 80 + 12 + 2 = 158 KB
+// EPI_RESID_NORM while one workgroup covers K: the residual of the workgroup's outputs (M rows of x times its weight rows)
+// and the norm weight of its rows, bf16, fetched once like the bias: at most RESID_SLOTS values, (M + 1) * rows
+constexpr int RESID_OFF = BIAS_OFF + BIAS_ROWS * 2;
+constexpr int RESID_SLOTS = 1024;
+constexpr int RESID_MAX_ROWS = 128;  // (one 4-byte-per-lane request of a wave covers a row of x: 64 lanes x 2 values)
+constexpr int ST_SMEM_BYTES = RESID_OFF + RESID_SLOTS * 2;  // 64 + 80 + 12 + 2 + 2 = 160 KB
 // nested absmax: the same 12 KB hold three buffers of 8-bit absmax codes (16 rows x 64 bytes, rows 80 bytes apart so that
 // the sixteen rows a wave reads spread over the banks), the 256-entry map and the second-level absmax of the workgroup's
 // blocks
@@ -207,6 +212,22 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             ssp[j] = (wave < M && lane + 64 * j < a.epi.in_parts) ? a.epi.in_sumsq[wave * a.epi.in_parts + lane + 64 * j] : 0.0f;
+    }
+    // EPI_RESID_NORM with one K range: wave m fetches the residual of row m of x for the workgroup's rows, wave 0 the
+    // norm weight of those rows as well (row M of the staging area); rows past the tensors read as zeros or as the
+    // next row's values and are never stored
+    const int rpw = hot_rows_per_wg;
+    const bool resid_staged = (EPI & EPI_RESID_NORM) && splits == 1;
+    if (resid_staged) {
+        const uint32_t lane2 = (uint32_t)lane * 4u;
+        if (wave < M && 2 * lane < rpw) {
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.epi.resid_in), 0, (int)(2 * M * N), 0x00020000);
+            dma4(rs, RESID_OFF + wave * rpw * 2, (uint32_t)(wave * N + r0) * 2u + lane2, 0);
+        }
+        if (wave == 0 && 2 * lane < rpw) {
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.epi.norm_weight), 0, (int)(2 * N), 0x00020000);
+            dma4(rs, RESID_OFF + M * rpw * 2, (uint32_t)r0 * 2u + lane2, 0);
+        }
     }
     // the two code-book values of this thread's table entry (entry tid >> 2): requested next, so that waiting for them
     // later waits for nothing that is requested after them
@@ -386,9 +407,12 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     uint32_t red_r = red_addr((uint32_t)wave * 1024u + (uint32_t)((16 * g + n) ^ (((wave >> 2) & 1) << 4)) * 4u);
     struct Pending {
         float p[4];
-        uint32_t bias;  // of row r0 + 16 t + n, bf16 bits
+        uint32_t bias;         // of row r0 + 16 t + n, bf16 bits
+        uint32_t resid, normw;  // EPI_RESID_NORM, one K range: residual of (row m of x, that row) and the row's norm weight
     };
     uint32_t bias_r = BIAS_OFF + (uint32_t)n * 2u;
+    uint32_t resid_r = RESID_OFF + (uint32_t)(min(wave, M - 1) * rpw + n) * 2u;
+    uint32_t normw_r = RESID_OFF + (uint32_t)(M * rpw + n) * 2u;
     auto read_partials = [&]() {  // of the oldest tile not yet finished
         Pending pd;
 #pragma unroll
@@ -399,6 +423,13 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
             pd.bias = lds_read_u16(bias_r);
             bias_r += 32;
         }
+        pd.resid = pd.normw = 0;
+        if (resid_staged) {
+            pd.resid = lds_read_u16(resid_r);
+            pd.normw = lds_read_u16(normw_r);
+            resid_r += 32;
+            normw_r += 32;
+        }
         return pd;
     };
     // where row r0 + n of this workgroup sits in row m of the output, in bytes; stores go through a buffer that ends
@@ -407,6 +438,12 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
     const bool pairs = (EPI & EPI_SILU_PAIRS) != 0;
     const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         a.out + (int64_t)(reducer ? wave : 0) * (pairs ? (N >> 1) : N), 0, pairs ? r1 : 2 * r1, 0x00020000);
+    // (EPI_RESID_NORM, one K range: the two tensors the epilogue stores instead of `out`, same rows, same range check)
+    const __amdgpu_buffer_rsrc_t resid_out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        ((EPI & EPI_RESID_NORM) ? a.epi.resid_out : a.out) + (int64_t)(reducer ? wave : 0) * N, 0, 2 * r1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xnext_out_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        ((EPI & EPI_RESID_NORM) ? a.epi.xnext_out : a.out) + (int64_t)(reducer ? wave : 0) * N, 0, 2 * r1, 0x00020000);
+    float resid_ss = 0.0f;  // sum of squares of the new residual over this lane's rows (lanes 0..15 of wave m: row m of x)
     // ... adds them in that order, then the four lane groups (two register swaps across the wave: no LDS round trip),
     // and stores the 16 outputs
     auto finish_tile = [&](int t, const Pending& pd) {
@@ -424,6 +461,17 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
             const uint32_t at = out_lane + 32u * (uint32_t)t;  // byte offset of row r0 + 16 t + n
             if (EPI & EPI_ROWSCALE) sum *= rstd;
             if (a.bias) sum += bf16_bits_to_f32((uint16_t)pd.bias);
+            if (EPI & EPI_RESID_NORM) {
+                // d = bf16(sum + bias); r = bf16(resid + d) -> resid_out; bf16(r * w_next) -> xnext_out; r^2 into the
+                // workgroup's share of row m's sum of squares
+                const float d = nf4x::round_bf16(sum);
+                const float res = nf4x::resid_add(bf16_bits_to_f32(pd.resid), d);
+                if (g == 0) {
+                    __builtin_amdgcn_raw_buffer_store_b16((short)f32_to_bf16_bits(res), resid_out_rsrc, at, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b16((short)f32_to_bf16_bits(res * bf16_bits_to_f32(pd.normw)), xnext_out_rsrc, at, 0, 0);
+                    if (r0 + 16 * t + n < r1) resid_ss = fmaf(res, res, resid_ss);
+                }
+            } else
             if (EPI & EPI_SILU_PAIRS) {
                 // rows 2j, 2j + 1 = gate j, up j: the even row's lane takes the odd row's value (lane ^ 1)
                 const float mine = nf4x::round_bf16(sum);
@@ -555,6 +603,12 @@ __global__ __launch_bounds__(ST_THREADS, 1) void gemv_stage_kernel(NF4_HOT_PARAM
         if (t + 4 < tiles) tile_body(t + 4, I0{}, I1{}, std::false_type{});
     }
     if (reducer) finish_tile(tiles - 1, read_partials());
+    if (resid_staged && reducer) {
+        // lanes 0..15 hold the rows n, n + 16, ... of the workgroup: added in a fixed order, one slot per workgroup
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) resid_ss += __shfl_xor(resid_ss, o, 64);
+        if (lane == 0) a.epi.out_sumsq[wave * hot_wgs_per_split + part] = resid_ss;
+    }
     wait_vm<0>();  // loads issued past the end of the range still target this workgroup's LDS
     if (splits > 1) {
         // The workgroups that share these rows (one per K range) count their arrival once all their partial sums have
@@ -672,7 +726,8 @@ hipError_t allow_lds_mg() {
 // What the kernel takes: fp32 absmax, blocksize 64, K a multiple of 256 up to 16384 (fp16 arithmetic beyond 8192; beyond
 // 16384 every weight would have to be rounded like the dequantised one), N a multiple of 8 (loads fetch eight whole rows),
 // offsets that fit 32 bits; of the epilogues the row scale (at most 512 partial sums) and the (gate, up) pairs (even N)
-// while K is not split over workgroups, the residual step only where it is.
+// while K is not split over workgroups, the residual step where it is and, with one K range, where a workgroup has
+// at most 128 weight rows and (M + 1) times as many values fit the 2 KB they are staged in.
 // second-level absmax values a workgroup of the plan may need (nested absmax)
 static int64_t stage_am2_count(const MatmulArgs& a, const StagePlan& p) {
     const int64_t blocks = (int64_t)p.rows_per_wg * (a.K >> 6);  // from the first block of its first row to the last of its last
@@ -692,7 +747,13 @@ bool gemv_stage_possible(const MatmulArgs& a) {
     if (a.bias && splits == 1 && ((reinterpret_cast<uintptr_t>(a.bias) & 3u) || make_stage_plan(a.N, a.K, 256).rows_per_wg > BIAS_ROWS))
         return false;
     if (a.epi.flags == EPI_RESID_NORM) {
-        if (splits == 1) return false;  // (the workgroup that adds the K ranges does the residual step; one K range has no such place)
+        // K split: the workgroup that adds the K ranges does the residual step.  One K range: the finishing waves do,
+        // on a residual staged in LDS -- a row of x per request, (M + 1) rows of values in all
+        if (splits == 1) {
+            const int rows = make_stage_plan(a.N, a.K, 256).rows_per_wg;
+            if (rows > RESID_MAX_ROWS || (a.M + 1) * rows > RESID_SLOTS) return false;
+            if ((reinterpret_cast<uintptr_t>(a.epi.resid_in) | reinterpret_cast<uintptr_t>(a.epi.norm_weight)) & 3u) return false;
+        }
     } else if (a.epi.flags != EPI_NONE) {
         if ((a.epi.flags & ~(EPI_ROWSCALE | EPI_SILU_PAIRS)) || splits != 1) return false;
         if ((a.epi.flags & EPI_ROWSCALE) && a.epi.in_parts > 512) return false;
@@ -703,7 +764,16 @@ bool gemv_stage_possible(const MatmulArgs& a) {
 
 int gemv_stage_splits(int64_t K) { return stage_splits(K); }
 
-int gemv_stage_norm_parts(int64_t N, int64_t K, int cus) { return stage_splits(K) > 1 ? make_stage_plan(N, K, cus).wgs_per_split : 0; }
+// EPI_RESID_NORM: partial sums of squares per row of x = the row ranges of the plan (0: no residual epilogue for this shape)
+int gemv_stage_norm_parts(int64_t M, int64_t N, int64_t K, int cus) {
+    if (stage_splits(K) == 1) {
+        const int rows = make_stage_plan(N, K, 256).rows_per_wg;
+        if (rows > RESID_MAX_ROWS || (M + 1) * rows > RESID_SLOTS) return 0;
+        const int rows_here = make_stage_plan(N, K, cus).rows_per_wg;
+        if (rows_here > RESID_MAX_ROWS || (M + 1) * rows_here > RESID_SLOTS) return 0;
+    }
+    return make_stage_plan(N, K, cus).wgs_per_split;
+}
 
 size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int s = stage_splits(K);
@@ -723,6 +793,8 @@ hipError_t launch_gemv_stage(const MatmulArgs& a, int cus, hipStream_t stream) {
     const StagePlan p = make_stage_plan(a.N, a.K, cus);
     if (a.nested.q && stage_am2_count(a, p) > AM2_MAX) return hipErrorNotSupported;
     if (a.bias && p.splits == 1 && p.rows_per_wg > BIAS_ROWS) return hipErrorNotSupported;
+    if (a.epi.flags == EPI_RESID_NORM && p.splits == 1 && (p.rows_per_wg > RESID_MAX_ROWS || (a.M + 1) * p.rows_per_wg > RESID_SLOTS))
+        return hipErrorNotSupported;
     switch ((a.M + 3) / 4) {
         case 1: return launch_mg<1>(a, p, stream);
         case 2: return launch_mg<2>(a, p, stream);

@@ -281,7 +281,10 @@ def test_epilogue_argument_errors(ta):
     assert lib.nf4hip_gemv_norm_parts(16, 16384, 4096) == 0 and lib.nf4hip_gemv_norm_parts(1, 64, 20480) == 0
     assert lib.nf4hip_gemv_norm_parts(4, 8192, 28672) > 0
     assert lib.nf4hip_gemv_norm_parts(8, 8192, 8192) == 128  # staged kernel, K split two ways: 128 row ranges
-    assert lib.nf4hip_gemv_norm_parts(16, 8192, 4096) == 0  # the product alone goes to the staged kernel, which has no residual epilogue
+    # the product alone goes to the staged kernel, one K range: its residual epilogue holds (M + 1) x rows per workgroup
+    # values in LDS, at most 1024 -- 17 x 32 here, one partial sum per workgroup; 17 x 64 on twice the rows is too many
+    assert lib.nf4hip_gemv_norm_parts(16, 8192, 4096) == 256
+    assert lib.nf4hip_gemv_norm_parts(16, 16384, 4096) == 0 and lib.nf4hip_gemv_norm_parts(9, 16384, 4096) == 256
     assert lib.nf4hip_gemv_norm_parts(3, 64, 4096) > 0
     assert lib.nf4hip_gemv_norm_parts(8, 4096, 14336) == 64  # staged kernel, K split four ways: one partial sum per row range
 

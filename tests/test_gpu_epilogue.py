@@ -133,6 +133,58 @@ def test_resid_norm_epilogue_of_the_staged_kernel(ta, F, M, shape):
     torch.testing.assert_close(sumsq.double().sum(-1), r_ref.double().pow(2).sum(-1), rtol=1e-5, atol=0)
 
 
+@pytest.mark.parametrize("M,shape", [(1, (4096, 4096)), (9, (4096, 4096)), (16, (4096, 4096)), (16, (14336, 4096)), (8, (28672, 4096)),
+                                     (16, (1000, 2048)), (5, (8, 512)), (16, (2040, 4096))])
+def test_resid_norm_epilogue_of_the_staged_kernel_one_k_range(ta, F, M, shape):
+    """The same where one workgroup covers K: the finishing waves do the residual step on a residual and norm weight
+    staged in LDS -- few rows per workgroup, (M + 1) rows of values in all -- and leave one partial sum of squares per
+    workgroup.  With sixteen rows of x the output projection of the decode step takes this route by the dispatcher's
+    own rule."""
+    N, K = shape
+    lib = ta._lib.load()
+    print(f"staged resid_norm, one K range M={M} N={N} K={K}", flush=True)
+    qw, absmax, code = _quantized(ta, N, K, seed=N + K + 5)
+    x = _randn((M, K), seed=3 * N + M + 1).to(DEV)
+    resid = _randn((M, N), seed=5 * N + M + 1, std=2.0).to(DEV)
+    nw = (1.0 + _randn((N,), seed=N + 6, std=0.1).float()).to(torch.bfloat16).to(DEV)
+    bias = _randn((N,), seed=N + 7, std=0.5).to(DEV) if N in (1000, 14336) else None
+    assert lib.nf4hip_gemv_prefer_staged(1) == 0
+    try:
+        import ctypes
+
+        plan = (ctypes.c_int * 4)()
+        assert lib.nf4hip_gemv_plan(M, N, K, 64, 0, ctypes.byref(plan)) == 0 and plan[0] == 5, "the staged kernel serves the plain product"
+        assert _served(F, M, N, K, resid_norm=True)
+        got = F.matmul_nf4_epilogue(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw))
+        delta = F.matmul_nf4(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K))
+        parts = lib.nf4hip_gemv_norm_parts(M, N, K)
+    finally:
+        assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+    assert got is not None
+    r, xnext, sumsq = got
+    r_ref = (resid.float() + delta.float()).to(torch.bfloat16)
+    assert torch.equal(_bits(r), _bits(r_ref)) and torch.equal(_bits(xnext), _bits((r_ref.float() * nw.float()).to(torch.bfloat16)))
+    assert sumsq.shape == (M, parts) and parts > 0
+    torch.testing.assert_close(sumsq.double().sum(-1), r_ref.double().pow(2).sum(-1), rtol=1e-5, atol=0)
+    # the same call again on the same buffers: the same bits (nothing depends on which workgroup finishes first)
+    assert lib.nf4hip_gemv_prefer_staged(1) == 0
+    try:
+        again = F.matmul_nf4_epilogue(x, qw, bias, absmax, code, 64, torch.bfloat16, (N, K), resid_norm=(resid, nw))
+    finally:
+        assert lib.nf4hip_gemv_prefer_staged(-1) == 0
+    assert all(torch.equal(a_.view(torch.int16) if a_.dtype == torch.bfloat16 else a_, b_.view(torch.int16) if b_.dtype == torch.bfloat16 else b_)
+               for a_, b_ in zip(again, got))
+
+
+def test_resid_norm_epilogue_too_many_rows_for_the_staging(ta, F):
+    """[28672, 4096] with sixteen rows of x: 112 weight rows per workgroup times seventeen rows of values do not fit
+    the staging area; the staged kernel serves the plain product, so the epilogue form is refused (the caller's
+    two-step route adds to the same sums)."""
+    lib = ta._lib.load()
+    assert lib.nf4hip_gemv_norm_parts(16, 28672, 4096) == 0
+    assert not _served(F, 16, 28672, 4096, resid_norm=True)
+
+
 def _deq(oracle, qw, absmax, code, shape):
     return oracle.dequantize_4bit_eager(qw.cpu(), absmax.cpu(), code.cpu(), 64, torch.bfloat16, shape).double()
 

@@ -89,7 +89,7 @@ int stage_mode() {
 // 6.7 / 7.0 / 8.5 / 11.8; [4096, 4096] 6.2 / 6.5 / 7.1 / 8.1 vs 5.1 / 6.3 / 7.7 / 9.4; [1024, 4096] 5.7 / 6.1 / 6.7 / 7.6 vs 4.1 / 4.6 / 5.1 /
 // 6.6.  The staged kernel streams faster and starts more slowly (its first tile needs the first requests of all sixteen
 // waves): every weight of a hundred million elements or more, from five rows of x on beyond forty million, from nine
-// rows on beyond 2^24.
+// rows on beyond 2^24 (from five where a workgroup's rows are whole tiles).
 bool stage_serves(const MatmulArgs& a) {
     const int mode = stage_mode();
     if (mode == 0 || !gemv_stage_possible(a)) return false;
@@ -113,7 +113,13 @@ bool stage_serves(const MatmulArgs& a) {
     if (gemv_stage_splits(a.K) > 1) return weights >= ((int64_t)1 << 25) && a.M >= 5;
     if (weights >= 100000000) return true;
     if (weights >= 40000000) return a.M >= 5;
-    return weights >= ((int64_t)1 << 24) && a.M >= 9;
+    if (weights < ((int64_t)1 << 24)) return false;
+    if (a.M >= 9) return true;
+    // 5..8 rows of x: where every workgroup has whole 16-row tiles and all sixteen waves a slice of K -- [4096, 4096]
+    // 6.7 / 6.9 / 7.4 us with 5 / 6 / 8 rows against 7.4 / 7.6 / 7.8, [8192, 4096] 8.9 / 8.8 / 9.0 against 9.3 / 9.3 / 9.6; with a
+    // half-filled last tile per workgroup [6144, 4096] 8.4 / 8.5 / 8.9 against 8.2 / 8.4 / 8.5, [5120, 4096] 8.2 / 8.2 / 8.6 against
+    // 7.9 / 8.2 / 8.4
+    return a.M >= 5 && a.K == 4096 && a.N % (256 * 16) == 0;
 }
 
 }  // namespace

@@ -202,6 +202,7 @@ bool gemv_stage_possible(const MatmulArgs& a);
 size_t gemv_stage_workspace_bytes(int64_t M, int64_t N, int64_t K);
 enum : int { GEMV_KERNEL_ROWS = 1, GEMV_KERNEL_QUAD = 2, GEMV_KERNEL_QUAD_HALVES = 3, GEMV_KERNEL_TILES = 4, GEMV_KERNEL_STAGED = 5 };
 int gemv_kernel_for(int64_t M, int64_t N, int64_t K, int block_log2, bool nested);
+int gemv_plan_cus();  // CU count of the current device, 256 where there is none: what launch plans are judged on
 int gemv_stage_norm_parts(int64_t M, int64_t N, int64_t K, int cus);  // EPI_RESID_NORM: partial sums per row of x (0: not served)
 int gemv_stage_splits(int64_t K);  // K ranges of the staged kernel: 1 while the sixteen waves of a workgroup cover K (4096)
 hipError_t gemv_stage_setup();

@@ -126,6 +126,15 @@ bool stage_serves(const MatmulArgs& a) {
 
 // ---- dispatch -------------------------------------------------------------------------------
 
+// The CU count the launch plans are made for: the current device's, or 256 (the part this library is written for)
+// where no device answers -- what the "is this served" answers are judged on, so that they agree with the launch.
+int gemv_plan_cus() {
+    int cus = 256;
+    if (device_setup(&cus) != hipSuccess) cus = 256;
+    return cus;
+}
+
+
 void gemv_set_staged(int mode) { g_stage_mode.store(mode < -1 || mode > 1 ? -1 : mode, std::memory_order_relaxed); }
 
 size_t gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {

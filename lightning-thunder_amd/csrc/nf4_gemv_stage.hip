@@ -737,20 +737,20 @@ static int64_t stage_am2_count(const MatmulArgs& a, const StagePlan& p) {
 bool gemv_stage_possible(const MatmulArgs& a) {
     if (a.block_log2 != 6) return false;
     // nested absmax: plain calls; a lane's four blocks must share one second-level value; the workgroup's values fit
-    // their table (judged on the plan for 256 CUs; a launch on fewer checks again)
-    if (a.nested.q && (a.epi.flags != EPI_NONE || a.nested.nested_log2 < 2 || stage_am2_count(a, make_stage_plan(a.N, a.K, 256)) > AM2_MAX))
+    // their table (judged on the plan for the current device's CUs, 256 where there is none)
+    if (a.nested.q && (a.epi.flags != EPI_NONE || a.nested.nested_log2 < 2 || stage_am2_count(a, make_stage_plan(a.N, a.K, gemv_plan_cus())) > AM2_MAX))
         return false;
     if (a.M < 1 || a.M > 16 || a.K % SLICE_K || a.K > 16384 || a.N % 8) return false;
     if ((int64_t)a.N * (a.K >> 1) >= ((int64_t)1 << 31)) return false;
     const int splits = stage_splits(a.K);
-    // a bias is staged in LDS by 4-byte loads, BIAS_ROWS rows per workgroup (judged like the nested tables)
-    if (a.bias && splits == 1 && ((reinterpret_cast<uintptr_t>(a.bias) & 3u) || make_stage_plan(a.N, a.K, 256).rows_per_wg > BIAS_ROWS))
+    // a bias is staged in LDS by 4-byte loads, BIAS_ROWS rows per workgroup (judged on the same plan)
+    if (a.bias && splits == 1 && ((reinterpret_cast<uintptr_t>(a.bias) & 3u) || make_stage_plan(a.N, a.K, gemv_plan_cus()).rows_per_wg > BIAS_ROWS))
         return false;
     if (a.epi.flags == EPI_RESID_NORM) {
         // K split: the workgroup that adds the K ranges does the residual step.  One K range: the finishing waves do,
         // on a residual staged in LDS -- a row of x per request, (M + 1) rows of values in all
         if (splits == 1) {
-            const int rows = make_stage_plan(a.N, a.K, 256).rows_per_wg;
+            const int rows = make_stage_plan(a.N, a.K, gemv_plan_cus()).rows_per_wg;
             if (rows > RESID_MAX_ROWS || (a.M + 1) * rows > RESID_SLOTS) return false;
             if ((reinterpret_cast<uintptr_t>(a.epi.resid_in) | reinterpret_cast<uintptr_t>(a.epi.norm_weight)) & 3u) return false;
         }
@@ -767,10 +767,8 @@ int gemv_stage_splits(int64_t K) { return stage_splits(K); }
 // EPI_RESID_NORM: partial sums of squares per row of x = the row ranges of the plan (0: no residual epilogue for this shape)
 int gemv_stage_norm_parts(int64_t M, int64_t N, int64_t K, int cus) {
     if (stage_splits(K) == 1) {
-        const int rows = make_stage_plan(N, K, 256).rows_per_wg;
+        const int rows = make_stage_plan(N, K, cus).rows_per_wg;
         if (rows > RESID_MAX_ROWS || (M + 1) * rows > RESID_SLOTS) return 0;
-        const int rows_here = make_stage_plan(N, K, cus).rows_per_wg;
-        if (rows_here > RESID_MAX_ROWS || (M + 1) * rows_here > RESID_SLOTS) return 0;
     }
     return make_stage_plan(N, K, cus).wgs_per_split;
 }
